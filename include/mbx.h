@@ -1,0 +1,151 @@
+/*
+ * mbx.h — C ABI of libmbx.so: the dropless-MoE hot path for AMD MI355X (gfx950).
+ *
+ * Every entry point takes raw device pointers, explicit sizes and a HIP stream, enqueues
+ * its kernels on that stream and returns without synchronising.  Nothing here allocates
+ * device memory: outputs and scratch are caller-provided (the *_scratch_bytes functions
+ * say how much).  Return value: 0 on success, a positive hipError_t if the HIP runtime
+ * reported one, or a negative MBX_E* code for a rejected argument.
+ *
+ * All index tensors of the permutation ops (indices, bin_ids, bins, padded_bins) are
+ * int32.  "bins" are inclusive cumulative sums: expert e owns sorted slots
+ * [bins[e-1], bins[e]) with bins[-1] := 0.
+ *
+ * Each declaration names the interface of databricks/megablocks it stands in for.
+ */
+#ifndef MBX_H_
+#define MBX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mbx_stream_t; /* a hipStream_t; NULL = the default stream */
+
+enum mbx_itype { MBX_I16 = 0, MBX_I32 = 1, MBX_I64 = 2 };
+enum mbx_dtype { MBX_BF16 = 0, MBX_F16 = 1, MBX_F32 = 2 };
+enum mbx_layout { MBX_NN = 0, MBX_NT = 1, MBX_TN = 2 };
+
+#define MBX_EINVAL (-1)   /* bad enum / negative size / null pointer */
+#define MBX_ESCRATCH (-2) /* scratch buffer too small */
+#define MBX_ERANGE (-3)   /* size beyond what the kernels index with 32 bits */
+
+/* Human-readable text for a return code (static storage). */
+const char* mbx_error_string(int code);
+/* ABI version of the loaded library. */
+int mbx_version(void);
+
+/* ------------------------------------------------------------------ routing ops */
+
+/* csrc/histogram.h:61-81 `histogram(x, num_bins)`: out[r, b] = #{c : x[r, c] == b},
+ * b in [0, num_bins); values outside the range are counted nowhere.  x is
+ * [rows, n] of `itype`, out is int32 [rows, num_bins].  All rows in one call. */
+int mbx_histogram(const void* x, int itype, int64_t rows, int64_t n, int num_bins,
+                  int32_t* out, mbx_stream_t stream);
+
+/* csrc/sort.h:59-86 `sort(x, end_bit, x_out, iota_out)`: stable LSD radix sort of n keys
+ * on bits [0, end_bit); the payload is 0..n-1 in the key type.  keys_out[i] =
+ * x[perm_out[i]].  With end_bit equal to the key width the order is the signed order. */
+size_t mbx_sort_scratch_bytes(int64_t n, int itype, int end_bit);
+int mbx_sort(const void* x, int itype, int64_t n, int end_bit, void* keys_out,
+             void* perm_out, void* scratch, size_t scratch_bytes, mbx_stream_t stream);
+
+/* csrc/cumsum.h:104-156 `inclusive_cumsum / exclusive_cumsum(x, dim=1, out)`: scan of
+ * every row of x [rows, n]. */
+int mbx_cumsum(const void* x, int itype, int64_t rows, int64_t n, int exclusive, void* out,
+               mbx_stream_t stream);
+
+/* csrc/indices.h:69-93 `indices(padded_bins, block_size, block_rows, block_cols, out)`:
+ * column indices (int16) of the block-diagonal topology; block-rows past the last bin
+ * are written as 0. */
+int mbx_topology(const int32_t* padded_bins, int num_bins, int block_size, int block_rows,
+                 int block_cols, int16_t* out, mbx_stream_t stream);
+
+/* csrc/replicate.h:130-183 `replicate_forward(x, bins, out)`: out[b, bins[i-1]:bins[i]] =
+ * x[b, i]; columns at or past bins[-1] are written as 0.  elem_bytes is 2 or 4. */
+int mbx_replicate_forward(const void* x, int elem_bytes, int64_t batch, int num_bins,
+                          const int32_t* bins, void* out, int64_t columns, mbx_stream_t stream);
+
+/* csrc/replicate.h:185-206 `replicate_backward(grad, bins, out)`: out[b, i] =
+ * sum(grad[b, bins[i-1]:bins[i]]) with fp32 accumulation. */
+int mbx_replicate_backward(const void* grad, int dtype, int64_t batch, int64_t columns,
+                           const int32_t* bins, int num_bins, void* out, mbx_stream_t stream);
+
+/* --------------------------------------------------------------- permutation ops */
+
+/* megablocks/backend/kernels.py:107-170 `gather` / `padded_gather` (_padded_copy,
+ * A_TO_B): out row r of expert e (r counted from padded_bins[e-1], or bins[e-1] when
+ * padded_bins is NULL) receives x[indices[i] / top_k] for the i-th sorted slot of e,
+ * times weights[indices[i]] (fp32 product, rounded once) when weights is not NULL.
+ * out has out_rows rows; rows owned by no slot (padding) are written as zeros.
+ * x is [tokens, hidden]. */
+int mbx_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
+               const int32_t* indices, const int32_t* bins, const int32_t* padded_bins,
+               int num_bins, const void* weights, int w_dtype, void* out, int64_t out_rows,
+               mbx_stream_t stream);
+
+/* megablocks/backend/kernels.py:173-207 `scatter` / `padded_scatter` (_padded_copy,
+ * !A_TO_B, then sum over top_k): out[t] = sum_j round(x[row(t*top_k+j)] * w[t*top_k+j]),
+ * each product rounded to the storage type and the sum taken in fp32, like the
+ * reference's two passes but without the [tokens, top_k, hidden] temporary.
+ * scratch: 4 * tokens * top_k bytes (the slot -> row map). */
+int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
+                const int32_t* indices, const int32_t* bin_ids, const int32_t* bins,
+                const int32_t* padded_bins, int num_bins, const void* weights, int w_dtype,
+                void* out, void* scratch, size_t scratch_bytes, mbx_stream_t stream);
+
+/* megablocks/backend/kernels.py:217-307 `scatter_wgrad` / `padded_scatter_wgrad`:
+ * wgrad[indices[i]] = <x[row(i)], grad[indices[i] / top_k]> (fp32 accumulate, stored
+ * in the type of x). */
+int mbx_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int hidden,
+                      int top_k, const int32_t* indices, const int32_t* bin_ids,
+                      const int32_t* bins, const int32_t* padded_bins, int num_bins,
+                      void* wgrad, mbx_stream_t stream);
+
+/* megablocks/backend/kernels.py:392-418 `binned_gather`: out [num_bins, capacity, hidden];
+ * entry j of expert e = x[indices[bins[e-1]+j] / top_k] (* weight) for j < min(count_e,
+ * capacity), zeros otherwise. */
+int mbx_binned_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
+                      const int32_t* indices, const int32_t* bins, int num_bins, int capacity,
+                      const void* weights, int w_dtype, void* out, mbx_stream_t stream);
+
+/* megablocks/backend/kernels.py:421-449 `binned_scatter`: the inverse of the above with the
+ * sum over top_k; slots that were dropped contribute zero.  x is [num_bins, capacity,
+ * hidden]; scratch: 4 * tokens * top_k bytes. */
+int mbx_binned_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
+                       const int32_t* indices, const int32_t* bins, int num_bins, int capacity,
+                       const void* weights, int w_dtype, void* out, void* scratch,
+                       size_t scratch_bytes, mbx_stream_t stream);
+
+/* megablocks/backend/kernels.py:521-543 `binned_scatter_wgrad`: wgrad[slot] =
+ * <x[e, j], grad[slot / top_k]> for kept slots, 0 for dropped ones. */
+int mbx_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens,
+                             int hidden, int top_k, const int32_t* indices, const int32_t* bins,
+                             int num_bins, int capacity, void* wgrad, mbx_stream_t stream);
+
+/* ------------------------------------------------------------------ grouped GEMM */
+
+/* grouped_gemm.backend.gmm(a, b, batch_sizes, trans_a, trans_b, c) as called through
+ * megablocks/grouped_gemm_util.py:25-26 (call sites megablocks/layers/mlp.py:414-523,
+ * megablocks/layers/glu.py:84-205).  Row groups are given on the device as inclusive
+ * int32 `bins` (no host copy of the sizes is needed); group e owns rows
+ * [bins[e-1], bins[e]) of a.
+ *   MBX_NN: c[r_e, :n] = a[r_e, :k] @ b[e] (b is [E, k, n])          rows = a.rows
+ *   MBX_NT: c[r_e, :n] = a[r_e, :k] @ b[e]^T (b is [E, n, k])
+ *   MBX_TN: c[e] = a[r_e, :k]^T @ b[r_e, :n] (c is [E, k, n]; all-zero for an empty group)
+ * fp32 accumulation; a, b, c share `dtype`.  Rows of c at or past bins[E-1] are not
+ * written (NN / NT). */
+int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bins,
+            int num_groups, int64_t rows, int k, int n, int layout, mbx_stream_t stream);
+
+/* megablocks/layers/gelu.py:9-13 `_gelu_backward_inplace(g, x)`: g *= d/dx gelu_tanh(x). */
+int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel,
+                              mbx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MBX_H_ */

@@ -1,0 +1,98 @@
+"""ctypes binding of libmbx.so (declared in include/mbx.h).
+
+The library is required: importing this module raises if it has not been built, and no
+operator has a PyTorch or CPU fallback.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'libmbx.so')
+
+I16, I32, I64 = 0, 1, 2
+BF16, F16, F32 = 0, 1, 2
+NN, NT, TN = 0, 1, 2
+
+ITYPE = {torch.int16: I16, torch.int32: I32, torch.int64: I64}
+DTYPE = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
+
+_vp, _i, _i64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
+
+_SIGNATURES = {
+    'mbx_version': (ctypes.c_int, []),
+    'mbx_error_string': (ctypes.c_char_p, [_i]),
+    'mbx_histogram': (_i, [_vp, _i, _i64, _i64, _i, _vp, _vp]),
+    'mbx_sort_scratch_bytes': (_sz, [_i64, _i, _i]),
+    'mbx_sort': (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _sz, _vp]),
+    'mbx_cumsum': (_i, [_vp, _i, _i64, _i64, _i, _vp, _vp]),
+    'mbx_topology': (_i, [_vp, _i, _i, _i, _i, _vp, _vp]),
+    'mbx_replicate_forward': (_i, [_vp, _i, _i64, _i, _vp, _vp, _i64, _vp]),
+    'mbx_replicate_backward': (_i, [_vp, _i, _i64, _i64, _vp, _i, _vp, _vp]),
+    'mbx_gather': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _vp]),
+    'mbx_scatter': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _sz, _vp]),
+    'mbx_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
+    'mbx_binned_gather': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _vp]),
+    'mbx_binned_scatter': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _sz, _vp]),
+    'mbx_binned_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _vp]),
+    'mbx_gmm': (_i, [_vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
+    'mbx_gelu_backward_inplace': (_i, [_vp, _vp, _i, _i64, _vp]),
+}
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f'{LIB_PATH} is missing: build the HIP kernels first with `python -m megablocks_amd.build` '
+            '(needs hipcc; cross-compiles for gfx950 without a GPU).')
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)   # AttributeError if the library lacks a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def check(code: int, what: str = 'mbx'):
+    if code != 0:
+        raise RuntimeError(f'{what} failed: {lib.mbx_error_string(code).decode()} (code {code})')
+
+
+def ptr(t):
+    """Device address of a tensor (None -> NULL)."""
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError('expected a tensor on the GPU')  # TORCH_CHECK(x.is_cuda()) in csrc/*.h
+
+
+def itype_of(t):
+    if t.dtype not in ITYPE:
+        raise RuntimeError(f'expected an int16/int32/int64 tensor but got {t.dtype}')
+    return ITYPE[t.dtype]
+
+
+def dtype_of(t):
+    if t.dtype not in DTYPE:
+        raise RuntimeError(f'expected a bfloat16/float16/float32 tensor but got {t.dtype}')
+    return DTYPE[t.dtype]
+
+
+def as_i32(t):
+    """Index tensors cross the ABI as contiguous int32."""
+    if t is None:
+        return None
+    if t.dtype != torch.int32:
+        t = t.to(torch.int32)
+    return t.contiguous()

@@ -1,0 +1,241 @@
+"""Token permutation kernels (host side), mirroring megablocks/backend/kernels.py.
+
+Same function names, argument order, shape checks (ValueError) and results as the
+reference's Triton launch wrappers; the work is done by the HIP kernels of libmbx.so on
+the current stream.  `weights=None` means an unscaled copy.
+"""
+import torch
+
+from megablocks_amd import _lib
+from megablocks_amd._lib import lib
+
+
+def assert_is_tensor(x, ndim):
+    if x.ndim != ndim:
+        raise ValueError(f'Expected {ndim}-tensor but got {x.ndim}-tensor')
+
+
+def assert_is_matrix(x):
+    assert_is_tensor(x, 2)
+
+
+def assert_is_vector(x):
+    if x.ndim != 1:
+        raise ValueError(f'Expected 1-tensor but got {x.ndim}-tensor')
+
+
+def assert_equal(a, b):
+    if a != b:
+        raise ValueError(f'Expected dimensions to be equal but got {a} and {b}.',)
+
+
+def _w(weights):
+    """(pointer, dtype code) of the optional router weights."""
+    if weights is None:
+        return None, 0, None
+    weights = weights.contiguous()
+    return _lib.ptr(weights), _lib.dtype_of(weights), weights
+
+
+def _scratch(n_slots, device):
+    return torch.empty(max(n_slots, 1), dtype=torch.int32, device=device)
+
+
+def _gather(x, indices, bin_ids, weights, bins, padded_bins, top_k, output_rows, what):
+    _lib.require_cuda(x, indices, bins, padded_bins, weights)
+    x = x.contiguous()
+    indices, bins, padded_bins = _lib.as_i32(indices), _lib.as_i32(bins), _lib.as_i32(padded_bins)
+    wp, wdt, weights = _w(weights)
+    out = torch.empty((output_rows, x.shape[1]), dtype=x.dtype, device=x.device)
+    with torch.cuda.device_of(x):
+        _lib.check(lib.mbx_gather(_lib.ptr(x), _lib.dtype_of(x), x.shape[0], x.shape[1], top_k, _lib.ptr(indices),
+                                  _lib.ptr(bins), _lib.ptr(padded_bins), bins.shape[0], wp, wdt, _lib.ptr(out),
+                                  output_rows, _lib.stream()), what)
+    return out
+
+
+def padded_gather(x, indices, bin_ids, weights, bins, padded_bins, top_k):
+    """megablocks/backend/kernels.py:107-138."""
+    assert_is_matrix(x)
+    assert_is_vector(indices)
+    assert_is_vector(bin_ids)
+    assert_is_vector(bins)
+    assert_is_vector(padded_bins)
+    assert_equal(indices.shape[0], x.shape[0] * top_k)
+    assert_equal(bin_ids.shape[0], x.shape[0] * top_k)
+    assert_equal(bins.size(), padded_bins.size())
+    if weights is not None:
+        assert_equal(weights.shape[0], x.shape[0] * top_k)
+    # The output size depends on the routing: one host read of the last padded bin bound,
+    # as in the reference (kernels.py:123).  Padding rows are zeroed by the kernel itself.
+    output_rows = int(padded_bins[-1].item()) if padded_bins.numel() else 0
+    return _gather(x, indices, bin_ids, weights, bins, padded_bins, top_k, output_rows, 'padded_gather')
+
+
+def gather(x, indices, bin_ids, weights, bins, top_k):
+    """megablocks/backend/kernels.py:141-170."""
+    assert_is_matrix(x)
+    assert_is_vector(indices)
+    assert_is_vector(bin_ids)
+    assert_is_vector(bins)
+    assert_equal(indices.shape[0], x.shape[0] * top_k)
+    assert_equal(bin_ids.shape[0], x.shape[0] * top_k)
+    if weights is not None:
+        assert_equal(weights.shape[0], x.shape[0] * top_k)
+    return _gather(x, indices, bin_ids, weights, bins, None, top_k, x.shape[0] * top_k, 'gather')
+
+
+def padded_scatter(x, indices, bin_ids, weights, bins, padded_bins, top_k):
+    """megablocks/backend/kernels.py:173-203 (the copy and the sum over top_k in one pass)."""
+    assert_is_matrix(x)
+    assert_is_vector(indices)
+    assert_is_vector(bin_ids)
+    assert_is_vector(bins)
+    assert_is_vector(padded_bins)
+    assert_equal(indices.shape[0], bin_ids.shape[0])
+    assert_equal(bins.size(), padded_bins.size())
+    if weights is not None:
+        assert_equal(indices.shape[0], weights.shape[0])
+    return _scatter(x, indices, bin_ids, weights, bins, padded_bins, top_k)
+
+
+def scatter(x, indices, bin_ids, weights, bins, top_k):
+    """megablocks/backend/kernels.py:206-207."""
+    assert_is_matrix(x)
+    assert_is_vector(indices)
+    assert_is_vector(bin_ids)
+    assert_is_vector(bins)
+    assert_equal(indices.shape[0], bin_ids.shape[0])
+    if weights is not None:
+        assert_equal(indices.shape[0], weights.shape[0])
+    return _scatter(x, indices, bin_ids, weights, bins, None, top_k)
+
+
+def _scatter(x, indices, bin_ids, weights, bins, padded_bins, top_k):
+    _lib.require_cuda(x, indices, bin_ids, bins, padded_bins, weights)
+    x = x.contiguous()
+    n_slots = indices.shape[0]
+    tokens = n_slots // top_k
+    if padded_bins is None:
+        assert_equal(x.shape[0], n_slots)
+    indices, bin_ids = _lib.as_i32(indices), _lib.as_i32(bin_ids)
+    bins, padded_bins = _lib.as_i32(bins), _lib.as_i32(padded_bins)
+    wp, wdt, weights = _w(weights)
+    out = torch.empty((tokens, x.shape[1]), dtype=x.dtype, device=x.device)
+    scratch = _scratch(n_slots, x.device)
+    with torch.cuda.device_of(x):
+        _lib.check(lib.mbx_scatter(_lib.ptr(x), _lib.dtype_of(x), tokens, x.shape[1], top_k, _lib.ptr(indices),
+                                   _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins), bins.shape[0], wp, wdt,
+                                   _lib.ptr(out), _lib.ptr(scratch), scratch.numel() * 4, _lib.stream()), 'scatter')
+    return out
+
+
+def padded_scatter_wgrad(x, grad, indices, bin_ids, bins, padded_bins, top_k):
+    """megablocks/backend/kernels.py:279-303."""
+    assert_is_matrix(x)
+    assert_is_matrix(grad)
+    assert_is_vector(indices)
+    assert_is_vector(bin_ids)
+    assert_is_vector(bins)
+    assert_is_vector(padded_bins)
+    assert_equal(indices.shape[0], bin_ids.shape[0])
+    assert_equal(bins.size(), padded_bins.size())
+    return _scatter_wgrad(x, grad, indices, bin_ids, bins, padded_bins, top_k)
+
+
+def scatter_wgrad(x, grad, indices, bin_ids, bins, top_k):
+    """megablocks/backend/kernels.py:306-307."""
+    assert_is_matrix(x)
+    assert_is_matrix(grad)
+    assert_is_vector(indices)
+    assert_is_vector(bin_ids)
+    assert_is_vector(bins)
+    assert_equal(indices.shape[0], bin_ids.shape[0])
+    return _scatter_wgrad(x, grad, indices, bin_ids, bins, None, top_k)
+
+
+def _scatter_wgrad(x, grad, indices, bin_ids, bins, padded_bins, top_k):
+    _lib.require_cuda(x, grad, indices, bin_ids, bins, padded_bins)
+    x = x.contiguous()
+    grad = grad.contiguous().to(x.dtype)
+    assert_equal(x.shape[1], grad.shape[1])
+    n_slots = indices.shape[0]
+    tokens = n_slots // top_k
+    assert_equal(grad.shape[0], tokens)
+    indices, bin_ids = _lib.as_i32(indices), _lib.as_i32(bin_ids)
+    bins, padded_bins = _lib.as_i32(bins), _lib.as_i32(padded_bins)
+    out = torch.empty((n_slots,), dtype=x.dtype, device=x.device)
+    with torch.cuda.device_of(x):
+        _lib.check(lib.mbx_scatter_wgrad(_lib.ptr(x), _lib.ptr(grad), _lib.dtype_of(x), tokens, x.shape[1], top_k,
+                                         _lib.ptr(indices), _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins),
+                                         bins.shape[0], _lib.ptr(out), _lib.stream()), 'scatter_wgrad')
+    return out
+
+
+def binned_gather(x, indices, weights, bins, expert_capacity, top_k):
+    """megablocks/backend/kernels.py:392-418."""
+    assert_is_matrix(x)
+    assert_is_vector(indices)
+    assert_is_vector(bins)
+    assert_equal(indices.shape[0], x.shape[0] * top_k)
+    if weights is not None:
+        assert_equal(weights.shape[0], x.shape[0] * top_k)
+    _lib.require_cuda(x, indices, bins, weights)
+    x = x.contiguous()
+    indices, bins = _lib.as_i32(indices), _lib.as_i32(bins)
+    wp, wdt, weights = _w(weights)
+    num_experts = bins.shape[0]
+    out = torch.empty((num_experts, expert_capacity, x.shape[1]), dtype=x.dtype, device=x.device)
+    with torch.cuda.device_of(x):
+        _lib.check(lib.mbx_binned_gather(_lib.ptr(x), _lib.dtype_of(x), x.shape[0], x.shape[1], top_k, _lib.ptr(indices),
+                                         _lib.ptr(bins), num_experts, expert_capacity, wp, wdt, _lib.ptr(out),
+                                         _lib.stream()), 'binned_gather')
+    return out
+
+
+def binned_scatter(x, indices, weights, bins, top_k):
+    """megablocks/backend/kernels.py:421-449."""
+    assert_is_tensor(x, 3)
+    assert_is_vector(indices)
+    assert_is_vector(bins)
+    assert_equal(bins.shape[0], x.shape[0])
+    if weights is not None:
+        assert_equal(indices.shape[0], weights.shape[0])
+    _lib.require_cuda(x, indices, bins, weights)
+    x = x.contiguous()
+    num_experts, expert_capacity, hidden_size = x.shape
+    n_slots = indices.shape[0]
+    tokens = n_slots // top_k
+    indices, bins = _lib.as_i32(indices), _lib.as_i32(bins)
+    wp, wdt, weights = _w(weights)
+    out = torch.empty((tokens, hidden_size), dtype=x.dtype, device=x.device)
+    scratch = _scratch(n_slots, x.device)
+    with torch.cuda.device_of(x):
+        _lib.check(lib.mbx_binned_scatter(_lib.ptr(x), _lib.dtype_of(x), tokens, hidden_size, top_k, _lib.ptr(indices),
+                                          _lib.ptr(bins), num_experts, expert_capacity, wp, wdt, _lib.ptr(out),
+                                          _lib.ptr(scratch), scratch.numel() * 4, _lib.stream()), 'binned_scatter')
+    return out
+
+
+def binned_scatter_wgrad(x, grad, indices, bins, top_k):
+    """megablocks/backend/kernels.py:521-543."""
+    assert_is_tensor(x, 3)
+    assert_is_matrix(grad)
+    assert_is_vector(indices)
+    assert_is_vector(bins)
+    assert_equal(bins.shape[0], x.shape[0])
+    _lib.require_cuda(x, grad, indices, bins)
+    x = x.contiguous()
+    grad = grad.contiguous().to(x.dtype)
+    num_experts, expert_capacity, hidden_size = x.shape
+    assert_equal(grad.shape[1], hidden_size)
+    n_slots = indices.shape[0]
+    tokens = n_slots // top_k
+    assert_equal(grad.shape[0], tokens)
+    indices, bins = _lib.as_i32(indices), _lib.as_i32(bins)
+    out = torch.empty((n_slots,), dtype=x.dtype, device=x.device)
+    with torch.cuda.device_of(x):
+        _lib.check(lib.mbx_binned_scatter_wgrad(_lib.ptr(x), _lib.ptr(grad), _lib.dtype_of(x), tokens, hidden_size, top_k,
+                                                _lib.ptr(indices), _lib.ptr(bins), num_experts, expert_capacity,
+                                                _lib.ptr(out), _lib.stream()), 'binned_scatter_wgrad')
+    return out

@@ -1,0 +1,63 @@
+"""Builds libmbx.so (the HIP kernels + C ABI) in-tree for gfx950 with hipcc.
+
+    python -m megablocks_amd.build            # compile what is out of date
+    python -m megablocks_amd.build --force    # recompile everything
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, 'csrc')
+BUILD = os.path.join(HERE, 'build')
+LIB = os.path.join(HERE, 'libmbx.so')
+SOURCES = ['routing.hip', 'permute.hip', 'gmm.hip']
+HEADERS = [os.path.join(CSRC, 'common.h'), os.path.join(os.path.dirname(HERE), 'include', 'mbx.h')]
+ARCH = 'gfx950'
+# -packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from scalar float code.
+FLAGS = ['-O3', '-fPIC', '-std=c++17', f'--offload-arch={ARCH}', '-Xclang', '-target-feature', '-Xclang',
+         '-packed-fp32-ops', '-Wno-unused-command-line-argument']
+
+
+def _hipcc():
+    for cand in (os.environ.get('HIPCC'), '/opt/rocm/bin/hipcc', 'hipcc'):
+        if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
+            return cand
+    return 'hipcc'
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = '\n'.join(l for l in proc.stdout.splitlines() if "is not a recognized feature for this target" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f'command failed: {" ".join(cmd)}\n{out}')
+    return out
+
+
+def build(force: bool = False, verbose: bool = False) -> str:
+    os.makedirs(BUILD, exist_ok=True)
+    hipcc = _hipcc()
+    objs = []
+    newest_header = max(os.path.getmtime(h) for h in HEADERS)
+    procs = []
+    for src in SOURCES:
+        s = os.path.join(CSRC, src)
+        o = os.path.join(BUILD, src.replace('.hip', '.o'))
+        objs.append(o)
+        stale = force or not os.path.exists(o) or os.path.getmtime(o) < max(os.path.getmtime(s), newest_header)
+        if stale:
+            cmd = [hipcc] + FLAGS + ['-c', s, '-o', o]
+            if verbose:
+                print(' '.join(cmd), flush=True)
+            procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for cmd, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError(f'command failed: {" ".join(cmd)}\n{out}')
+    if procs or force or not os.path.exists(LIB):
+        _run([hipcc, '-shared', '-fPIC', f'--offload-arch={ARCH}', '-o', LIB] + objs)
+    return LIB
+
+
+if __name__ == '__main__':
+    print(build(force='--force' in sys.argv, verbose=True))

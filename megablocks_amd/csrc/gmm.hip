@@ -1,0 +1,453 @@
+// Grouped GEMM for variable per-expert row counts on gfx950 matrix cores.
+//
+//   NN: c[r_e] = a[r_e] @ b[e]        NT: c[r_e] = a[r_e] @ b[e]^T       TN: c[e] = a[r_e]^T @ b[r_e]
+//
+// Tiling: one workgroup computes a BM x BN tile of c with v_mfma_f32_32x32x16 (bf16 or f16
+// inputs, fp32 accumulators).  Operand tiles are staged through LDS, double buffered, with
+// the global loads of tile t+1 in flight while tile t is multiplied.  An operand whose
+// reduction dimension is contiguous in memory ("KC": a in NN/NT, b in NT) is kept as
+// [row][k] in LDS and read with 128-bit LDS loads; an operand whose reduction dimension is
+// strided ("MC": b in NN, both in TN) is kept as [k][col] and read with the gfx950
+// transposing LDS load (ds_read_b64_tr_b16), which hands every lane the four k-consecutive
+// values of its column.  The tile -> (expert, row tile) schedule is computed on the device
+// from the inclusive row bins, so no host copy of the group sizes is needed and empty
+// experts cost nothing (NN/NT) or produce an all-zero block (TN).
+#include "common.h"
+
+namespace mbx {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ f32x16 mfma32(const u32x4& a, const u32x4& b, const f32x16& c) {
+  if (DT == MBX_BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
+// One operand of the product as seen by a workgroup.
+struct Operand {
+  const uint16_t* base;  // element (row, k) of a KC operand is base[row * ld + k];
+                         // element (k, col) of an MC operand is base[k * ld + col]
+  int64_t ld;
+  int r0;      // first row (KC) / column (MC) of the tile in the non-reduction dimension
+  int r_lim;   // bound of that dimension (rows are clamped, columns are zero-filled)
+};
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int PAD_KC_, int PAD_MC_>
+struct Tile {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+  static constexpr int PAD_KC = PAD_KC_, PAD_MC = PAD_MC_;
+  static constexpr int THREADS = WM * WN * kWave;
+  static constexpr int WTM = BM / WM, WTN = BN / WN;   // tile of one wave
+  static constexpr int TM = WTM / 32, TN = WTN / 32;    // 32x32 MFMA tiles per wave
+  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % 16 == 0, "tile shape");
+};
+
+// LDS footprint (in elements) of one operand tile with R non-reduction rows/columns.
+template <bool MC, int R, int BK, int PAD_KC, int PAD_MC>
+struct OperandLds {
+  static constexpr int STRIDE = MC ? (R + PAD_MC) : (BK + PAD_KC);
+  static constexpr int ELEMS = MC ? BK * STRIDE : R * STRIDE;
+};
+
+// Global -> registers: every thread fetches CH 16-byte chunks of the operand tile.
+template <bool MC, int R, int BK, int THREADS>
+struct Stager {
+  static constexpr int CHUNKS = R * BK / 8;
+  static constexpr int CH = CHUNKS / THREADS;
+  static_assert(CHUNKS % THREADS == 0, "tile must split evenly over the threads");
+
+  static __device__ __forceinline__ void load(const Operand& op, int k0, int k_end, u32x4 (&reg)[CH]) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + i * THREADS;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (!MC) {
+        const int r = c / (BK / 8), kc = (c % (BK / 8)) * 8;
+        int row = op.r0 + r;
+        if (row > op.r_lim - 1) row = op.r_lim - 1;
+        if (k0 + kc < k_end) v = *(const u32x4*)(op.base + (int64_t)row * op.ld + (k0 + kc));
+      } else {
+        const int kk = c / (R / 8), rc = (c % (R / 8)) * 8;
+        if (k0 + kk < k_end && op.r0 + rc < op.r_lim) v = *(const u32x4*)(op.base + (int64_t)(k0 + kk) * op.ld + (op.r0 + rc));
+      }
+      reg[i] = v;
+    }
+  }
+
+  template <int STRIDE>
+  static __device__ __forceinline__ void store(uint16_t* lds, const u32x4 (&reg)[CH]) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + i * THREADS;
+      if (!MC) {
+        const int r = c / (BK / 8), kc = (c % (BK / 8)) * 8;
+        *(u32x4*)(lds + r * STRIDE + kc) = reg[i];
+      } else {
+        const int kk = c / (R / 8), rc = (c % (R / 8)) * 8;
+        *(u32x4*)(lds + kk * STRIDE + rc) = reg[i];
+      }
+    }
+  }
+};
+
+// LDS -> MFMA operand registers for the 32 rows/columns starting at `r` and k-step `ks`.
+template <bool MC, int STRIDE>
+__device__ __forceinline__ u32x4 read_frag(const uint16_t* lds, int r, int ks) {
+  const int lane = lane_id();
+  if (!MC) {
+    return *(const u32x4*)(lds + (r + (lane & 31)) * STRIDE + ks * 16 + (lane >> 5) * 8);
+  } else {
+    const int g = lane >> 4, s = lane & 15;
+    const uint16_t* p = lds + (ks * 16 + (g >> 1) * 8 + (s >> 2)) * STRIDE + r + (g & 1) * 16 + (s & 3) * 4;
+    typedef __attribute__((address_space(3))) s16x4_t* lds_ptr_t;
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p));
+    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p + 4 * STRIDE));
+    u32x4 v;
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    v[0] = l2[0]; v[1] = l2[1]; v[2] = h2[0]; v[3] = h2[1];
+    return v;
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  if (DT == MBX_BF16) return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)a) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)b) << 16);
+}
+
+// The workgroup-level product: acc += A_tile(k) * B_tile(k) over k in [k_begin, k_end),
+// then c[m0.., n0..] = acc for rows < m_lim and columns < n_lim.
+template <int DT, bool A_MC, bool B_MC, typename T>
+__device__ __forceinline__ void block_gemm(const Operand& opa, const Operand& opb, int k_begin, int k_end,
+                                           uint16_t* __restrict__ c, int64_t ldc, int m_lim, int n_lim, uint16_t* lds) {
+  typedef OperandLds<A_MC, T::BM, T::BK, T::PAD_KC, T::PAD_MC> LA;
+  typedef OperandLds<B_MC, T::BN, T::BK, T::PAD_KC, T::PAD_MC> LB;
+  typedef Stager<A_MC, T::BM, T::BK, T::THREADS> SA;
+  typedef Stager<B_MC, T::BN, T::BK, T::THREADS> SB;
+  constexpr int STAGE = LA::ELEMS + LB::ELEMS;
+
+  const int wave = threadIdx.x / kWave, lane = lane_id();
+  const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
+
+  f32x16 acc[T::TM][T::TN];
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int nk = (k_end - k_begin + T::BK - 1) / T::BK;
+  u32x4 ra[SA::CH], rb[SB::CH];
+  if (nk > 0) {
+    SA::load(opa, k_begin, k_end, ra);
+    SB::load(opb, k_begin, k_end, rb);
+    SA::template store<LA::STRIDE>(lds, ra);
+    SB::template store<LB::STRIDE>(lds + LA::ELEMS, rb);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    uint16_t* cur = lds + (kt & 1) * STAGE;
+    uint16_t* nxt = lds + ((kt + 1) & 1) * STAGE;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      SA::load(opa, k_begin + (kt + 1) * T::BK, k_end, ra);
+      SB::load(opb, k_begin + (kt + 1) * T::BK, k_end, rb);
+    }
+#pragma unroll
+    for (int ks = 0; ks < T::BK / 16; ++ks) {
+      u32x4 fa[T::TM], fb[T::TN];
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i) fa[i] = read_frag<A_MC, LA::STRIDE>(cur, wm + i * 32, ks);
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) fb[j] = read_frag<B_MC, LB::STRIDE>(cur + LA::ELEMS, wn + j * 32, ks);
+      // operands swapped: the accumulator tile is c^T, so a lane owns runs of four
+      // consecutive columns of one row of c and can store them as one 8-byte word.
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) acc[i][j] = mfma32<DT>(fb[j], fa[i], acc[i][j]);
+    }
+    if (more) {
+      SA::template store<LA::STRIDE>(nxt, ra);
+      SB::template store<LB::STRIDE>(nxt + LA::ELEMS, rb);
+    }
+    __syncthreads();
+  }
+
+  // accumulator (i, j), register r of lane l holds c[m][n] with
+  //   m = opa.r0 + wm + 32 i + (l % 32),  n = opb.r0 + wn + 32 j + 8 (r / 4) + 4 (l / 32) + (r % 4)
+  const bool n_vec = (ldc % 4 == 0) && (((uintptr_t)c & 7u) == 0);
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i) {
+    const int m = opa.r0 + wm + i * 32 + (lane & 31);
+    if (m >= m_lim) continue;
+    uint16_t* crow = c + (int64_t)m * ldc;
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = opb.r0 + wn + j * 32 + q * 8 + (lane >> 5) * 4;
+        const f32x16& v = acc[i][j];
+        if (n + 3 < n_lim && n_vec) {
+          u32x2 w;
+          w[0] = pack2<DT>(v[q * 4 + 0], v[q * 4 + 1]);
+          w[1] = pack2<DT>(v[q * 4 + 2], v[q * 4 + 3]);
+          *(u32x2*)(crow + n) = w;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (n + t < n_lim) crow[n + t] = (uint16_t)(pack2<DT>(v[q * 4 + t], 0.f) & 0xffffu);
+        }
+      }
+    }
+  }
+}
+
+// ---- NN / NT: row tiles follow the expert bins --------------------------------------
+// Linear workgroup id -> (expert, column tile, row tile inside the expert), row tiles
+// fastest, so that the workgroups in flight together share b[e] column panels.
+template <int DT, bool B_MC, typename T>
+__global__ void __launch_bounds__(T::THREADS)
+gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
+                const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  int id = blockIdx.x;
+  int e = 0, start = 0, end = 0, mt = 0;
+  for (; e < num_groups; ++e) {
+    end = bins[e];
+    mt = (end - start + T::BM - 1) / T::BM;
+    const int span = mt * tiles_n;
+    if (id < span) break;
+    id -= span;
+    start = end;
+  }
+  if (e >= num_groups) return;  // surplus workgroup (uniform over the block)
+  const int tn = id / mt, tm = id % mt;
+
+  Operand opa, opb;
+  opa.base = a; opa.ld = k; opa.r0 = start + tm * T::BM; opa.r_lim = end;
+  if (B_MC) { opb.base = b + (int64_t)e * k * n; opb.ld = n; }
+  else { opb.base = b + (int64_t)e * n * k; opb.ld = k; }
+  opb.r0 = tn * T::BN; opb.r_lim = n;
+  block_gemm<DT, false, B_MC, T>(opa, opb, 0, k, c, n, end, n, lds);
+}
+
+// ---- TN: one [k, n] product per expert, reduced over the expert's rows ----------------
+template <int DT, typename T>
+__global__ void __launch_bounds__(T::THREADS)
+gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
+              const int32_t* __restrict__ bins, int k, int n, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  const int e = blockIdx.y;
+  const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+  const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
+  Operand opa, opb;
+  opa.base = a; opa.ld = k; opa.r0 = tm * T::BM; opa.r_lim = k;
+  opb.base = b; opb.ld = n; opb.r0 = tn * T::BN; opb.r_lim = n;
+  block_gemm<DT, true, true, T>(opa, opb, start, end, c + (int64_t)e * k * n, n, k, n, lds);
+}
+
+// ---- fallback for shapes the MFMA path does not take (odd sizes, fp32) ----------------
+// c(m, n) = sum_r a(m, r) b(r, n) with arbitrary element strides; 32x32 tile, fp32 FMA.
+template <int DT>
+__global__ void __launch_bounds__(256)
+gmm_generic_kernel(const void* __restrict__ a_, const void* __restrict__ b_, void* __restrict__ c_,
+                   const int32_t* __restrict__ bins, int layout, int k, int n) {
+  typedef typename Elem<DT>::type E;
+  const E* a = (const E*)a_;
+  const E* b = (const E*)b_;
+  E* c = (E*)c_;
+  __shared__ float as[32][33], bs[32][33];
+  const int e = blockIdx.z;
+  const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
+  const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;  // 32 x 8
+  int m_dim, r_begin, r_end;
+  if (layout == MBX_TN) { m_dim = k; r_begin = start; r_end = end; }
+  else { m_dim = end - start; r_begin = 0; r_end = k; }
+  const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+  if (m0 >= m_dim) return;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int r0 = r_begin; r0 < r_end; r0 += 32) {
+    for (int i = ty; i < 32; i += 8) {
+      const int m = m0 + i, r = r0 + tx;   // as[i][tx] = a(m, r)
+      float va = 0.f, vb = 0.f;
+      if (m < m_dim && r < r_end)
+        va = Elem<DT>::to_f32(layout == MBX_TN ? a[(int64_t)r * k + m] : a[(int64_t)(start + m) * k + r]);
+      const int rr = r0 + i, nn = n0 + tx;  // bs[i][tx] = b(rr, nn)
+      if (rr < r_end && nn < n) {
+        if (layout == MBX_TN) vb = Elem<DT>::to_f32(b[(int64_t)rr * n + nn]);
+        else if (layout == MBX_NN) vb = Elem<DT>::to_f32(b[((int64_t)e * k + rr) * n + nn]);
+        else vb = Elem<DT>::to_f32(b[((int64_t)e * n + nn) * k + rr]);
+      }
+      as[i][tx] = va;
+      bs[i][tx] = vb;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int r = 0; r < 32; ++r) {
+      const float bv = bs[r][tx];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[q] += as[ty + 8 * q][r] * bv;
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int m = m0 + ty + 8 * q, nn = n0 + tx;
+    if (m < m_dim && nn < n) {
+      if (layout == MBX_TN) c[((int64_t)e * k + m) * n + nn] = Elem<DT>::from_f32(acc[q]);
+      else c[(int64_t)(start + m) * n + nn] = Elem<DT>::from_f32(acc[q]);
+    }
+  }
+}
+
+// ---- GELU backward, in place ---------------------------------------------------------
+template <int DT>
+__global__ void gelu_backward_kernel(void* __restrict__ g_, const void* __restrict__ x_, int64_t numel) {
+  typedef typename Elem<DT>::type E;
+  E* g = (E*)g_;
+  const E* x = (const E*)x_;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < numel; i += stride) {
+    const float xv = Elem<DT>::to_f32(x[i]);
+    const float t = tanhf(0.79788456f * xv * (1.f + 0.044715f * xv * xv));
+    const float ff = 0.5f * xv * ((1.f - t * t) * (0.79788456f + 0.1070322243f * xv * xv)) + 0.5f * (1.f + t);
+    g[i] = Elem<DT>::from_f32(Elem<DT>::to_f32(g[i]) * ff);
+  }
+}
+
+// Tile shapes.  256x256x64 with four waves (2x2, 128x128 each) keeps the accumulators in
+// 256 registers per lane and needs 144 KiB of the 160 KiB LDS for two stages.
+typedef Tile<256, 256, 64, 2, 2, 8, 16> TileBig;
+
+template <int DT, bool A_MC, bool B_MC, typename T>
+constexpr size_t lds_bytes() {
+  return 2 * sizeof(uint16_t) *
+         (size_t)(OperandLds<A_MC, T::BM, T::BK, T::PAD_KC, T::PAD_MC>::ELEMS + OperandLds<B_MC, T::BN, T::BK, T::PAD_KC, T::PAD_MC>::ELEMS);
+}
+
+template <typename K>
+int allow_lds(K kernel, size_t bytes) {
+  return (int)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+template <int DT>
+int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
+             int layout, hipStream_t s) {
+  typedef TileBig T;
+  const uint16_t* ap = (const uint16_t*)a;
+  const uint16_t* bp = (const uint16_t*)b;
+  uint16_t* cp = (uint16_t*)c;
+  if (layout == MBX_TN) {
+    const int tiles_m = (int)ceil_div(k, T::BM), tiles_n = (int)ceil_div(n, T::BN);
+    constexpr size_t lds = lds_bytes<DT, true, true, T>();
+    auto kern = gmm_tn_kernel<DT, T>;
+    int rc = allow_lds(kern, lds);
+    if (rc) return rc;
+    kern<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)num_groups), T::THREADS, lds, s>>>(ap, bp, cp, bins, k, n, tiles_m, tiles_n);
+    return launch_status();
+  }
+  const int tiles_n = (int)ceil_div(n, T::BN);
+  const int64_t max_mt = ceil_div(rows, T::BM) + num_groups;
+  const int64_t grid = max_mt * tiles_n;
+  if (grid > 0x7fffffff) return MBX_ERANGE;
+  if (layout == MBX_NT) {
+    constexpr size_t lds = lds_bytes<DT, false, false, T>();
+    auto kern = gmm_rows_kernel<DT, false, T>;
+    int rc = allow_lds(kern, lds);
+    if (rc) return rc;
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_n);
+  } else {
+    constexpr size_t lds = lds_bytes<DT, false, true, T>();
+    auto kern = gmm_rows_kernel<DT, true, T>;
+    int rc = allow_lds(kern, lds);
+    if (rc) return rc;
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_n);
+  }
+  return launch_status();
+}
+
+template <int DT>
+int gmm_generic(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
+                int layout, hipStream_t s) {
+  // The row count of a group is only known on the device: size the grid for the worst case.
+  const int64_t m_bound = layout == MBX_TN ? k : rows;
+  const int64_t gy = ceil_div(m_bound, 32), gx = ceil_div(n, 32);
+  if (gy > 65535 || num_groups > 65535) return MBX_ERANGE;
+  if (gy == 0 || gx == 0) return 0;
+  gmm_generic_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)num_groups), 256, 0, s>>>(a, b, c, bins, layout, k, n);
+  return launch_status();
+}
+
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+}  // namespace
+}  // namespace mbx
+
+using namespace mbx;
+
+extern "C" {
+
+int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bins, int num_groups, int64_t rows, int k,
+            int n, int layout, mbx_stream_t stream) {
+  if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
+  if (layout != MBX_NN && layout != MBX_NT && layout != MBX_TN) return MBX_EINVAL;
+  if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
+  if (num_groups == 0) return 0;
+  if (!bins) return MBX_EINVAL;
+  if (rows > 0x7fffffff) return MBX_ERANGE;
+  hipStream_t s = as_stream(stream);
+  if (layout == MBX_TN) {
+    if ((int64_t)k * n == 0) return 0;
+    if (!c || (rows > 0 && (!a || !b))) return MBX_EINVAL;
+  } else {
+    if (rows == 0 || n == 0) return 0;
+    if (!c || (k > 0 && (!a || !b))) return MBX_EINVAL;
+  }
+  // MFMA path: 16-byte global loads need k (and n, where n is the contiguous dimension of an
+  // operand) to be multiples of 8 and the bases to be 16-byte aligned.
+  bool fast = dtype != MBX_F32 && aligned16(a) && aligned16(b) && k > 0;
+  if (layout == MBX_NT) fast = fast && k % 8 == 0;
+  if (layout == MBX_NN) fast = fast && k % 8 == 0 && n % 8 == 0;
+  if (layout == MBX_TN) fast = fast && k % 8 == 0 && n % 8 == 0;
+  if (fast) {
+    if (dtype == MBX_BF16) return gmm_mfma<MBX_BF16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+    return gmm_mfma<MBX_F16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+  }
+  switch (dtype) {
+    case MBX_BF16: return gmm_generic<MBX_BF16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+    case MBX_F16: return gmm_generic<MBX_F16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+    default: return gmm_generic<MBX_F32>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+  }
+}
+
+int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel, mbx_stream_t stream) {
+  if (numel < 0) return MBX_EINVAL;
+  if (numel == 0) return 0;
+  if (!g || !x) return MBX_EINVAL;
+  int64_t blocks = ceil_div(numel, 256 * 4);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case MBX_BF16: gelu_backward_kernel<MBX_BF16><<<(unsigned)blocks, 256, 0, s>>>(g, x, numel); break;
+    case MBX_F16: gelu_backward_kernel<MBX_F16><<<(unsigned)blocks, 256, 0, s>>>(g, x, numel); break;
+    case MBX_F32: gelu_backward_kernel<MBX_F32><<<(unsigned)blocks, 256, 0, s>>>(g, x, numel); break;
+    default: return MBX_EINVAL;
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,480 @@
+// Token permutation kernels: gather into expert-major order, fused weighted top-k combine
+// back to token order, router-weight gradient, and the capacity-binned variants.
+// HBM-bound row copies: one wave per row, 128-bit loads and stores when the row is a
+// multiple of 16 bytes and the buffers are 16-byte aligned.
+#include "common.h"
+
+namespace mbx {
+namespace {
+
+constexpr int kRowThreads = 256;
+constexpr int kRowWaves = kRowThreads / kWave;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int DT> struct Vec16 {  // 16 bytes of storage <-> fp32 lanes
+  static constexpr int kElems = 16 / (int)sizeof(typename Elem<DT>::type);
+  static __device__ __forceinline__ void unpack(const u32x4& v, float* f) {
+    if (DT == MBX_F32) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(v[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint16_t lo = (uint16_t)(v[i] & 0xffffu), hi = (uint16_t)(v[i] >> 16);
+        if (DT == MBX_BF16) { f[2 * i] = bf16_to_f32(lo); f[2 * i + 1] = bf16_to_f32(hi); }
+        else { f[2 * i] = (float)__builtin_bit_cast(_Float16, lo); f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, hi); }
+      }
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* f) {
+    u32x4 v;
+    if (DT == MBX_F32) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = __float_as_uint(f[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint16_t lo, hi;
+        if (DT == MBX_BF16) { lo = f32_to_bf16(f[2 * i]); hi = f32_to_bf16(f[2 * i + 1]); }
+        else { lo = __builtin_bit_cast(uint16_t, (_Float16)f[2 * i]); hi = __builtin_bit_cast(uint16_t, (_Float16)f[2 * i + 1]); }
+        v[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+      }
+    }
+    return v;
+  }
+};
+
+// dst[0:hidden] = round(src * scale) (or a plain copy), by one wave.
+template <int DT, bool VEC>
+__device__ __forceinline__ void wave_copy_row(const typename Elem<DT>::type* __restrict__ src,
+                                              typename Elem<DT>::type* __restrict__ dst, int hidden,
+                                              bool scaled, float scale) {
+  const int lane = lane_id();
+  if (VEC) {
+    constexpr int E = Vec16<DT>::kElems;
+    const int nvec = hidden / E;
+    const u32x4* s = (const u32x4*)src;
+    u32x4* d = (u32x4*)dst;
+    if (!scaled) {
+      int c = lane;
+      for (; c + 3 * kWave < nvec; c += 4 * kWave) {
+        const u32x4 v0 = s[c], v1 = s[c + kWave], v2 = s[c + 2 * kWave], v3 = s[c + 3 * kWave];
+        d[c] = v0; d[c + kWave] = v1; d[c + 2 * kWave] = v2; d[c + 3 * kWave] = v3;
+      }
+      for (; c < nvec; c += kWave) d[c] = s[c];
+    } else {
+      for (int c = lane; c < nvec; c += kWave) {
+        float f[E];
+        Vec16<DT>::unpack(s[c], f);
+#pragma unroll
+        for (int i = 0; i < E; ++i) f[i] *= scale;
+        d[c] = Vec16<DT>::pack(f);
+      }
+    }
+  } else {
+    for (int c = lane; c < hidden; c += kWave)
+      dst[c] = scaled ? Elem<DT>::from_f32(Elem<DT>::to_f32(src[c]) * scale) : src[c];
+  }
+}
+
+template <int DT, bool VEC>
+__device__ __forceinline__ void wave_zero_row(typename Elem<DT>::type* __restrict__ dst, int hidden) {
+  const int lane = lane_id();
+  if (VEC) {
+    const int nvec = hidden / Vec16<DT>::kElems;
+    u32x4* d = (u32x4*)dst;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int c = lane; c < nvec; c += kWave) d[c] = z;
+  } else {
+    for (int c = lane; c < hidden; c += kWave) dst[c] = Elem<DT>::from_f32(0.f);
+  }
+}
+
+template <int DT, bool VEC>
+__device__ __forceinline__ float wave_dot_row(const typename Elem<DT>::type* __restrict__ a,
+                                              const typename Elem<DT>::type* __restrict__ b, int hidden) {
+  const int lane = lane_id();
+  float acc = 0.f;
+  if (VEC) {
+    constexpr int E = Vec16<DT>::kElems;
+    const int nvec = hidden / E;
+    const u32x4* av = (const u32x4*)a;
+    const u32x4* bv = (const u32x4*)b;
+    for (int c = lane; c < nvec; c += kWave) {
+      float fa[E], fb[E];
+      Vec16<DT>::unpack(av[c], fa);
+      Vec16<DT>::unpack(bv[c], fb);
+#pragma unroll
+      for (int i = 0; i < E; ++i) acc += fa[i] * fb[i];
+    }
+  } else {
+    for (int c = lane; c < hidden; c += kWave) acc += Elem<DT>::to_f32(a[c]) * Elem<DT>::to_f32(b[c]);
+  }
+  return wave_sum(acc);
+}
+
+// Sorted slot feeding output row `row` of the expert-major buffer, or -1 for a padding row.
+__device__ __forceinline__ int slot_of_row(int row, const int32_t* __restrict__ bins,
+                                           const int32_t* __restrict__ padded_bins, int num_bins, int n_slots) {
+  if (padded_bins == nullptr) return row < n_slots ? row : -1;
+  const int e = upper_bound_i32(padded_bins, num_bins, row);
+  if (e >= num_bins) return -1;
+  const int pstart = e > 0 ? padded_bins[e - 1] : 0;
+  const int start = e > 0 ? bins[e - 1] : 0;
+  const int pos = start + (row - pstart);
+  return (pos < bins[e] && pos < n_slots) ? pos : -1;
+}
+
+// ------------------------------------------------------------------ gather
+template <int DT, bool VEC>
+__global__ void __launch_bounds__(kRowThreads)
+gather_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ indices,
+              const int32_t* __restrict__ bins, const int32_t* __restrict__ padded_bins, int num_bins,
+              const void* __restrict__ weights, int w_dtype, void* __restrict__ out_, int64_t out_rows) {
+  typedef typename Elem<DT>::type E;
+  const E* x = (const E*)x_;
+  E* out = (E*)out_;
+  const int n_slots = (int)(tokens * top_k);
+  const int wave = threadIdx.x / kWave;
+  for (int64_t row = (int64_t)blockIdx.x * kRowWaves + wave; row < out_rows; row += (int64_t)gridDim.x * kRowWaves) {
+    E* dst = out + row * hidden;
+    const int pos = slot_of_row((int)row, bins, padded_bins, num_bins, n_slots);
+    int s = pos >= 0 ? indices[pos] : -1;
+    if (s < 0 || s >= n_slots) { wave_zero_row<DT, VEC>(dst, hidden); continue; }
+    const float scale = weights ? load_as_f32(weights, s, w_dtype) : 1.f;
+    wave_copy_row<DT, VEC>(x + (int64_t)(s / top_k) * hidden, dst, hidden, weights != nullptr, scale);
+  }
+}
+
+// ------------------------------------------------------------------ slot -> row maps
+__global__ void inverse_map_kernel(const int32_t* __restrict__ indices, const int32_t* __restrict__ bin_ids,
+                                   const int32_t* __restrict__ bins, const int32_t* __restrict__ padded_bins,
+                                   int num_bins, int n_slots, int32_t* __restrict__ inv) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_slots) return;
+  const int s = indices[i];
+  if (s < 0 || s >= n_slots) return;
+  int row = i;
+  if (padded_bins != nullptr) {
+    const int e = bin_ids[i];
+    if (e < 0 || e >= num_bins) return;
+    if (e > 0) row = i - bins[e - 1] + padded_bins[e - 1];
+  }
+  inv[s] = row;
+}
+
+__global__ void binned_inverse_map_kernel(const int32_t* __restrict__ indices, const int32_t* __restrict__ bins,
+                                          int capacity, int n_slots, int32_t* __restrict__ inv) {
+  const int e = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  const int start = e > 0 ? bins[e - 1] : 0;
+  int count = bins[e] - start;
+  if (count > capacity) count = capacity;
+  if (j >= count || start + j >= n_slots) return;
+  const int s = indices[start + j];
+  if (s < 0 || s >= n_slots) return;
+  inv[s] = e * capacity + j;
+}
+
+__global__ void fill_kernel(int32_t* __restrict__ p, int64_t n, int32_t v) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = v;
+}
+
+// ------------------------------------------------------------------ combine (scatter)
+// out[t] = sum_j round(x[inv[t*k+j]] * w[t*k+j]); one wave per token.  Each product is
+// rounded to the storage type before the fp32 sum, as the reference's scaled copy into a
+// [tokens, top_k, hidden] buffer followed by sum(dim=1) does.
+template <int DT, bool VEC>
+__global__ void __launch_bounds__(kRowThreads)
+combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ inv,
+               const void* __restrict__ weights, int w_dtype, void* __restrict__ out_) {
+  typedef typename Elem<DT>::type E;
+  const E* x = (const E*)x_;
+  E* out = (E*)out_;
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  for (int64_t t = (int64_t)blockIdx.x * kRowWaves + wave; t < tokens; t += (int64_t)gridDim.x * kRowWaves) {
+    E* dst = out + t * hidden;
+    const int64_t s0 = t * top_k;
+    if (top_k == 1) {
+      const int row = inv[s0];
+      if (row < 0) { wave_zero_row<DT, VEC>(dst, hidden); continue; }
+      const float scale = weights ? load_as_f32(weights, s0, w_dtype) : 1.f;
+      wave_copy_row<DT, VEC>(x + (int64_t)row * hidden, dst, hidden, weights != nullptr, scale);
+      continue;
+    }
+    if (VEC) {
+      constexpr int EV = Vec16<DT>::kElems;
+      const int nvec = hidden / EV;
+      for (int c = lane; c < nvec; c += kWave) {
+        float acc[EV];
+#pragma unroll
+        for (int i = 0; i < EV; ++i) acc[i] = 0.f;
+        for (int j = 0; j < top_k; ++j) {
+          const int row = inv[s0 + j];
+          if (row < 0) continue;
+          const float scale = weights ? load_as_f32(weights, s0 + j, w_dtype) : 1.f;
+          float f[EV];
+          Vec16<DT>::unpack(((const u32x4*)(x + (int64_t)row * hidden))[c], f);
+#pragma unroll
+          for (int i = 0; i < EV; ++i)
+            acc[i] += weights ? Elem<DT>::to_f32(Elem<DT>::from_f32(f[i] * scale)) : f[i];
+        }
+        ((u32x4*)dst)[c] = Vec16<DT>::pack(acc);
+      }
+    } else {
+      for (int c = lane; c < hidden; c += kWave) {
+        float acc = 0.f;
+        for (int j = 0; j < top_k; ++j) {
+          const int row = inv[s0 + j];
+          if (row < 0) continue;
+          const float v = Elem<DT>::to_f32(x[(int64_t)row * hidden + c]);
+          acc += weights ? Elem<DT>::to_f32(Elem<DT>::from_f32(v * load_as_f32(weights, s0 + j, w_dtype))) : v;
+        }
+        dst[c] = Elem<DT>::from_f32(acc);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ wgrad
+template <int DT, bool VEC>
+__global__ void __launch_bounds__(kRowThreads)
+wgrad_kernel(const void* __restrict__ x_, const void* __restrict__ grad_, int64_t tokens, int hidden, int top_k,
+             const int32_t* __restrict__ indices, const int32_t* __restrict__ bin_ids, const int32_t* __restrict__ bins,
+             const int32_t* __restrict__ padded_bins, int num_bins, void* __restrict__ wgrad_) {
+  typedef typename Elem<DT>::type E;
+  const E* x = (const E*)x_;
+  const E* grad = (const E*)grad_;
+  E* wgrad = (E*)wgrad_;
+  const int n_slots = (int)(tokens * top_k);
+  const int wave = threadIdx.x / kWave;
+  for (int i = blockIdx.x * kRowWaves + wave; i < n_slots; i += gridDim.x * kRowWaves) {
+    const int s = indices[i];
+    if (s < 0 || s >= n_slots) continue;
+    int row = i;
+    if (padded_bins != nullptr) {
+      const int e = bin_ids[i];
+      if (e < 0 || e >= num_bins) continue;
+      if (e > 0) row = i - bins[e - 1] + padded_bins[e - 1];
+    }
+    const float d = wave_dot_row<DT, VEC>(x + (int64_t)row * hidden, grad + (int64_t)(s / top_k) * hidden, hidden);
+    if (lane_id() == 0) wgrad[s] = Elem<DT>::from_f32(d);
+  }
+}
+
+// ------------------------------------------------------------------ binned variants
+template <int DT, bool VEC>
+__global__ void __launch_bounds__(kRowThreads)
+binned_gather_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ indices,
+                     const int32_t* __restrict__ bins, int num_bins, int capacity, const void* __restrict__ weights,
+                     int w_dtype, void* __restrict__ out_) {
+  typedef typename Elem<DT>::type E;
+  const E* x = (const E*)x_;
+  E* out = (E*)out_;
+  const int n_slots = (int)(tokens * top_k);
+  const int wave = threadIdx.x / kWave;
+  const int64_t total = (int64_t)num_bins * capacity;
+  for (int64_t r = (int64_t)blockIdx.x * kRowWaves + wave; r < total; r += (int64_t)gridDim.x * kRowWaves) {
+    const int e = (int)(r / capacity), j = (int)(r % capacity);
+    const int start = e > 0 ? bins[e - 1] : 0;
+    E* dst = out + r * hidden;
+    int s = -1;
+    if (start + j < bins[e] && start + j < n_slots) s = indices[start + j];
+    if (s < 0 || s >= n_slots) { wave_zero_row<DT, VEC>(dst, hidden); continue; }
+    const float scale = weights ? load_as_f32(weights, s, w_dtype) : 1.f;
+    wave_copy_row<DT, VEC>(x + (int64_t)(s / top_k) * hidden, dst, hidden, weights != nullptr, scale);
+  }
+}
+
+template <int DT, bool VEC>
+__global__ void __launch_bounds__(kRowThreads)
+binned_wgrad_kernel(const void* __restrict__ x_, const void* __restrict__ grad_, int64_t tokens, int hidden, int top_k,
+                    const int32_t* __restrict__ indices, const int32_t* __restrict__ bins, int num_bins, int capacity,
+                    void* __restrict__ wgrad_) {
+  typedef typename Elem<DT>::type E;
+  const E* x = (const E*)x_;
+  const E* grad = (const E*)grad_;
+  E* wgrad = (E*)wgrad_;
+  const int n_slots = (int)(tokens * top_k);
+  const int wave = threadIdx.x / kWave;
+  const int64_t total = (int64_t)num_bins * capacity;
+  for (int64_t r = (int64_t)blockIdx.x * kRowWaves + wave; r < total; r += (int64_t)gridDim.x * kRowWaves) {
+    const int e = (int)(r / capacity), j = (int)(r % capacity);
+    const int start = e > 0 ? bins[e - 1] : 0;
+    if (start + j >= bins[e] || start + j >= n_slots) continue;
+    const int s = indices[start + j];
+    if (s < 0 || s >= n_slots) continue;
+    const float d = wave_dot_row<DT, VEC>(x + r * hidden, grad + (int64_t)(s / top_k) * hidden, hidden);
+    if (lane_id() == 0) wgrad[s] = Elem<DT>::from_f32(d);
+  }
+}
+
+template <typename T>
+__global__ void zero_kernel(T* __restrict__ p, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = (T)0;
+}
+
+// ------------------------------------------------------------------ host helpers
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+static inline bool can_vec(int dtype, int hidden, const void* a, const void* b, const void* c = nullptr) {
+  return ((int64_t)hidden * dtype_bytes(dtype)) % 16 == 0 && aligned16(a) && aligned16(b) && (c == nullptr || aligned16(c));
+}
+
+static inline unsigned row_grid(int64_t rows) {
+  int64_t blocks = ceil_div(rows, kRowWaves);
+  const int64_t cap = 256 * 16;  // 16 resident blocks of 4 waves per CU
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+#define MBX_DISPATCH_DT_VEC(dtype, vec, CALL)                    \
+  switch (dtype) {                                               \
+    case MBX_BF16: if (vec) { CALL(MBX_BF16, true); } else { CALL(MBX_BF16, false); } break; \
+    case MBX_F16: if (vec) { CALL(MBX_F16, true); } else { CALL(MBX_F16, false); } break;    \
+    case MBX_F32: if (vec) { CALL(MBX_F32, true); } else { CALL(MBX_F32, false); } break;    \
+    default: return MBX_EINVAL;                                  \
+  }
+
+static inline bool bad_dtype(int d) { return d != MBX_BF16 && d != MBX_F16 && d != MBX_F32; }
+
+}  // namespace
+}  // namespace mbx
+
+using namespace mbx;
+
+extern "C" {
+
+int mbx_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
+               const int32_t* bins, const int32_t* padded_bins, int num_bins, const void* weights, int w_dtype,
+               void* out, int64_t out_rows, mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || out_rows < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
+  if (out_rows == 0 || hidden == 0) return 0;
+  if (!out || (tokens > 0 && (!x || !indices)) || (padded_bins && !bins)) return MBX_EINVAL;
+  if (tokens * top_k > 0x7fffffff || out_rows > 0x7fffffff) return MBX_ERANGE;
+  const bool vec = can_vec(dtype, hidden, x ? x : out, out);
+  hipStream_t s = as_stream(stream);
+#define CALL(DT, V) gather_kernel<DT, V><<<row_grid(out_rows), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, indices, bins, padded_bins, num_bins, weights, w_dtype, out, out_rows)
+  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
+#undef CALL
+  return launch_status();
+}
+
+int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
+                const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins, int num_bins,
+                const void* weights, int w_dtype, void* out, void* scratch, size_t scratch_bytes, mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
+  if (tokens == 0 || hidden == 0) return 0;
+  if (!x || !out || !indices || (padded_bins && (!bins || !bin_ids))) return MBX_EINVAL;
+  const int64_t n_slots = tokens * top_k;
+  if (n_slots > 0x7fffffff) return MBX_ERANGE;
+  if (!scratch || scratch_bytes < (size_t)n_slots * sizeof(int32_t)) return MBX_ESCRATCH;
+  int32_t* inv = (int32_t*)scratch;
+  hipStream_t s = as_stream(stream);
+  const unsigned fb = (unsigned)(ceil_div(n_slots, 256) < 2048 ? ceil_div(n_slots, 256) : 2048);
+  fill_kernel<<<fb, 256, 0, s>>>(inv, n_slots, -1);
+  inverse_map_kernel<<<(unsigned)ceil_div(n_slots, 256), 256, 0, s>>>(indices, bin_ids, bins, padded_bins, num_bins, (int)n_slots, inv);
+  const bool vec = can_vec(dtype, hidden, x, out);
+#define CALL(DT, V) combine_kernel<DT, V><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out)
+  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
+#undef CALL
+  return launch_status();
+}
+
+int mbx_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int hidden, int top_k,
+                      const int32_t* indices, const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins,
+                      int num_bins, void* wgrad, mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (tokens == 0) return 0;
+  if (!wgrad || !indices || (hidden > 0 && (!x || !grad)) || (padded_bins && (!bins || !bin_ids))) return MBX_EINVAL;
+  const int64_t n_slots = tokens * top_k;
+  if (n_slots > 0x7fffffff) return MBX_ERANGE;
+  const bool vec = can_vec(dtype, hidden, x, grad);
+  hipStream_t s = as_stream(stream);
+#define CALL(DT, V) wgrad_kernel<DT, V><<<row_grid(n_slots), kRowThreads, 0, s>>>(x, grad, tokens, hidden, top_k, indices, bin_ids, bins, padded_bins, num_bins, wgrad)
+  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
+#undef CALL
+  return launch_status();
+}
+
+int mbx_binned_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
+                      const int32_t* bins, int num_bins, int capacity, const void* weights, int w_dtype, void* out,
+                      mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || capacity < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
+  const int64_t total = (int64_t)num_bins * capacity;
+  if (total == 0 || hidden == 0) return 0;
+  if (!out || !bins || (tokens > 0 && (!x || !indices))) return MBX_EINVAL;
+  if (tokens * top_k > 0x7fffffff || total > 0x7fffffff) return MBX_ERANGE;
+  const bool vec = can_vec(dtype, hidden, x ? x : out, out);
+  hipStream_t s = as_stream(stream);
+#define CALL(DT, V) binned_gather_kernel<DT, V><<<row_grid(total), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, indices, bins, num_bins, capacity, weights, w_dtype, out)
+  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
+#undef CALL
+  return launch_status();
+}
+
+static int binned_inverse(const int32_t* indices, const int32_t* bins, int num_bins, int capacity, int64_t n_slots,
+                          int32_t* inv, hipStream_t s) {
+  const unsigned fb = (unsigned)(ceil_div(n_slots, 256) < 2048 ? ceil_div(n_slots, 256) : 2048);
+  fill_kernel<<<fb, 256, 0, s>>>(inv, n_slots, -1);
+  if (num_bins > 0 && capacity > 0) {
+    if (num_bins > 65535) return MBX_ERANGE;
+    dim3 grid((unsigned)ceil_div(capacity, 256), (unsigned)num_bins);
+    binned_inverse_map_kernel<<<grid, 256, 0, s>>>(indices, bins, capacity, (int)n_slots, inv);
+  }
+  return 0;
+}
+
+int mbx_binned_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
+                       const int32_t* bins, int num_bins, int capacity, const void* weights, int w_dtype, void* out,
+                       void* scratch, size_t scratch_bytes, mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || capacity < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
+  if (tokens == 0 || hidden == 0) return 0;
+  if (!out || !indices || (num_bins > 0 && !bins) || ((int64_t)num_bins * capacity > 0 && !x)) return MBX_EINVAL;
+  const int64_t n_slots = tokens * top_k;
+  if (n_slots > 0x7fffffff || (int64_t)num_bins * capacity > 0x7fffffff) return MBX_ERANGE;
+  if (!scratch || scratch_bytes < (size_t)n_slots * sizeof(int32_t)) return MBX_ESCRATCH;
+  int32_t* inv = (int32_t*)scratch;
+  hipStream_t s = as_stream(stream);
+  const int rc = binned_inverse(indices, bins, num_bins, capacity, n_slots, inv, s);
+  if (rc) return rc;
+  const bool vec = can_vec(dtype, hidden, x ? x : out, out);
+#define CALL(DT, V) combine_kernel<DT, V><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out)
+  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
+#undef CALL
+  return launch_status();
+}
+
+int mbx_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int hidden, int top_k,
+                             const int32_t* indices, const int32_t* bins, int num_bins, int capacity, void* wgrad,
+                             mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || capacity < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (tokens == 0) return 0;
+  const int64_t n_slots = tokens * top_k;
+  const int64_t total = (int64_t)num_bins * capacity;
+  if (!wgrad || !indices || (num_bins > 0 && !bins) || (total > 0 && hidden > 0 && (!x || !grad))) return MBX_EINVAL;
+  if (n_slots > 0x7fffffff || total > 0x7fffffff) return MBX_ERANGE;
+  hipStream_t s = as_stream(stream);
+  const unsigned fb = (unsigned)(ceil_div(n_slots, 256) < 2048 ? ceil_div(n_slots, 256) : 2048);
+  if (dtype_bytes(dtype) == 2) zero_kernel<uint16_t><<<fb, 256, 0, s>>>((uint16_t*)wgrad, n_slots);
+  else zero_kernel<uint32_t><<<fb, 256, 0, s>>>((uint32_t*)wgrad, n_slots);
+  if (total > 0) {
+    const bool vec = can_vec(dtype, hidden, x, grad);
+#define CALL(DT, V) binned_wgrad_kernel<DT, V><<<row_grid(total), kRowThreads, 0, s>>>(x, grad, tokens, hidden, top_k, indices, bins, num_bins, capacity, wgrad)
+    MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
+#undef CALL
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,119 @@
+"""Grouped GEMM entry points with the interface the reference reaches through
+megablocks/grouped_gemm_util.py:25-26 (`gg.backend.gmm`, `gg.ops.gmm`), served by the
+bf16/f16 MFMA kernels of libmbx.so.
+
+`batch_sizes` may be the host int64 tensor the reference passes (mlp.py:502) or, to avoid
+the device-to-host copy, a device tensor of per-expert row counts.
+"""
+import types
+
+import torch
+
+from megablocks_amd import _lib
+from megablocks_amd._lib import lib
+
+
+def grouped_gemm_is_available():
+    return True
+
+
+def assert_grouped_gemm_is_available():
+    assert grouped_gemm_is_available()
+
+
+def _device_bins(batch_sizes: torch.Tensor, device) -> torch.Tensor:
+    """Inclusive int32 row bins on the device for a vector of group sizes (cached on the tensor)."""
+    cached = getattr(batch_sizes, '_mbx_bins', None)
+    if cached is not None and cached[1] == batch_sizes._version and cached[0].device == device:
+        return cached[0]
+    if batch_sizes.ndim != 1:
+        raise ValueError('batch_sizes must be a vector')
+    if batch_sizes.is_cuda:
+        from megablocks_amd.ops.routing import inclusive_cumsum
+        bins = inclusive_cumsum(batch_sizes.to(torch.int32), 0).view(-1)
+    else:
+        bins = torch.cumsum(batch_sizes, 0).to(torch.int32).to(device)
+    try:
+        batch_sizes._mbx_bins = (bins, batch_sizes._version)
+    except Exception:
+        pass
+    return bins
+
+
+def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None):
+    """out[r_e] = a[r_e] @ b[e] (`trans_b`: @ b[e].T); `trans_a`: out[e] = a[r_e].T @ b[r_e].
+
+    a is [rows, k]; b is [E, k, n] ([E, n, k] with trans_b) or, with trans_a, [rows, n].
+    fp32 accumulation, output in a.dtype, written to `c` when given.
+    """
+    _lib.require_cuda(a, b, c)
+    if a.ndim != 2:
+        raise ValueError('gmm: a must be a matrix')
+    if a.dtype != b.dtype:
+        raise ValueError('gmm: a and b must share a dtype')
+    if trans_a and trans_b:
+        raise ValueError('gmm: trans_a and trans_b cannot both be set')
+    dt = _lib.dtype_of(a)
+    a, b = a.contiguous(), b.contiguous()
+    bins = _device_bins(batch_sizes, a.device)
+    groups = bins.shape[0]
+    rows = a.shape[0]
+    if trans_a:
+        if b.ndim != 2 or b.shape[0] != rows:
+            raise ValueError('gmm(trans_a): b must be [rows, n]')
+        k, n, layout = a.shape[1], b.shape[1], _lib.TN
+        shape = (groups, k, n)
+    else:
+        if b.ndim != 3 or b.shape[0] != groups:
+            raise ValueError('gmm: b must be [num_groups, ., .]')
+        k = a.shape[1]
+        if trans_b:
+            n, layout = b.shape[1], _lib.NT
+            if b.shape[2] != k:
+                raise ValueError('gmm(trans_b): inner dimensions differ')
+        else:
+            n, layout = b.shape[2], _lib.NN
+            if b.shape[1] != k:
+                raise ValueError('gmm: inner dimensions differ')
+        shape = (rows, n)
+    if c is None:
+        c = torch.empty(shape, dtype=a.dtype, device=a.device)
+    else:
+        if tuple(c.shape) != shape or c.dtype != a.dtype or not c.is_contiguous():
+            raise ValueError('gmm: c has the wrong shape, dtype or layout')
+    with torch.cuda.device_of(a):
+        _lib.check(lib.mbx_gmm(_lib.ptr(a), _lib.ptr(b), _lib.ptr(c), dt, _lib.ptr(bins), groups, rows, k, n, layout,
+                               _lib.stream()), 'gmm')
+    return c
+
+
+class GroupedGemm(torch.autograd.Function):
+    """Differentiable gmm(a, b, batch_sizes, trans_b): da = gmm(dc, b, trans_b flipped),
+    db = the per-group outer product (trans_a)."""
+
+    @staticmethod
+    def forward(ctx, a, b, batch_sizes, trans_b):
+        ctx.save_for_backward(a, b, batch_sizes)
+        ctx.trans_b = trans_b
+        return gmm(a, b, batch_sizes, trans_a=False, trans_b=trans_b)
+
+    @staticmethod
+    def backward(ctx, grad):
+        grad = grad.contiguous()
+        a, b, batch_sizes = ctx.saved_tensors
+        trans_b = ctx.trans_b
+        agrad = bgrad = None
+        if ctx.needs_input_grad[0]:
+            agrad = gmm(grad, b, batch_sizes, trans_a=False, trans_b=not trans_b)
+        if ctx.needs_input_grad[1]:
+            lhs, rhs = (grad, a) if trans_b else (a, grad)
+            bgrad = gmm(lhs, rhs, batch_sizes, trans_a=True, trans_b=False)
+        return agrad, bgrad, None, None
+
+
+def _ops_gmm(a, b, batch_sizes, trans_b=False):
+    return GroupedGemm.apply(a, b, batch_sizes, trans_b)
+
+
+backend = types.SimpleNamespace(gmm=gmm)
+ops = types.SimpleNamespace(gmm=_ops_gmm)

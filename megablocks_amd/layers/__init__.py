@@ -1,0 +1,8 @@
+from megablocks_amd.layers.arguments import Arguments
+from megablocks_amd.layers.dmoe import ParallelDroplessMLP, dMoE
+from megablocks_amd.layers.glu import SparseGLU
+from megablocks_amd.layers.mlp import MLP, SparseMLP
+from megablocks_amd.layers.moe import MoE, ParallelMLP, get_load_balancing_loss
+
+__all__ = ['MoE', 'dMoE', 'get_load_balancing_loss', 'ParallelMLP', 'ParallelDroplessMLP', 'SparseMLP', 'MLP',
+           'SparseGLU', 'Arguments']

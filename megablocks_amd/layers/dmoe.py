@@ -1,0 +1,136 @@
+"""The dropless MoE layer: megablocks/layers/dmoe.py.
+
+    grouped:  sort/histogram/cumsum -> gather -> grouped MLP -> weighted scatter
+    sparse:   the same over 128-padded expert groups, with the block-diagonal topology
+              metadata the reference builds for stk
+"""
+import numpy as np
+import torch
+
+import megablocks_amd.ops as ops
+from megablocks_amd.layers import common, dmlp_registry, moe, mpu
+from megablocks_amd.layers.arguments import Arguments
+from megablocks_amd.layers.mlp import Topology
+
+
+def promote_scalar(x):
+    return x.view(1) if not len(x.size()) else x
+
+
+class ParallelDroplessMLP(moe.ParallelMLP):
+
+    _builds_dense_mlp = False   # the reference builds a dense MLP here and replaces it at once (dmoe.py:25)
+
+    def __init__(self, args: Arguments):
+        super().__init__(args)
+        self.hidden_size = args.hidden_size
+        self.ffn_hidden_size = mpu.features_per_rank(args)
+        self.blocking = 128
+        self.mlp = dmlp_registry.get(args)
+        # bits needed for a block-column index of the intermediate sparse matrix (dmoe.py:27-33)
+        max_column_index = (self.ffn_hidden_size * self.num_experts) // self.blocking
+        self.transpose_sort_end_bit = max(int(np.ceil(np.log2(max(max_column_index, 1)))), 1)
+
+    def sparse_transpose(self, size, row_indices, column_indices, offsets):
+        """dmoe.py:35-66: metadata of the transposed block-sparse matrix."""
+        block_columns = size[1] // self.blocking
+        _, gather_indices = ops.sort(column_indices.int(), self.transpose_sort_end_bit)
+        column_indices_t = row_indices.gather(0, gather_indices.long())
+        block_offsets_t = gather_indices.int()
+        zero = torch.zeros((1,), dtype=torch.int32, device=row_indices.device)
+        nnz_per_column = ops.histogram(column_indices, block_columns)
+        nnz_per_column = ops.inclusive_cumsum(nnz_per_column, 0)
+        if nnz_per_column.dim() == 0:
+            nnz_per_column = nnz_per_column.unsqueeze(0)
+        offsets_t = torch.cat([zero, nnz_per_column])
+        return column_indices_t, offsets_t, block_offsets_t
+
+    def topology(self, x, padded_bins):
+        """dmoe.py:68-129."""
+        padded_tokens, _ = x.size()
+        assert padded_tokens % self.blocking == 0
+        if self.ffn_hidden_size % self.blocking != 0:
+            raise ValueError(f'The ffn_hidden_size {self.ffn_hidden_size} must be divisible by ' +
+                             f'the block size {self.blocking}. Please update your configuration.')
+        block_rows = padded_tokens // self.blocking
+        blocks_per_row = self.ffn_hidden_size // self.blocking
+        offsets = torch.arange(0, block_rows * blocks_per_row + 1, blocks_per_row, dtype=torch.int32, device=x.device)
+        column_indices = ops.topology(padded_bins, self.blocking, block_rows, blocks_per_row)
+        shape = (padded_tokens, self.ffn_hidden_size * mpu.experts_per_rank(self.args))
+        # every block-row holds blocks_per_row blocks, so block b lies in block-row b // blocks_per_row
+        row_indices = torch.arange(block_rows, dtype=torch.int32, device=x.device).repeat_interleave(
+            blocks_per_row).to(torch.int16)
+        column_indices_t, offsets_t, block_offsets_t = self.sparse_transpose(shape, row_indices, column_indices, offsets)
+        padded_tokens_per_expert = torch.diff(padded_bins, prepend=padded_bins.new_zeros(1))
+        return Topology(shape, self.blocking, row_indices, column_indices, offsets, column_indices_t, offsets_t,
+                        block_offsets_t, padded_tokens_per_expert)
+
+    def indices_and_padded_bins(self, top_experts):
+        """dmoe.py:131-154."""
+        top_experts = top_experts.int()
+        bin_ids, indices = ops.sort(top_experts, self.sort_end_bit)
+        tokens_per_expert = ops.histogram(top_experts, self.num_experts)
+        padded_tokens_per_expert = ops.round_up(tokens_per_expert, self.blocking)
+        padded_bins = promote_scalar(ops.inclusive_cumsum(padded_tokens_per_expert, 0))
+        bins = promote_scalar(ops.inclusive_cumsum(tokens_per_expert, 0))
+        return indices, bin_ids, bins, padded_bins, tokens_per_expert
+
+    def sparse_forward_once(self, x, expert_weights, top_experts):
+        """dmoe.py:156-193."""
+        expert_weights = expert_weights.flatten()
+        top_experts = top_experts.flatten()
+        with torch.no_grad():
+            indices, bin_ids, bins, padded_bins, tokens_per_expert = self.indices_and_padded_bins(top_experts)
+        x = x.view(-1, x.shape[-1])
+        x = ops.padded_gather(x, indices, bin_ids, bins, padded_bins, self.top_k)
+        with torch.no_grad():
+            topo = self.topology(x, padded_bins)
+        x = self.mlp(x, topo)
+        x = ops.padded_scatter(x, indices, bin_ids, expert_weights, bins, padded_bins, self.top_k)
+        return x, tokens_per_expert
+
+    def sparse_permute_and_compute(self, x, tokens_per_expert, indices, bin_ids, expert_weights, bins,
+                                   expert_capactiy, top_k):
+        """dmoe.py:196-237."""
+        padded_tokens_per_expert = ops.round_up(tokens_per_expert, self.blocking)
+        padded_bins = promote_scalar(ops.inclusive_cumsum(padded_tokens_per_expert, 0))
+        x = x.view(-1, x.shape[-1])
+        x = ops.padded_gather(x, indices, bin_ids, bins, padded_bins, top_k)
+        with torch.no_grad():
+            topo = self.topology(x, padded_bins)
+        x = self.mlp(x, topo)
+        return ops.padded_scatter(x, indices, bin_ids, expert_weights, bins, padded_bins, top_k)
+
+    def grouped_forward_once(self, x, expert_weights, top_experts):
+        """dmoe.py:239-258."""
+        expert_weights = expert_weights.flatten()
+        top_experts = top_experts.flatten()
+        with torch.no_grad():
+            indices, bin_ids, bins, tokens_per_expert = self.indices_and_bins(top_experts)
+        out = self.grouped_permute_and_compute(x, tokens_per_expert, indices, bin_ids, expert_weights, bins, -1,
+                                               self.args.moe_top_k)
+        return out, tokens_per_expert
+
+    def grouped_permute_and_compute(self, x, tokens_per_expert, indices, bin_ids, expert_weights, bins,
+                                    expert_capactiy, top_k):
+        """dmoe.py:260-280."""
+        x = x.view(-1, x.shape[-1])
+        x = ops.gather(x, indices, bin_ids, bins, top_k)
+        x = self.mlp(x, tokens_per_expert)
+        return ops.scatter(x, indices, bin_ids, expert_weights, bins, top_k)
+
+    def forward_once(self, x, expert_weights, top_experts):
+        if self.args.mlp_impl == 'sparse':
+            return self.sparse_forward_once(x, expert_weights, top_experts)
+        return self.grouped_forward_once(x, expert_weights, top_experts)
+
+    def permute_and_compute(self, x, tokens_per_expert, indices, bin_ids, expert_weights, bins, expert_capactiy,
+                            top_k):
+        fn = self.sparse_permute_and_compute if self.args.mlp_impl == 'sparse' else self.grouped_permute_and_compute
+        return fn(x, tokens_per_expert, indices, bin_ids, expert_weights, bins, expert_capactiy, top_k)
+
+
+class dMoE(moe.MoE):
+
+    def _init_experts_mlp(self, args: Arguments):
+        return ParallelDroplessMLP(args)

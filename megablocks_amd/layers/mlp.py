@@ -1,0 +1,228 @@
+"""Expert MLPs of the dropless MoE: megablocks/layers/mlp.py.
+
+Weights keep the reference layout `[num_experts * ffn_hidden_size, hidden_size]` for both
+w1 and w2 (mlp.py:315-330), so the first product is `x @ w1[e].T` (NT) and the second
+`h @ w2[e]` (NN).  The block-sparse formulation of the reference (`mlp_impl='sparse'`, stk
+sdd/dsd on a block-diagonal topology) is the same pair of grouped products taken over
+128-padded row groups, and is computed that way here.
+"""
+import dataclasses
+from typing import Any, Optional
+
+import torch
+
+from megablocks_amd import grouped_gemm_util as gg
+from megablocks_amd.layers import common, gelu, mpu
+from megablocks_amd.layers.arguments import DEFAULT_ACTIVATION_FN, Arguments, InitFn
+
+
+class ScaleGradient(torch.autograd.Function):
+    """mlp.py:18-31."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
+    def forward(ctx: Any, x: torch.Tensor, scale: float):
+        ctx.scale = scale
+        return x
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
+    def backward(ctx: Any, grad: torch.Tensor):
+        return grad * ctx.scale, None
+
+
+scale_gradient = ScaleGradient.apply
+
+
+def resolve_dtensor(weight: torch.Tensor):
+    """mlp.py:35-40."""
+    try:
+        from torch.distributed._tensor import DTensor
+    except Exception:  # torch built without distributed
+        return weight
+    if isinstance(weight, DTensor):
+        return weight.to_local()
+    return weight
+
+
+def create_moe_expert_weights(args: Arguments, num_experts: int, ffn_hidden_size: int, hidden_size: int,
+                              init_method: InitFn):
+    """mlp.py:43-88 without the expert-parallel slicing: [E, ffn, hidden], initialised in one call
+    so that the values do not depend on how experts are later divided."""
+    master_weights = torch.empty(num_experts, ffn_hidden_size, hidden_size, device=args.device,
+                                 dtype=common.dtype(args))
+    init_method(master_weights)
+    return master_weights
+
+
+def create_dmoe_expert_weights(args: Arguments, num_experts: int, rows: int, columns: int, init_method: InitFn):
+    """mlp.py:170-184."""
+    return create_moe_expert_weights(args, num_experts, rows, columns, init_method).view([-1, columns])
+
+
+class MLP(torch.nn.Module):
+    """Batched expert MLP of the capacity-factor MoE (mlp.py:91-167): w1 [E, hidden, ffn],
+    w2 [E, ffn, hidden], x [E, capacity, hidden]."""
+
+    def __init__(self, args: Arguments):
+        super().__init__()
+        self.args = args
+        experts = mpu.experts_per_rank(args)
+        self.w1 = torch.nn.Parameter(torch.empty(experts, args.hidden_size, mpu.features_per_rank(args),
+                                                 device=args.device, dtype=common.dtype(args)))
+        self.w2 = torch.nn.Parameter(torch.empty(experts, mpu.features_per_rank(args), args.hidden_size,
+                                                 device=args.device, dtype=common.dtype(args)))
+        mpu.set_expert_model_parallel_attributes(self.w1, args.moe_expert_model_parallelism)
+        mpu.set_expert_model_parallel_attributes(self.w2, args.moe_expert_model_parallelism)
+        with torch.no_grad():
+            w1 = create_moe_expert_weights(args, args.moe_num_experts, args.ffn_hidden_size, args.hidden_size,
+                                           args.init_method)
+            self.w1.copy_(w1.transpose(1, 2).contiguous())
+            self.w2.copy_(create_moe_expert_weights(args, args.moe_num_experts, args.ffn_hidden_size,
+                                                    args.hidden_size, args.output_layer_init_method))
+        self.gradient_scale = None
+
+    def scale_grad(self, w):
+        if self.gradient_scale is None:
+            return w
+        return scale_gradient(w, self.gradient_scale)
+
+    def forward(self, x):
+        w1, w2 = resolve_dtensor(self.scale_grad(self.w1)), resolve_dtensor(self.scale_grad(self.w2))
+        x = torch.bmm(x, w1)
+        x = self.args.activation_fn(x)
+        return torch.bmm(x, w2)
+
+
+@dataclasses.dataclass
+class Topology:
+    """Metadata of the block-diagonal sparse matrix the reference hands to stk (what
+    `stk.Matrix(shape, data, row_indices, column_indices, offsets, column_indices_t, offsets_t,
+    block_offsets_t)` carries at dmoe.py:120-129), plus the padded row groups it was built from."""
+    shape: tuple
+    blocking: int
+    row_indices: torch.Tensor
+    column_indices: torch.Tensor
+    offsets: torch.Tensor
+    column_indices_t: torch.Tensor
+    offsets_t: torch.Tensor
+    block_offsets_t: torch.Tensor
+    padded_tokens_per_expert: torch.Tensor   # int32 [E], multiples of `blocking`
+
+    def size(self):
+        return self.shape
+
+    @property
+    def nnz(self):
+        return self.column_indices.numel()
+
+
+class MemoryOptimizedGroupedMLP(torch.autograd.Function):
+    """GroupedMLP with a hand-scheduled backward that recomputes the activation and reuses
+    buffers (mlp.py:397-493)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
+    def forward(ctx, x, w1, w2, batch_sizes, activation_fn):
+        if ctx._fwd_used_autocast:
+            x, w1, w2 = x.to(ctx._dtype), w1.to(ctx._dtype), w2.to(ctx._dtype)
+        if not x.is_contiguous() or not w1.is_contiguous() or not w2.is_contiguous():
+            raise ValueError("Expected contiguous 'x', 'w1' and 'w2'.")
+        sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
+        activation_fn_out = activation_fn(sdd_out)
+        dsd_out = gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+        ctx.x_shape = x.shape
+        ctx.sdd_out_shape = sdd_out.shape
+        ctx.dtype = x.dtype
+        ctx.activation_fn = activation_fn
+        ctx.save_for_backward(w1, w2, batch_sizes, x, sdd_out)
+        return dsd_out
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
+    def backward(ctx: Any, ddsd_out: torch.Tensor):
+        if not ctx.needs_input_grad[0] or not ctx.needs_input_grad[1] or not ctx.needs_input_grad[2]:
+            raise ValueError('Expected all MLP inputs to need grad.')
+        w1, w2, batch_sizes, x, sdd_out = ctx.saved_tensors
+        ddsd_out = ddsd_out.contiguous()
+        activation_fn = ctx.activation_fn
+        default_act = activation_fn is DEFAULT_ACTIVATION_FN
+
+        # Recompute the activation (kept in the graph only when its gradient is taken by autograd).
+        if default_act:
+            activation_fn_out = activation_fn(sdd_out)
+        else:
+            with torch.set_grad_enabled(True):
+                sdd_out = sdd_out.detach().requires_grad_(True)
+                activation_fn_out = activation_fn(sdd_out)
+
+        dw2 = gg.backend.gmm(activation_fn_out.detach(), ddsd_out, batch_sizes, trans_a=True)
+
+        if default_act:
+            # d(activation output) overwrites the recomputed activation, then becomes d(sdd_out) in place.
+            dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True, c=activation_fn_out)
+            dsdd_out = gelu.gelu_backward_(dactivation_fn_out, sdd_out)
+        else:
+            dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True)
+            activation_fn_out.backward(dactivation_fn_out)
+            dsdd_out = sdd_out.grad
+
+        dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
+        dx = gg.backend.gmm(dsdd_out, w1, batch_sizes, c=ddsd_out)   # reuses the incoming gradient buffer
+        return dx, dw1, dw2, None, None
+
+
+memory_optimized_grouped_mlp = MemoryOptimizedGroupedMLP.apply
+# The block-sparse memory-optimised MLP (mlp.py:187-302) is the same schedule over padded groups.
+memory_optimized_mlp = MemoryOptimizedGroupedMLP.apply
+
+
+class SparseMLP(torch.nn.Module):
+    """Owner of the dMoE expert weights w1, w2 : [E * ffn, hidden] (mlp.py:308-394).  Its forward
+    takes the padded activations and the block-diagonal topology."""
+
+    def __init__(self, args: Arguments):
+        super().__init__()
+        self.args = args
+        self._num_rows_per_rank = mpu.experts_per_rank(args) * mpu.features_per_rank(args)
+        self.w1 = torch.nn.Parameter(torch.empty(self._num_rows_per_rank, args.hidden_size, device=args.device,
+                                                 dtype=common.dtype(args)))
+        self.w2 = torch.nn.Parameter(torch.empty(self._num_rows_per_rank, args.hidden_size, device=args.device,
+                                                 dtype=common.dtype(args)))
+        with torch.no_grad():
+            self.w1.copy_(create_dmoe_expert_weights(args, args.moe_num_experts, args.ffn_hidden_size,
+                                                     args.hidden_size, args.init_method))
+            self.w2.copy_(create_dmoe_expert_weights(args, args.moe_num_experts, args.ffn_hidden_size,
+                                                     args.hidden_size, args.output_layer_init_method))
+        self._should_set_parallelism_attribute = args.moe_expert_model_parallelism
+        mpu.set_expert_model_parallel_attributes(self.w1, self._should_set_parallelism_attribute)
+        mpu.set_expert_model_parallel_attributes(self.w2, self._should_set_parallelism_attribute)
+        self.gradient_scale = None
+
+    def scale_grad(self, w):
+        if self.gradient_scale is None:
+            return w
+        return scale_gradient(w, self.gradient_scale)
+
+    def _expert_views(self, *weights):
+        ne = mpu.experts_per_rank(self.args)
+        return [resolve_dtensor(self.scale_grad(w)).view(ne, -1, self.args.hidden_size) for w in weights]
+
+    def _compute(self, x, batch_sizes):
+        w1, w2 = self._expert_views(self.w1, self.w2)
+        if self.args.memory_optimized_mlp:
+            return memory_optimized_grouped_mlp(x, w1, w2, batch_sizes, self.args.activation_fn)
+        x = gg.ops.gmm(x, w1, batch_sizes, trans_b=True)
+        x = self.args.activation_fn(x)
+        return gg.ops.gmm(x, w2, batch_sizes)
+
+    def forward(self, x, topo: Topology):
+        return self._compute(x, topo.padded_tokens_per_expert)
+
+
+class GroupedMLP(SparseMLP):
+    """mlp.py:499-523.  `tokens_per_expert` stays on the device: the grouped GEMM reads the row
+    bins there, so the reference's `.cpu()` copy (mlp.py:502) is not needed."""
+
+    def forward(self, x, tokens_per_expert):
+        return self._compute(x, tokens_per_expert)

@@ -1,0 +1,153 @@
+"""GPU parity tests of the grouped GEMM: against the CPU oracle at small sizes and against an
+fp32 torch formulation on the GPU at the benchmark shapes.  Tolerance: relative Frobenius
+error <= 1e-2 (bf16/f16 inputs, fp32 accumulation)."""
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+@pytest.fixture(scope='module')
+def gg():
+    from megablocks_amd import grouped_gemm_util as gg
+    return gg
+
+
+def rel_err(a, b):
+    a, b = a.double(), b.double()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
+def _sizes(groups, rows, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    cuts = torch.sort(torch.randint(0, rows + 1, (groups - 1,), generator=g))[0]
+    sizes = torch.diff(torch.cat([torch.zeros(1, dtype=torch.int64), cuts, torch.tensor([rows])]))
+    for e in empty:                      # force some empty groups, keep the total
+        if e + 1 < groups:
+            sizes[e + 1] += sizes[e]
+            sizes[e] = 0
+    return sizes
+
+
+def _ref_gpu(a, b, sizes, trans_a, trans_b):
+    a, b = a.float(), b.float()
+    outs, start = [], 0
+    for e, n in enumerate(sizes.tolist()):
+        ae = a[start:start + n]
+        if trans_a:
+            outs.append(ae.t() @ b[start:start + n])
+        else:
+            outs.append(ae @ (b[e].t() if trans_b else b[e]))
+        start += n
+    return torch.stack(outs) if trans_a else torch.cat(outs)
+
+
+SMALL = [  # groups, rows, k, n
+    (1, 128, 128, 128), (4, 512, 64, 256), (8, 1000, 256, 512), (3, 777, 72, 40), (5, 300, 100, 36),
+    (2, 64, 8, 8), (16, 2048, 512, 1408), (4, 50, 33, 17), (1, 1, 16, 16), (8, 4096, 1024, 256),
+]
+
+
+@pytest.mark.parametrize('groups,rows,k,n', SMALL)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('mode', ['nn', 'nt', 'tn'])
+def test_gmm_vs_oracle(gg, groups, rows, k, n, dtype, mode):
+    sizes = _sizes(groups, rows, seed=groups * 1000 + rows, empty=(1,) if groups > 2 else ())
+    a = torch.randn(rows, k).to(dtype)
+    if mode == 'tn':
+        b = torch.randn(rows, n).to(dtype)
+    elif mode == 'nt':
+        b = (torch.randn(groups, n, k) * 0.1).to(dtype)
+    else:
+        b = (torch.randn(groups, k, n) * 0.1).to(dtype)
+    want = oracle.gmm(a, b, sizes, trans_a=mode == 'tn', trans_b=mode == 'nt')
+    got = gg.backend.gmm(a.cuda(), b.cuda(), sizes, trans_a=mode == 'tn', trans_b=mode == 'nt')
+    assert got.shape == want.shape and got.dtype == dtype
+    assert rel_err(got.cpu(), want) < TOL
+    if mode == 'tn':
+        for e, s in enumerate(sizes.tolist()):
+            if s == 0:
+                assert torch.count_nonzero(got[e]) == 0          # unused expert: exactly zero gradient
+    got_dev = gg.backend.gmm(a.cuda(), b.cuda(), sizes.cuda().int(), trans_a=mode == 'tn', trans_b=mode == 'nt')
+    assert torch.equal(got_dev, got)                              # device-resident sizes: same kernel, same result
+
+
+def test_gmm_c_argument_and_errors(gg):
+    sizes = torch.tensor([100, 28])
+    a = torch.randn(128, 64).bfloat16().cuda()
+    b = torch.randn(2, 64, 32).bfloat16().cuda()
+    c = torch.full((128, 32), 7.0).bfloat16().cuda()
+    out = gg.backend.gmm(a, b, sizes, c=c)
+    assert out is c and rel_err(c.cpu(), oracle.gmm(a.cpu(), b.cpu(), sizes)) < TOL
+    with pytest.raises(ValueError):
+        gg.backend.gmm(a, b, sizes, c=torch.empty(128, 31).bfloat16().cuda())
+    with pytest.raises(ValueError):
+        gg.backend.gmm(a, b.float(), sizes)
+    with pytest.raises(ValueError):
+        gg.backend.gmm(a, b, sizes, trans_b=True)
+    short = torch.tensor([60, 20])                                # rows past the last bin are left alone
+    c2 = torch.full((128, 32), 7.0).bfloat16().cuda()
+    gg.backend.gmm(a, b, short, c=c2)
+    assert bool((c2[80:] == 7.0).all()) and rel_err(c2[:80].cpu(), oracle.gmm(a[:80].cpu(), b.cpu(), short)) < TOL
+
+
+BIG = [  # name, groups, rows, hidden, ffn, skew
+    ('gpt2-64e', 64, 16384, 1024, 4096, False),
+    ('mixtral', 8, 16384, 4096, 14336, False),
+    ('finegrained-zipf', 64, 32768, 2048, 1408, True),
+    ('sparse-padded', 16, 12288, 2048, 8192, False),
+]
+
+
+@pytest.mark.parametrize('name,groups,rows,hidden,ffn,skew', BIG)
+def test_gmm_benchmark_shapes_vs_fp32(gg, name, groups, rows, hidden, ffn, skew):
+    torch.manual_seed(1)
+    if skew:
+        p = torch.arange(1, groups + 1).float() ** -1.2
+        p[-4:] = 0                                               # four experts receive nothing
+        sizes = torch.bincount(torch.multinomial(p, rows, replacement=True), minlength=groups)
+    else:
+        sizes = _sizes(groups, rows, seed=3)
+    x = torch.randn(rows, hidden, device='cuda').bfloat16()
+    w = (torch.randn(groups, ffn, hidden, device='cuda') * 0.02).bfloat16()
+    h = gg.backend.gmm(x, w, sizes, trans_b=True)                               # NT
+    assert rel_err(h, _ref_gpu(x, w, sizes, False, True)) < TOL
+    y = gg.backend.gmm(h, w, sizes)                                             # NN
+    assert rel_err(y, _ref_gpu(h, w, sizes, False, False)) < TOL
+    dw = gg.backend.gmm(h, x, sizes, trans_a=True)                              # TN
+    ref = _ref_gpu(h, x, sizes, True, False)
+    assert rel_err(dw, ref) < TOL
+    for e, s in enumerate(sizes.tolist()):
+        if s == 0:
+            assert torch.count_nonzero(dw[e]) == 0
+
+
+def test_gmm_autograd(gg):
+    sizes = torch.tensor([300, 0, 212])
+    a = torch.randn(512, 256, device='cuda').bfloat16().requires_grad_(True)
+    b = (torch.randn(3, 128, 256, device='cuda') * 0.1).bfloat16().requires_grad_(True)
+    gout = torch.randn(512, 128, device='cuda').bfloat16()
+    gg.ops.gmm(a, b, sizes, True).backward(gout)
+    af, bf = a.detach().float().requires_grad_(True), b.detach().float().requires_grad_(True)
+    outs, start = [], 0
+    for e, n in enumerate(sizes.tolist()):
+        outs.append(af[start:start + n] @ bf[e].t())
+        start += n
+    torch.cat(outs).backward(gout.float())
+    assert rel_err(a.grad, af.grad) < TOL and rel_err(b.grad, bf.grad) < TOL
+    assert torch.count_nonzero(b.grad[1]) == 0
+
+
+def test_gelu_backward_inplace():
+    from megablocks_amd.layers.gelu import gelu_backward_
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        x = torch.randn(1000, 257).to(dtype)
+        g = torch.randn(1000, 257).to(dtype)
+        want = oracle.gelu_tanh_backward(g.float(), x.float())
+        gd = g.cuda()
+        out = gelu_backward_(gd, x.cuda())
+        assert out is gd and rel_err(gd.cpu().float(), want) < (1e-5 if dtype == torch.float32 else 1e-2)

@@ -1,0 +1,294 @@
+"""GPU parity tests of the routing and permutation operators against the CPU oracle.
+
+Shapes follow the reference's tests/ops/*_test.py.  Integer results, permutations and
+unweighted copies must match bit for bit; weighted combines and dot products are held to
+a relative Frobenius error of 1e-2 (and in practice match the oracle to rounding).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def ops():
+    import megablocks_amd.ops as ops
+    return ops
+
+
+@pytest.fixture(scope='module')
+def kernels():
+    from megablocks_amd.backend import kernels
+    return kernels
+
+
+def dev(t):
+    return None if t is None else t.cuda()
+
+
+def rel_err(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
+# ------------------------------------------------------------------ histogram
+@pytest.mark.parametrize('m,n', [(1, 32), (2, 32), (2, 1024), (16, 1024), (1, 16384), (3, 300000)])
+@pytest.mark.parametrize('dtype', [torch.int16, torch.int32, torch.int64])
+@pytest.mark.parametrize('max_val', [2, 8, 64, 128, 1000, 20000])
+def test_histogram(ops, m, n, dtype, max_val):
+    hi = min(max_val, 32000) if dtype == torch.int16 else max_val
+    x = torch.randint(0, hi, (m, n)).to(dtype)
+    got = ops.histogram(dev(x), max_val)
+    assert got.dtype == torch.int32 and torch.equal(got.cpu(), oracle.histogram(x, max_val))
+    got1 = ops.histogram(dev(x[0]), max_val)
+    assert got1.shape == (max_val,) and torch.equal(got1.cpu(), oracle.histogram(x[0], max_val))
+
+
+def test_histogram_ignores_out_of_range_and_empty(ops):
+    x = torch.tensor([-1, 0, 3, 4, 7, 7, 100], dtype=torch.int32)
+    assert ops.histogram(dev(x), 4).tolist() == [1, 0, 0, 1]
+    assert ops.histogram(torch.empty(0, dtype=torch.int32).cuda(), 5).tolist() == [0] * 5
+    assert ops.histogram(dev(x), 0).numel() == 0
+    with pytest.raises(RuntimeError):
+        ops.histogram(x.float().cuda(), 4)
+
+
+# ------------------------------------------------------------------ sort
+SORT_CASES = [(n, dt, mv) for n in (1, 7, 64, 2048, 2049, 16384, 200000)
+              for dt in (torch.int16, torch.int32, torch.int64) for mv in (None, 2, 8, 128, 1024)]
+
+
+@pytest.mark.parametrize('n,dtype,max_val', SORT_CASES)
+def test_sort(ops, n, dtype, max_val):
+    if dtype == torch.int16 and n > 32767:
+        pytest.skip('an int16 payload cannot index this many elements')
+    info = torch.iinfo(dtype)
+    if max_val is None:
+        x = torch.randint(info.min // 2, info.max // 2, (n,), dtype=torch.int64).to(dtype)
+        end_bit = None
+    else:
+        x = torch.randint(0, max_val, (n,), dtype=torch.int64).to(dtype)
+        end_bit = max(int(np.ceil(np.log2(max_val))), 1)
+    keys, perm = ops.sort(dev(x), end_bit)
+    want_keys, want_perm = oracle.sort(x, end_bit)
+    assert keys.dtype == dtype and perm.dtype == dtype
+    assert torch.equal(keys.cpu(), want_keys)
+    assert torch.equal(perm.cpu(), want_perm)       # stable: ties in ascending original position
+
+
+def test_sort_end_bit_ignores_high_bits(ops):
+    x = torch.randint(0, 1 << 20, (5000,)).int()
+    keys, perm = ops.sort(dev(x), 5)
+    wk, wp = oracle.sort(x, 5)
+    assert torch.equal(keys.cpu(), wk) and torch.equal(perm.cpu(), wp)
+    k0, p0 = ops.sort(dev(x), 0)
+    assert torch.equal(k0.cpu(), x) and torch.equal(p0.cpu(), torch.arange(5000, dtype=torch.int32))
+    e = torch.empty(0, dtype=torch.int32).cuda()
+    assert ops.sort(e)[0].numel() == 0
+
+
+# ------------------------------------------------------------------ cumsum
+@pytest.mark.parametrize('m,n', [(1, 1), (1, 8), (3, 64), (2, 257), (16, 1024), (2, 5000)])
+@pytest.mark.parametrize('dtype', [torch.int16, torch.int32, torch.int64])
+def test_cumsum(ops, m, n, dtype):
+    x = torch.randint(0, 3, (m, n)).to(dtype)
+    assert torch.equal(ops.inclusive_cumsum(dev(x), 1).cpu(), oracle.inclusive_cumsum(x, 1))
+    assert torch.equal(ops.exclusive_cumsum(dev(x), 1).cpu(), oracle.exclusive_cumsum(x, 1))
+    got = ops.inclusive_cumsum(dev(x[0]), 0)
+    want = oracle.inclusive_cumsum(x[0], 0)
+    assert got.shape == want.shape and torch.equal(got.cpu(), want)   # [1] -> 0-dim, like the reference
+    with pytest.raises(RuntimeError):
+        ops.inclusive_cumsum(dev(x), 0)
+
+
+# ------------------------------------------------------------------ topology / replicate / round_up
+@pytest.mark.parametrize('sl,hs,ne', [(1024, 1536, 2), (1024, 1536, 16), (16384, 768, 64), (16384, 768, 128),
+                                      (8192, 4096, 512), (300, 256, 8)])
+def test_topology(ops, sl, hs, ne):
+    blocking = 128
+    top = torch.randint(0, ne, (sl,)).int()
+    tpe = oracle.histogram(top, ne)
+    pbins = oracle.inclusive_cumsum(oracle.round_up(tpe, blocking), 0).view(-1)
+    rows, cols = int(pbins[-1]) // blocking, hs // blocking
+    got = ops.topology(dev(pbins), blocking, rows, cols)
+    assert got.dtype == torch.int16 and torch.equal(got.cpu(), oracle.topology(pbins, blocking, rows, cols))
+    assert torch.equal(ops.round_up(dev(tpe), blocking).cpu(), oracle.round_up(tpe, blocking))
+
+
+@pytest.mark.parametrize('tokens,centers,top_k', [(8, 2, 1), (8, 2, 2), (64, 8, 4), (1024, 64, 2), (16384, 128, 8),
+                                                  (16384, 2, 1)])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.int16, torch.int32])
+def test_replicate(ops, tokens, centers, top_k, dtype):
+    assign = torch.randint(0, centers, (tokens,)).int()
+    tpe = oracle.histogram(assign, centers)
+    bins = oracle.inclusive_cumsum(tpe, 0).view(-1)
+    x = torch.randn(top_k, centers).half() if dtype == torch.float16 else torch.randint(-99, 99, (top_k, centers)).to(dtype)
+    got = ops.replicate(dev(x), dev(bins), tokens)
+    assert torch.equal(got.cpu(), oracle.replicate(x, bins, tokens))
+    if dtype == torch.float16:
+        from megablocks_amd.ops.routing import replicate_backward
+        out = torch.empty_like(x).cuda()
+        replicate_backward(got, dev(bins), out)
+        want = x.float() * tpe.view(1, -1)
+        assert torch.allclose(out.float().cpu(), want, rtol=1e-2, atol=1e-2)   # replicate_test.py:108
+        xg = dev(x).requires_grad_(True)
+        ops.replicate(xg, dev(bins), tokens).backward(torch.ones(top_k, tokens, dtype=dtype).cuda())
+        assert torch.allclose(xg.grad.float().cpu(), tpe.float().expand(top_k, -1), rtol=1e-2)
+
+
+# ------------------------------------------------------------------ gather / scatter
+PERMUTE_CASES = [(4, 2, 2, 1), (4, 2, 2, 2), (1024, 1, 4, 1), (1024, 1, 64, 4), (1024, 1536, 4, 1), (1024, 1536, 64, 2),
+                 (1024, 1536, 128, 4), (16384, 768, 4, 1), (16384, 768, 64, 2), (16384, 768, 128, 4), (16384, 1, 128, 2),
+                 (2048, 4096, 8, 2), (777, 100, 5, 3)]
+
+
+def _routing(sl, ne, top_k, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    top = torch.randint(0, ne, (sl * top_k,), generator=g).int()
+    bin_ids, indices = oracle.sort(top, max(int(np.ceil(np.log2(ne))), 1))
+    tpe = oracle.histogram(top, ne)
+    bins = oracle.inclusive_cumsum(tpe, 0).view(-1)
+    pbins = oracle.inclusive_cumsum(oracle.round_up(tpe, 128), 0).view(-1)
+    return indices, bin_ids, bins, pbins
+
+
+@pytest.mark.parametrize('sl,hs,ne,top_k', PERMUTE_CASES)
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+def test_gather_and_padded_gather(kernels, sl, hs, ne, top_k, dtype):
+    indices, bin_ids, bins, pbins = _routing(sl, ne, top_k)
+    x = torch.randn(sl, hs).to(dtype)
+    w = torch.rand(sl * top_k).to(dtype)
+    args = [dev(t) for t in (indices, bin_ids)]
+    got = kernels.gather(dev(x), *args, None, dev(bins), top_k)
+    assert torch.equal(got.cpu(), oracle.gather(x, indices, bin_ids, None, bins, top_k))
+    got = kernels.padded_gather(dev(x), *args, None, dev(bins), dev(pbins), top_k)
+    assert torch.equal(got.cpu(), oracle.padded_gather(x, indices, bin_ids, None, bins, pbins, top_k))
+    got = kernels.gather(dev(x), *args, dev(w), dev(bins), top_k)
+    assert torch.equal(got.cpu(), oracle.gather(x, indices, bin_ids, w, bins, top_k))   # one rounding, same as oracle
+    got = kernels.padded_gather(dev(x), *args, dev(w), dev(bins), dev(pbins), top_k)
+    assert torch.equal(got.cpu(), oracle.padded_gather(x, indices, bin_ids, w, bins, pbins, top_k))
+
+
+@pytest.mark.parametrize('sl,hs,ne,top_k', PERMUTE_CASES)
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+def test_scatter_and_padded_scatter(kernels, sl, hs, ne, top_k, dtype):
+    indices, bin_ids, bins, pbins = _routing(sl, ne, top_k, seed=1)
+    xt = torch.randn(sl, hs).to(dtype)
+    w = torch.rand(sl * top_k).to(dtype)
+    args = [dev(t) for t in (indices, bin_ids)]
+    x = oracle.gather(xt, indices, bin_ids, None, bins, top_k)
+    xp = oracle.padded_gather(xt, indices, bin_ids, None, bins, pbins, top_k)
+    for weights in (None, w):
+        got = kernels.scatter(dev(x), *args, dev(weights), dev(bins), top_k)
+        want = oracle.scatter(x, indices, bin_ids, weights, bins, top_k)
+        got_p = kernels.padded_scatter(dev(xp), *args, dev(weights), dev(bins), dev(pbins), top_k)
+        want_p = oracle.padded_scatter(xp, indices, bin_ids, weights, bins, pbins, top_k)
+        if top_k <= 2:          # one rounding per product and at most one add: bit-exact
+            assert torch.equal(got.cpu(), want) and torch.equal(got_p.cpu(), want_p)
+        else:                   # fp32 sum order over top_k may differ from torch's reduction
+            assert rel_err(got, want) < 1e-2 and rel_err(got_p, want_p) < 1e-2
+            assert torch.allclose(got.float().cpu(), want.float(), rtol=5e-3, atol=5e-3)
+    if top_k == 1:              # unweighted round trip is the identity, bit for bit
+        back = kernels.scatter(kernels.gather(dev(xt), *args, None, dev(bins), 1), *args, None, dev(bins), 1)
+        assert torch.equal(back.cpu(), xt)
+
+
+@pytest.mark.parametrize('sl,hs,ne,top_k', PERMUTE_CASES)
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+def test_scatter_wgrad(kernels, sl, hs, ne, top_k, dtype):
+    indices, bin_ids, bins, pbins = _routing(sl, ne, top_k, seed=2)
+    xt = torch.randn(sl, hs).to(dtype)
+    grad = torch.randn(sl, hs).to(dtype)
+    args = [dev(t) for t in (indices, bin_ids)]
+    x = oracle.gather(xt, indices, bin_ids, None, bins, top_k)
+    xp = oracle.padded_gather(xt, indices, bin_ids, None, bins, pbins, top_k)
+    got = kernels.scatter_wgrad(dev(x), dev(grad), *args, dev(bins), top_k)
+    want = oracle.scatter_wgrad(x, grad, indices, bin_ids, bins, top_k)
+    assert rel_err(got, want) < 1e-2
+    got = kernels.padded_scatter_wgrad(dev(xp), dev(grad), *args, dev(bins), dev(pbins), top_k)
+    want = oracle.padded_scatter_wgrad(xp, grad, indices, bin_ids, bins, pbins, top_k)
+    assert rel_err(got, want) < 1e-2
+
+
+@pytest.mark.parametrize('sl,hs,ne,top_k', [(4, 2, 2, 1), (1024, 1536, 4, 2), (1024, 1536, 64, 4), (16384, 768, 128, 1),
+                                            (16384, 768, 4, 4), (1000, 50, 7, 2)])
+@pytest.mark.parametrize('cap_factor', [0.5, 1.0, 2.0])
+def test_binned_ops(kernels, sl, hs, ne, top_k, cap_factor):
+    dtype = torch.float16
+    indices, bin_ids, bins, pbins = _routing(sl, ne, top_k, seed=3)
+    cap = max(int(cap_factor * sl * top_k / ne), 1)
+    xt = torch.randn(sl, hs).to(dtype)
+    w = torch.rand(sl * top_k).to(dtype)
+    grad = torch.randn(sl, hs).to(dtype)
+    got = kernels.binned_gather(dev(xt), dev(indices), None, dev(bins), cap, top_k)
+    want = oracle.binned_gather(xt, indices, None, bins, cap, top_k)
+    assert torch.equal(got.cpu(), want)
+    got_w = kernels.binned_gather(dev(xt), dev(indices), dev(w), dev(bins), cap, top_k)
+    assert torch.equal(got_w.cpu(), oracle.binned_gather(xt, indices, w, bins, cap, top_k))
+    sc = kernels.binned_scatter(got, dev(indices), dev(w), dev(bins), top_k)
+    want_sc = oracle.binned_scatter(want, indices, w, bins, top_k)
+    assert rel_err(sc, want_sc) < 1e-2 and torch.allclose(sc.float().cpu(), want_sc.float(), rtol=5e-3, atol=5e-3)
+    wg = kernels.binned_scatter_wgrad(got, dev(grad), dev(indices), dev(bins), top_k)
+    assert rel_err(wg, oracle.binned_scatter_wgrad(want, grad, indices, bins, top_k)) < 1e-2
+
+
+def test_shape_errors_are_value_errors(kernels):
+    x = torch.randn(4, 8).cuda()
+    idx = torch.zeros(4, dtype=torch.int32).cuda()
+    bins = torch.tensor([4], dtype=torch.int32).cuda()
+    with pytest.raises(ValueError):
+        kernels.gather(x.view(-1), idx, idx, None, bins, 1)          # not a matrix
+    with pytest.raises(ValueError):
+        kernels.gather(x, idx[:3], idx, None, bins, 1)                # tokens * top_k mismatch
+    with pytest.raises(ValueError):
+        kernels.padded_gather(x, idx, idx, None, bins, torch.cat([bins, bins]), 1)
+    with pytest.raises(ValueError):
+        kernels.binned_scatter(x, idx, None, bins, 1)                 # needs a 3-tensor
+
+
+# ------------------------------------------------------------------ autograd pairing
+def test_autograd_pairing_matches_oracle_autograd(ops):
+    sl, hs, ne, top_k = 512, 256, 8, 2
+    indices, bin_ids, bins, pbins = _routing(sl, ne, top_k, seed=4)
+    x = torch.randn(sl, hs)
+    w = torch.rand(sl * top_k)
+    gout = torch.randn(sl, hs)
+    # oracle: differentiable formulation on the CPU in fp32
+    xo, wo = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    tok = indices.long() // top_k
+    y = xo.index_select(0, tok) * 2.0
+    out = torch.zeros(sl, hs).index_add(0, tok, y * wo[indices.long()].unsqueeze(1))
+    out.backward(gout)
+    for padded in (False, True):
+        xg, wg = dev(x).requires_grad_(True), dev(w).requires_grad_(True)
+        i, b, bn, pb = dev(indices), dev(bin_ids), dev(bins), dev(pbins)
+        if padded:
+            yg = ops.padded_gather(xg, i, b, bn, pb, top_k) * 2.0
+            og = ops.padded_scatter(yg, i, b, wg, bn, pb, top_k)
+        else:
+            yg = ops.gather(xg, i, b, bn, top_k) * 2.0
+            og = ops.scatter(yg, i, b, wg, bn, top_k)
+        og.backward(dev(gout))
+        assert rel_err(og, out) < 1e-5 and rel_err(xg.grad, xo.grad) < 1e-5 and rel_err(wg.grad, wo.grad) < 1e-5
+
+
+def test_full_size_round_trip_properties(ops):
+    # Mixtral-shaped permutation at full size, checked through size-independent properties
+    T, h, E, k = 8192, 4096, 8, 2
+    x = torch.randn(T, h, device='cuda').bfloat16()
+    top = torch.randint(0, E, (T * k,), device='cuda').int()
+    bin_ids, indices = ops.sort(top, 3)
+    tpe = ops.histogram(top, E)
+    bins = ops.inclusive_cumsum(tpe, 0)
+    assert int(tpe.sum()) == T * k and int(bins[-1]) == T * k
+    assert bool((bin_ids[1:] >= bin_ids[:-1]).all())                               # sortedness
+    assert torch.equal(torch.sort(indices.long())[0], torch.arange(T * k, device='cuda'))  # a permutation
+    assert torch.equal(top[indices.long()], bin_ids)
+    g = ops.gather(x, indices, bin_ids, bins, k)
+    assert torch.equal(g, x[indices.long() // k])                                  # bit-exact copy
+    half = torch.full((T * k,), 0.5, device='cuda').bfloat16()
+    back = ops.scatter(g, indices, bin_ids, half, bins, k)                         # 0.5 x + 0.5 x == x exactly
+    assert torch.equal(back, x)
