@@ -1,0 +1,231 @@
+#!/usr/bin/env python3
+"""Benchmark of the dropless-MoE layer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--no-cpu]
+
+A step is one forward+backward of the dMoE layer on a batch of synthetic tokens that is
+already resident in HBM.  Prints ONE JSON line: whole-job tokens/s, the grouped-GEMM roofline
+(algorithmic FLOPs / live HIP-event kernel time vs the bf16 dense MFMA peak), per-kernel
+figures for the permutation kernels (algorithmic bytes / kernel time vs the HBM peak), and the
+CPU formulation of the same path timed on this host's cores as a baseline.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_PEAK = {'bf16': 2.5e15, 'f16': 2.5e15, 'f32': 157.3e12}
+HBM_PEAK = 8e12
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
+# keyed by (workload, kernel); None until measured for the workload at hand.
+MEASURED_TRAFFIC = {}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--config', default='c3', choices=['c1', 'c2', 'c3', 'c4', 'c5'])
+    ap.add_argument('--tokens', type=int, default=None, help='override the token count (not the headline number)')
+    ap.add_argument('--memory-optimized', action='store_true')
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
+    ap.add_argument('--cpu-tokens', type=int, default=None)
+    return ap.parse_args()
+
+
+def dtype_name(dt):
+    import torch
+    return {torch.bfloat16: 'bf16', torch.float16: 'f16', torch.float32: 'f32'}[dt]
+
+
+def gpu_leg(args, w, inp):
+    import torch
+
+    from megablocks_amd import _lib, synthetic
+
+    dev = torch.device('cuda', 0)
+    torch.cuda.set_device(dev)
+    layer = synthetic.build_layer(w, inp, device=dev, memory_optimized=args.memory_optimized)
+    x = inp['x'].to(w.dtype).to(dev).requires_grad_(True)
+    grad = inp['grad'].to(w.dtype).to(dev)
+    routing = None
+    if w.routing != 'router':
+        ew = inp['expert_weights'].to(w.dtype).to(dev).requires_grad_(True)
+        routing = (inp['scores'].to(w.dtype).to(dev), ew, inp['top_experts'].to(dev))
+
+    def step():
+        x.grad = None
+        if routing is not None:
+            routing[1].grad = None
+        for p in layer.parameters():
+            p.grad = None
+        synthetic.layer_step(layer, w, x, grad, routing)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    ms_wall = wall * 1e3 / args.steps
+
+    # second pass with HIP events around every grouped-GEMM / permutation launch
+    _lib.profile_hook = []
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    records, _lib.profile_hook = _lib.profile_hook, None
+    agg = {}
+    for name, meta, a, b in records:
+        d = agg.setdefault(name, dict(ms=[], meta=meta))
+        d['ms'].append(a.elapsed_time(b))
+    return ms_per_step, ms_wall, agg, layer
+
+
+def summarize(w, agg, slots_scale):
+    """Per-kernel algorithmic work / measured time.  `slots_scale` = real slots / rows handed to the
+    kernels (< 1 only in block-sparse mode, whose groups are padded to 128 rows)."""
+    dn = dtype_name(w.dtype)
+    gemm, perm = {}, {}
+    for name, d in agg.items():
+        m = d['meta']
+        avg_ms = statistics.fmean(d['ms'])
+        launches = len(d['ms'])
+        if name.startswith('gmm'):
+            flops = 2.0 * m['rows'] * slots_scale * m['k'] * m['n']
+            gemm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, flops_per_launch=flops,
+                              tflops=round(flops / (avg_ms * 1e-3) / 1e12, 1),
+                              frac_of_mfma_peak=round(flops / (avg_ms * 1e-3) / MFMA_PEAK[dn], 4))
+        else:
+            nbytes = float(w.tokens + w.slots) * m['hidden'] * m['elem']
+            perm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, bytes_per_launch=nbytes,
+                              gbps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
+                              frac_of_hbm_peak=round(nbytes / (avg_ms * 1e-3) / HBM_PEAK, 4))
+    return gemm, perm
+
+
+def cpu_leg(args, w, inp_full):
+    """The CPU formulation (oracle) of the same layer, fp32, forward+backward, on a bounded sample."""
+    import torch
+
+    import oracle
+    from megablocks_amd import synthetic
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    # aim at roughly 10-30 s of CPU work: scale the token count to about 2e12 FLOP per step
+    if args.cpu_tokens:
+        T = args.cpu_tokens
+    else:
+        per_token = w.gemm_flops() / w.tokens
+        T = int(min(w.tokens, max(256, 2.0e12 // per_token)))
+    inp = inp_full if T == w.tokens else synthetic.make_inputs(w, tokens=T, seed=0)
+    act = w.activation()
+
+    def step():
+        x = inp['x'].clone().requires_grad_(True)
+        rw = inp['router_weight'].clone().requires_grad_(True)
+        w1, w2 = inp['w1'].requires_grad_(True), inp['w2'].requires_grad_(True)
+        v1 = None if inp['v1'] is None else inp['v1'].requires_grad_(True)
+        for p in (w1, w2, v1):
+            if p is not None:
+                p.grad = None
+        if w.routing == 'router':
+            _, ew, te = oracle.router_forward(x, rw, w.top_k, w.normalize)
+        else:
+            ew, te = inp['expert_weights'].clone().requires_grad_(True), inp['top_experts']
+        out, _ = oracle.dmoe_forward(x, ew, te, w1, w2, v1, num_experts=w.experts, top_k=w.top_k, activation=act)
+        out.backward(inp['grad'])
+
+    step()  # warm-up
+    times = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    return dict(value=round(T / t, 1), unit='tokens/s', cores=cores, kind='port',
+                sample=f'{T} of {w.tokens} tokens of workload {w.name}, fp32, fwd+bwd, 1 warm-up + 2 timed steps '
+                       f'(median {t:.2f} s), torch {torch.get_num_threads()} threads',
+                seconds_per_step=round(t, 3))
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f'bench.py: this build runs on one GPU holding all experts; --gpus {args.gpus} is not supported '
+              '(the expert-parallel all-to-all is out of scope).', file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from megablocks_amd import synthetic
+
+    w = synthetic.WORKLOADS[args.config]
+    if args.tokens:
+        import dataclasses
+        w = dataclasses.replace(w, tokens=args.tokens)
+    inp = synthetic.make_inputs(w, seed=0)
+    ms_per_step, ms_wall, agg, layer = gpu_leg(args, w, inp)
+
+    slots_scale = 1.0
+    if w.mlp_impl == 'sparse':
+        # every gmm record carries the padded row count the kernels were handed
+        any_gmm = next(d for n, d in agg.items() if n.startswith('gmm'))
+        slots_scale = w.slots / float(any_gmm['meta']['rows'])
+    gemm, perm = summarize(w, agg, slots_scale)
+
+    dn = dtype_name(w.dtype)
+    gemm_ms = sum(g['avg_ms'] * g['launches'] for g in gemm.values()) / args.steps
+    perm_ms = sum(p['avg_ms'] * p['launches'] for p in perm.values()) / args.steps
+    dom_name, dom = max(gemm.items(), key=lambda kv: kv[1]['avg_ms'] * kv[1]['launches'])
+    roofline = dict(bound='mfma', kernel=dom_name, achieved=dom['tflops'], peak=MFMA_PEAK[dn] / 1e12, unit='TFLOP/s',
+                    frac=dom['frac_of_mfma_peak'], traffic=MEASURED_TRAFFIC.get((w.name, dom_name)),
+                    flops_per_launch=dom['flops_per_launch'], avg_launch_ms=dom['avg_ms'])
+    all_gemm_tflops = w.gemm_flops() / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None
+
+    out = {
+        'metric': 'dmoe_layer_fwd_bwd_tokens_per_s',
+        'value': round(w.tokens / (ms_per_step * 1e-3), 1),
+        'unit': 'tokens/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': round(ms_per_step, 4),
+        'ms_per_step_wall': round(ms_wall, 4),
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': dn,
+        'data': 'synthetic',
+        'config': {'workload': f'{w.name}: {w.description}', 'tokens': w.tokens, 'hidden': w.hidden, 'ffn': w.ffn,
+                   'experts': w.experts, 'top_k': w.top_k, 'mlp_type': w.mlp_type, 'mlp_impl': w.mlp_impl,
+                   'routing': w.routing, 'memory_optimized_mlp': args.memory_optimized},
+        'roofline': roofline,
+        'gemm': {'ms_per_step': round(gemm_ms, 4), 'tflops_all_launches': round(all_gemm_tflops, 1),
+                 'frac_of_mfma_peak': round(all_gemm_tflops * 1e12 / MFMA_PEAK[dn], 4), 'kernels': gemm},
+        'permute': {'ms_per_step': round(perm_ms, 4), 'kernels': perm},
+    }
+    if not args.no_cpu:
+        del layer
+        torch.cuda.empty_cache()
+        out['cpu_baseline'] = cpu_leg(args, w, inp)
+    else:
+        out['cpu_baseline'] = None
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

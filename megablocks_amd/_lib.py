@@ -96,3 +96,30 @@ def as_i32(t):
     if t.dtype != torch.int32:
         t = t.to(torch.int32)
     return t.contiguous()
+
+
+# ---- optional per-launch timing (used by bench.py; off by default) -----------------------
+# When `profile_hook` is a list, every operator appends (name, meta, start_event, end_event)
+# for each launch, the events recorded on the stream the kernel was enqueued on.
+profile_hook = None
+
+
+class record:
+    """`with record('gmm_nt', rows=..., k=..., n=...):` around a launch."""
+    __slots__ = ('name', 'meta', 'ev0')
+
+    def __init__(self, name, **meta):
+        self.name, self.meta, self.ev0 = name, meta, None
+
+    def __enter__(self):
+        if profile_hook is not None:
+            self.ev0 = torch.cuda.Event(enable_timing=True)
+            self.ev0.record()
+        return self
+
+    def __exit__(self, *exc):
+        if self.ev0 is not None:
+            ev1 = torch.cuda.Event(enable_timing=True)
+            ev1.record()
+            profile_hook.append((self.name, self.meta, self.ev0, ev1))
+        return False

@@ -47,7 +47,9 @@ def _gather(x, indices, bin_ids, weights, bins, padded_bins, top_k, output_rows,
     indices, bins, padded_bins = _lib.as_i32(indices), _lib.as_i32(bins), _lib.as_i32(padded_bins)
     wp, wdt, weights = _w(weights)
     out = torch.empty((output_rows, x.shape[1]), dtype=x.dtype, device=x.device)
-    with torch.cuda.device_of(x):
+    with torch.cuda.device_of(x), _lib.record('gather_weighted' if weights is not None else 'gather',
+                                              rows_in=x.shape[0], rows_out=output_rows, hidden=x.shape[1],
+                                              elem=x.element_size()):
         _lib.check(lib.mbx_gather(_lib.ptr(x), _lib.dtype_of(x), x.shape[0], x.shape[1], top_k, _lib.ptr(indices),
                                   _lib.ptr(bins), _lib.ptr(padded_bins), bins.shape[0], wp, wdt, _lib.ptr(out),
                                   output_rows, _lib.stream()), what)
@@ -123,7 +125,9 @@ def _scatter(x, indices, bin_ids, weights, bins, padded_bins, top_k):
     wp, wdt, weights = _w(weights)
     out = torch.empty((tokens, x.shape[1]), dtype=x.dtype, device=x.device)
     scratch = _scratch(n_slots, x.device)
-    with torch.cuda.device_of(x):
+    with torch.cuda.device_of(x), _lib.record('scatter_weighted' if weights is not None else 'scatter',
+                                              rows_in=n_slots, rows_out=tokens, hidden=x.shape[1],
+                                              elem=x.element_size()):
         _lib.check(lib.mbx_scatter(_lib.ptr(x), _lib.dtype_of(x), tokens, x.shape[1], top_k, _lib.ptr(indices),
                                    _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins), bins.shape[0], wp, wdt,
                                    _lib.ptr(out), _lib.ptr(scratch), scratch.numel() * 4, _lib.stream()), 'scatter')
@@ -165,7 +169,8 @@ def _scatter_wgrad(x, grad, indices, bin_ids, bins, padded_bins, top_k):
     indices, bin_ids = _lib.as_i32(indices), _lib.as_i32(bin_ids)
     bins, padded_bins = _lib.as_i32(bins), _lib.as_i32(padded_bins)
     out = torch.empty((n_slots,), dtype=x.dtype, device=x.device)
-    with torch.cuda.device_of(x):
+    with torch.cuda.device_of(x), _lib.record('scatter_wgrad', rows_in=n_slots, rows_out=tokens, hidden=x.shape[1],
+                                              elem=x.element_size()):
         _lib.check(lib.mbx_scatter_wgrad(_lib.ptr(x), _lib.ptr(grad), _lib.dtype_of(x), tokens, x.shape[1], top_k,
                                          _lib.ptr(indices), _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins),
                                          bins.shape[0], _lib.ptr(out), _lib.stream()), 'scatter_wgrad')

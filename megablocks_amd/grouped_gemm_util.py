@@ -81,7 +81,8 @@ def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None):
     else:
         if tuple(c.shape) != shape or c.dtype != a.dtype or not c.is_contiguous():
             raise ValueError('gmm: c has the wrong shape, dtype or layout')
-    with torch.cuda.device_of(a):
+    with torch.cuda.device_of(a), _lib.record(('gmm_nn', 'gmm_nt', 'gmm_tn')[layout], rows=rows, k=k, n=n,
+                                              elem=a.element_size(), groups=groups):
         _lib.check(lib.mbx_gmm(_lib.ptr(a), _lib.ptr(b), _lib.ptr(c), dt, _lib.ptr(bins), groups, rows, k, n, layout,
                                _lib.stream()), 'gmm')
     return c
