@@ -65,22 +65,34 @@ struct Stager {
   static constexpr int CH = CHUNKS / THREADS;
   static_assert(CHUNKS % THREADS == 0, "tile must split evenly over the threads");
 
-  static __device__ __forceinline__ void load(const Operand& op, int k0, int k_end, u32x4 (&reg)[CH]) {
+  // Always loads from an in-bounds (clamped) address and zeroes what lies outside the operand, so
+  // the loop body has no branches: the loads of the tile after the last one are redundant, not wild.
+  static __device__ __forceinline__ void load(const Operand& op, int k0, int k_begin, int k_end, u32x4 (&reg)[CH]) {
     const int tid = threadIdx.x;
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int c = tid + i * THREADS;
-      u32x4 v = {0u, 0u, 0u, 0u};
+      const u32x4 zero = {0u, 0u, 0u, 0u};
       if (!MC) {
         const int r = c / (BK / 8), kc = (c % (BK / 8)) * 8;
         int row = op.r0 + r;
         if (row > op.r_lim - 1) row = op.r_lim - 1;
-        if (k0 + kc < k_end) v = *(const u32x4*)(op.base + (int64_t)row * op.ld + (k0 + kc));
+        int kk = k0 + kc;
+        const bool ok = kk < k_end;
+        if (kk > k_end - 8) kk = k_end - 8;
+        if (kk < k_begin) kk = k_begin;
+        const u32x4 v = *(const u32x4*)(op.base + (int64_t)row * op.ld + kk);
+        reg[i] = ok ? v : zero;
       } else {
-        const int kk = c / (R / 8), rc = (c % (R / 8)) * 8;
-        if (k0 + kk < k_end && op.r0 + rc < op.r_lim) v = *(const u32x4*)(op.base + (int64_t)(k0 + kk) * op.ld + (op.r0 + rc));
+        const int kr = c / (R / 8), rc = (c % (R / 8)) * 8;
+        int kk = k0 + kr, col = op.r0 + rc;
+        const bool ok = kk < k_end && col < op.r_lim;
+        if (kk > k_end - 1) kk = k_end - 1;
+        if (kk < k_begin) kk = k_begin;
+        if (col > op.r_lim - 8) col = op.r_lim - 8;
+        const u32x4 v = *(const u32x4*)(op.base + (int64_t)kk * op.ld + col);
+        reg[i] = ok ? v : zero;
       }
-      reg[i] = v;
     }
   }
 
@@ -120,10 +132,15 @@ __device__ __forceinline__ u32x4 read_frag(const uint16_t* lds, int r, int ks) {
   }
 }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
-  if (DT == MBX_BF16) return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
-  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)a) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)b) << 16);
+  const f32x2_t v = {a, b};
+  if (DT == MBX_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));  // v_cvt_pk_bf16_f32, RNE
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
 }
 
 // The workgroup-level product: acc += A_tile(k) * B_tile(k) over k in [k_begin, k_end),
@@ -149,41 +166,65 @@ __device__ __forceinline__ void block_gemm(const Operand& opa, const Operand& op
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int nk = (k_end - k_begin + T::BK - 1) / T::BK;
+  constexpr int KS = T::BK / 16;
+  static_assert(KS % 2 == 0, "the operand double buffer assumes an even number of k-steps per tile");
   u32x4 ra[SA::CH], rb[SB::CH];
+  u32x4 fa[2][T::TM], fb[2][T::TN];   // MFMA operands, double buffered across k-steps
+
+  auto read_frags = [&](const uint16_t* stage, int ks, int buf) {
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i) fa[buf][i] = read_frag<A_MC, LA::STRIDE>(stage, wm + i * 32, ks);
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) fb[buf][j] = read_frag<B_MC, LB::STRIDE>(stage + LA::ELEMS, wn + j * 32, ks);
+  };
+  // operands swapped: the accumulator tile is c^T, so a lane owns runs of four consecutive
+  // columns of one row of c and can store them as one 8-byte word.
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) {
+#ifndef MBX_TUNE_NO_MFMA
+        acc[i][j] = mfma32<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
+#else
+        acc[i][j][0] += __uint_as_float(fb[buf][j][0] ^ fa[buf][i][0]);
+#endif
+      }
+  };
+
   if (nk > 0) {
-    SA::load(opa, k_begin, k_end, ra);
-    SB::load(opb, k_begin, k_end, rb);
+    SA::load(opa, k_begin, k_begin, k_end, ra);
+    SB::load(opb, k_begin, k_begin, k_end, rb);
     SA::template store<LA::STRIDE>(lds, ra);
     SB::template store<LB::STRIDE>(lds + LA::ELEMS, rb);
+    __syncthreads();
+    read_frags(lds, 0, 0);
   }
-  __syncthreads();
+  // Per K tile: the global loads of the next tile are issued first and land in registers while
+  // k-steps 0..KS-2 run; each k-step first issues the LDS reads of the following k-step, then
+  // its MFMAs.  Before the last k-step the staged tile goes to the other LDS buffer, the
+  // workgroup synchronises, and the first operands of the next tile are read, so that the
+  // barrier and the LDS latency are covered by the MFMAs of the last k-step.
   for (int kt = 0; kt < nk; ++kt) {
     uint16_t* cur = lds + (kt & 1) * STAGE;
     uint16_t* nxt = lds + ((kt + 1) & 1) * STAGE;
-    const bool more = kt + 1 < nk;
-    if (more) {
-      SA::load(opa, k_begin + (kt + 1) * T::BK, k_end, ra);
-      SB::load(opb, k_begin + (kt + 1) * T::BK, k_end, rb);
+#ifndef MBX_TUNE_NO_GLOBAL
+    SA::load(opa, k_begin + (kt + 1) * T::BK, k_begin, k_end, ra);
+    SB::load(opb, k_begin + (kt + 1) * T::BK, k_begin, k_end, rb);
+#endif
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KS - 1; ++ks) {
+      read_frags(cur, ks + 1, (ks + 1) & 1);
+      multiply(ks & 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int ks = 0; ks < T::BK / 16; ++ks) {
-      u32x4 fa[T::TM], fb[T::TN];
-#pragma unroll
-      for (int i = 0; i < T::TM; ++i) fa[i] = read_frag<A_MC, LA::STRIDE>(cur, wm + i * 32, ks);
-#pragma unroll
-      for (int j = 0; j < T::TN; ++j) fb[j] = read_frag<B_MC, LB::STRIDE>(cur + LA::ELEMS, wn + j * 32, ks);
-      // operands swapped: the accumulator tile is c^T, so a lane owns runs of four
-      // consecutive columns of one row of c and can store them as one 8-byte word.
-#pragma unroll
-      for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j) acc[i][j] = mfma32<DT>(fb[j], fa[i], acc[i][j]);
-    }
-    if (more) {
-      SA::template store<LA::STRIDE>(nxt, ra);
-      SB::template store<LB::STRIDE>(nxt + LA::ELEMS, rb);
-    }
+    SA::template store<LA::STRIDE>(nxt, ra);
+    SB::template store<LB::STRIDE>(nxt + LA::ELEMS, rb);
     __syncthreads();
+    read_frags(nxt, 0, KS & 1);
+    multiply((KS - 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // accumulator (i, j), register r of lane l holds c[m][n] with
@@ -215,15 +256,31 @@ __device__ __forceinline__ void block_gemm(const Operand& opa, const Operand& op
   }
 }
 
+// Workgroups are dispatched to the 8 XCDs round-robin by workgroup id, and every XCD has its own
+// L2.  The logical tile order is cut into runs of kXcdRun tiles and run r goes to XCD r % 8, so
+// the workgroups resident on one XCD at a time form a compact block of tiles (same expert, a few
+// row tiles x a few column tiles) whose operand panels are fetched into that L2 once.
+constexpr int kXcds = 8;
+constexpr int kXcdRun = 32;
+
+__device__ __forceinline__ int xcd_tile_id(int block) {
+  const int xcd = block % kXcds, l = block / kXcds;
+  return ((l / kXcdRun) * kXcds + xcd) * kXcdRun + (l % kXcdRun);
+}
+
+static inline int64_t xcd_grid(int64_t tiles) {
+  const int64_t q = (int64_t)kXcds * kXcdRun;
+  return (tiles + q - 1) / q * q;
+}
+
 // ---- NN / NT: row tiles follow the expert bins --------------------------------------
-// Linear workgroup id -> (expert, column tile, row tile inside the expert), row tiles
-// fastest, so that the workgroups in flight together share b[e] column panels.
+// Logical tile id -> (expert, column tile, row tile inside the expert), row tiles fastest.
 template <int DT, bool B_MC, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  int id = blockIdx.x;
+  int id = xcd_tile_id(blockIdx.x);
   int e = 0, start = 0, end = 0, mt = 0;
   for (; e < num_groups; ++e) {
     end = bins[e];
@@ -248,16 +305,22 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
 template <int DT, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
-              const int32_t* __restrict__ bins, int k, int n, int tiles_m, int tiles_n) {
+              const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  const int e = blockIdx.y;
-  const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+  const int id = xcd_tile_id(blockIdx.x);
+  const int per_group = tiles_m * tiles_n;
+  const int e = id / per_group;
+  if (e >= num_groups) return;
+  const int t = id % per_group;
+  const int tm = t % tiles_m, tn = t / tiles_m;
   const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
   Operand opa, opb;
   opa.base = a; opa.ld = k; opa.r0 = tm * T::BM; opa.r_lim = k;
   opb.base = b; opb.ld = n; opb.r0 = tn * T::BN; opb.r_lim = n;
   block_gemm<DT, true, true, T>(opa, opb, start, end, c + (int64_t)e * k * n, n, k, n, lds);
 }
+
+#include "gmm_dma.h"
 
 // ---- fallback for shapes the MFMA path does not take (odd sizes, fp32) ----------------
 // c(m, n) = sum_r a(m, r) b(r, n) with arbitrary element strides; 32x32 tile, fp32 FMA.
@@ -331,7 +394,8 @@ __global__ void gelu_backward_kernel(void* __restrict__ g_, const void* __restri
 
 // Tile shapes.  256x256x64 with four waves (2x2, 128x128 each) keeps the accumulators in
 // 256 registers per lane and needs 144 KiB of the 160 KiB LDS for two stages.
-typedef Tile<256, 256, 64, 2, 2, 8, 16> TileBig;
+typedef Tile<256, 256, 64, 4, 2, 8, 32> TileBig;
+typedef dma::Tile<256, 256, 2, 4> TileDma;
 
 template <int DT, bool A_MC, bool B_MC, typename T>
 constexpr size_t lds_bytes() {
@@ -344,10 +408,9 @@ int allow_lds(K kernel, size_t bytes) {
   return (int)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
-template <int DT>
+template <int DT, typename T>
 int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
              int layout, hipStream_t s) {
-  typedef TileBig T;
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
   uint16_t* cp = (uint16_t*)c;
@@ -357,12 +420,14 @@ int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num
     auto kern = gmm_tn_kernel<DT, T>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    kern<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)num_groups), T::THREADS, lds, s>>>(ap, bp, cp, bins, k, n, tiles_m, tiles_n);
+    const int64_t grid = xcd_grid((int64_t)tiles_m * tiles_n * num_groups);
+    if (grid > 0x7fffffff) return MBX_ERANGE;
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n);
     return launch_status();
   }
   const int tiles_n = (int)ceil_div(n, T::BN);
   const int64_t max_mt = ceil_div(rows, T::BM) + num_groups;
-  const int64_t grid = max_mt * tiles_n;
+  const int64_t grid = xcd_grid(max_mt * tiles_n);
   if (grid > 0x7fffffff) return MBX_ERANGE;
   if (layout == MBX_NT) {
     constexpr size_t lds = lds_bytes<DT, false, false, T>();
@@ -376,6 +441,41 @@ int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
     kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_n);
+  }
+  return launch_status();
+}
+
+// Launch of the direct-to-LDS kernels (k a multiple of 32 for NN / NT, operands below 2 GiB).
+template <int DT, typename T>
+int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
+            int layout, hipStream_t s) {
+  const uint16_t* ap = (const uint16_t*)a;
+  const uint16_t* bp = (const uint16_t*)b;
+  uint16_t* cp = (uint16_t*)c;
+  constexpr size_t lds = T::LDS_BYTES;
+  if (layout == MBX_TN) {
+    const int tiles_m = (int)ceil_div(k, T::BM), tiles_n = (int)ceil_div(n, T::BN);
+    auto kern = dma::gmm_tn_kernel<DT, T>;
+    int rc = allow_lds(kern, lds);
+    if (rc) return rc;
+    const int64_t grid = xcd_grid((int64_t)tiles_m * tiles_n * num_groups);
+    if (grid > 0x7fffffff) return MBX_ERANGE;
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n);
+    return launch_status();
+  }
+  const int tiles_n = (int)ceil_div(n, T::BN);
+  const int64_t grid = xcd_grid((ceil_div(rows, T::BM) + num_groups) * tiles_n);
+  if (grid > 0x7fffffff) return MBX_ERANGE;
+  if (layout == MBX_NT) {
+    auto kern = dma::gmm_rows_kernel<DT, false, T>;
+    int rc = allow_lds(kern, lds);
+    if (rc) return rc;
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
+  } else {
+    auto kern = dma::gmm_rows_kernel<DT, true, T>;
+    int rc = allow_lds(kern, lds);
+    if (rc) return rc;
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
   }
   return launch_status();
 }
@@ -424,8 +524,16 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
   if (layout == MBX_NN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (layout == MBX_TN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (fast) {
-    if (dtype == MBX_BF16) return gmm_mfma<MBX_BF16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-    return gmm_mfma<MBX_F16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+    // direct-to-LDS kernels: 32-wide K tiles (NN / NT) and 32-bit byte offsets inside each operand
+    const int64_t lim = (int64_t)1 << 31;
+    bool dma_ok = rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
+    if (layout != MBX_TN) dma_ok = dma_ok && k % dma::BK == 0;
+    if (dma_ok) {
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+      return gmm_dma<MBX_F16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+    }
+    if (dtype == MBX_BF16) return gmm_mfma<MBX_BF16, TileBig>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+    return gmm_mfma<MBX_F16, TileBig>(a, b, c, bins, num_groups, rows, k, n, layout, s);
   }
   switch (dtype) {
     case MBX_BF16: return gmm_generic<MBX_BF16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
