@@ -37,6 +37,8 @@ def parse():
     ap.add_argument('--memory-optimized', action='store_true')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
     ap.add_argument('--cpu-tokens', type=int, default=None)
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also launch one plain 1 GiB device copy (a known-size reference for HBM byte counters)')
     return ap.parse_args()
 
 
@@ -88,6 +90,12 @@ def gpu_leg(args, w, inp):
         step()
     torch.cuda.synchronize()
     records, _lib.profile_hook = _lib.profile_hook, None
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     agg = {}
     for name, meta, a, b in records:
         d = agg.setdefault(name, dict(ms=[], meta=meta))
