@@ -394,8 +394,8 @@ __global__ void gelu_backward_kernel(void* __restrict__ g_, const void* __restri
 
 // Tile shapes.  256x256x64 with four waves (2x2, 128x128 each) keeps the accumulators in
 // 256 registers per lane and needs 144 KiB of the 160 KiB LDS for two stages.
-typedef Tile<256, 256, 64, 4, 2, 8, 32> TileBig;
-typedef dma::Tile<256, 256, 2, 4> TileDma;
+typedef Tile<256, 256, 64, 2, 2, 8, 32> TileBig;
+typedef dma::Tile<256, 256, 2, 2, 64, 2> TileDma;
 
 template <int DT, bool A_MC, bool B_MC, typename T>
 constexpr size_t lds_bytes() {
@@ -458,7 +458,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     auto kern = dma::gmm_tn_kernel<DT, T>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    const int64_t grid = xcd_grid((int64_t)tiles_m * tiles_n * num_groups);
+    const int64_t grid = xcd_grid(dma::tn_tiles_per_group(tiles_m, tiles_n) * num_groups);
     if (grid > 0x7fffffff) return MBX_ERANGE;
     kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n);
     return launch_status();
@@ -524,10 +524,10 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
   if (layout == MBX_NN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (layout == MBX_TN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (fast) {
-    // direct-to-LDS kernels: 32-wide K tiles (NN / NT) and 32-bit byte offsets inside each operand
+    // direct-to-LDS kernels: whole K tiles (NN / NT) and 32-bit byte offsets inside each operand
     const int64_t lim = (int64_t)1 << 31;
     bool dma_ok = rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
-    if (layout != MBX_TN) dma_ok = dma_ok && k % dma::BK == 0;
+    if (layout != MBX_TN) dma_ok = dma_ok && k % TileDma::BK == 0;
     if (dma_ok) {
       if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);
       return gmm_dma<MBX_F16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);

@@ -1,19 +1,21 @@
-// Grouped-GEMM main loop with direct-to-LDS global loads and a four-stage LDS ring.
+// Grouped-GEMM main loop with direct-to-LDS global loads and an LDS ring of K tiles.
 //
 // Included by gmm.hip (uses its u32x4 / f32x16 types, mfma32, pack2 and the XCD tile mapping).
 //
 // Why: with 256x256 output tiles a compute unit has to pull 64 bytes of operands per 16
-// MFMA-cycles from L2 / Infinity Cache, whose latency under load is a few thousand cycles.  Loads
-// that pass through registers can only be one tile ahead (the registers are the limit), which
-// leaves the matrix cores idle most of the time.  Here the loads are `buffer_load_dwordx4 ... lds`:
-// they write LDS directly, occupy no registers, and three K tiles (96 KiB) are kept in flight per
-// compute unit while a fourth is multiplied.
+// MFMA-cycles.  Loads that pass through registers can only run one tile ahead and cost 64
+// registers per lane; `buffer_load_dwordx4 ... lds` writes LDS directly, so a whole K tile
+// (or several) is in flight while another is multiplied, with no register cost.
 //
-// LDS layout of one operand tile (R = 256 rows or columns, BK = 32):
-//   KC operand (reduction dim contiguous in memory): [row][32 k] = 64-byte rows, 16-byte chunk c
-//     of row r stored at chunk position c ^ ((r >> 2) & 3), so that the 16 lanes a ds_read_b128
-//     serves per cycle (16 consecutive rows, same chunk) touch 16 distinct 16-byte bank groups of
-//     the 64-bank LDS.
+// The L1 (TCP) of a compute unit handles about 0.35 distinct 128-byte lines per clock no matter how
+// few bytes of a line are wanted, so operand rows are fetched 128 bytes at a time: BK = 64 for the
+// operands whose reduction dimension is contiguous in memory.
+//
+// LDS layout of one operand tile (R = 256 rows or columns):
+//   KC operand (reduction dim contiguous in memory): [row][BK k], 16-byte chunk c of row r stored
+//     at chunk position c ^ swz(r), swz(r) = (r >> 1) & 7 for 128-byte rows (BK 64) and
+//     (r >> 2) & 3 for 64-byte rows (BK 32), so that the 16 lanes a ds_read_b128 serves per cycle
+//     (16 consecutive rows, same chunk) touch 16 distinct 16-byte bank groups of the 64-bank LDS.
 //   MC operand (reduction dim strided): [k][256 cols] = 512-byte rows, 32-byte pair p of row k
 //     stored at pair position p ^ (2 (k & 3)), so that the 32 lanes a ds_read_b64_tr_b16 serves per
 //     cycle (4 k-rows x two adjacent 32-byte pairs) touch 8 distinct pairs of a 256-byte bank line.
@@ -23,25 +25,27 @@
 #pragma once
 
 namespace dma {
+#ifdef MBX_TUNE_TIMING
+__device__ unsigned long long mbx_tune_counters[8];
+#endif
 
-constexpr int BK = 32;
-constexpr int STAGES = 4;
-
-template <int BM_, int BN_, int WM_, int WN_, int PREFETCH_ = 0>
+template <int BM_, int BN_, int WM_, int WN_, int BK_, int STAGES_>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, PREFETCH = PREFETCH_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, STAGES = STAGES_;
+  static constexpr int KS = BK / 16;                                           // MFMA k-steps per tile
   static constexpr int WAVES = WM * WN, THREADS = WAVES * kWave;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int A_INSTRS = A_BYTES / 1024, B_INSTRS = B_BYTES / 1024;  // wave-wide 1 KiB loads per tile
-  // L2 warm-up: per tile and operand, one 4-byte load per 64 bytes of the tile PREFETCH tiles ahead
-  static constexpr int PF_INSTRS_A = PREFETCH > 0 ? A_BYTES / 64 / kWave : 0, PF_INSTRS_B = PREFETCH > 0 ? B_BYTES / 64 / kWave : 0;
-  static constexpr int LOADS_PER_WAVE = (A_INSTRS + B_INSTRS + PF_INSTRS_A + PF_INSTRS_B) / WAVES;
-  static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_BYTES + (PREFETCH > 0 ? 256 * WAVES : 0);
-  static_assert(PREFETCH == 0 || (PF_INSTRS_A % WAVES == 0 && PF_INSTRS_B % WAVES == 0), "warm-up loads must split evenly over the waves");
+  static constexpr int LOADS_PER_WAVE = (A_INSTRS + B_INSTRS) / WAVES;
+  static constexpr size_t RING_BYTES = (size_t)STAGES * STAGE_BYTES, EPILOGUE_BYTES = (size_t)BM * (BN * 2 + 16);
+  static constexpr size_t LDS_BYTES = RING_BYTES > EPILOGUE_BYTES ? RING_BYTES : EPILOGUE_BYTES;
+  static_assert(BK == 32 || BK == 64, "K tile");
+  static_assert(STAGES >= 2 && LDS_BYTES <= 160 * 1024, "LDS ring");
   static_assert(A_INSTRS % WAVES == 0 && B_INSTRS % WAVES == 0, "loads must split evenly over the waves");
-  static_assert(WAVES % 2 == 0, "the MC swizzle needs the parity of a wave's load index to be fixed");
+  static_assert(WAVES % 2 == 0, "the swizzles need the parity of a wave's load index to be fixed");
+  static_assert((STAGES - 1) * LOADS_PER_WAVE < 64, "vmcnt is a 6-bit counter");
 };
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
@@ -66,13 +70,14 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
 }
 
 // Per-lane byte offset (inside an operand tile) of the MFMA operand of the 32 rows/cols starting
-// at `r`, k-step 0.  KC: k-step 1 is the same address with bit 5 flipped.  MC: k-step 1 is +8192.
-template <bool MC>
+// at `r`, k-step 0.  KC: k-step s is the same address with bits 5.. XORed by 32 s.  MC: +8192 s.
+template <bool MC, int BK>
 __device__ __forceinline__ uint32_t frag_lane_offset(int r) {
   const int lane = lane_id();
   if (!MC) {
-    const int row = lane & 31, xr = (row >> 2) & 3;
-    return (uint32_t)((r + row) * 64 + (((lane >> 5) ^ xr) << 4));
+    const int row = lane & 31;
+    const int swz = BK == 64 ? (row >> 1) & 7 : (row >> 2) & 3;
+    return (uint32_t)((r + row) * (BK * 2) + (((lane >> 5) ^ swz) << 4));
   } else {
     const int g = lane >> 4, s = lane & 15;
     const int k = (g >> 1) * 8 + (s >> 2);
@@ -97,38 +102,37 @@ __device__ __forceinline__ u32x4 read_frag(uint32_t tile_addr, uint32_t lane_off
 // ---- global -> LDS ----
 // Byte offset (from the operand's buffer base) fetched by this lane in the wave's first load of
 // tile 0; `r0` is the tile origin in the non-reduction dimension, `ld_bytes` the row pitch.
-template <bool MC>
+template <bool MC, int BK>
 __device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t ld_bytes) {
   const int lane = lane_id();
-  if (!MC) {  // 16 rows x 4 chunks per instruction
-    const int row = lane >> 2, pc = lane & 3;
-    const int c = pc ^ ((row >> 2) & 3);
-    return (uint32_t)(r0 + row) * ld_bytes + (uint32_t)(c << 4);
-  } else {    // 2 k-rows x 32 chunks per instruction; instruction j holds k = 2j, 2j + 1
+  if (!MC) {
+    if (BK == 64) {  // 8 rows x 8 chunks per instruction; instruction j holds rows 8j .. 8j + 7
+      const int row = lane >> 3, pc = lane & 7;
+      const int c = pc ^ ((4 * (wave & 1) + (row >> 1)) & 7);     // ((8j + row) >> 1) & 7 with j = wave (mod 2)
+      return (uint32_t)(r0 + row) * ld_bytes + (uint32_t)(c << 4);
+    } else {         // 16 rows x 4 chunks per instruction
+      const int row = lane >> 2, pc = lane & 3;
+      const int c = pc ^ ((row >> 2) & 3);
+      return (uint32_t)(r0 + row) * ld_bytes + (uint32_t)(c << 4);
+    }
+  } else {           // 2 k-rows x 32 chunks per instruction; instruction j holds k = 2j, 2j + 1
     const int kl = lane >> 5, pc = lane & 31;
-    const int k3 = (2 * (wave & 1) + kl) & 3;          // (2j + kl) & 3 with j = wave (mod 2)
+    const int k3 = (2 * (wave & 1) + kl) & 3;                     // (2j + kl) & 3 with j = wave (mod 2)
     const int c = ((((pc >> 1) ^ (2 * k3)) << 1) | (pc & 1));
     return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
   }
 }
 
-template <bool MC, int INSTRS, int WAVES>
+template <bool MC, int BK, int INSTRS, int WAVES>
 __device__ __forceinline__ void issue_operand(__amdgpu_buffer_rsrc_t rsrc, lds_ptr tile, int wave, uint32_t lane_off,
                                               uint32_t tile_off, uint32_t ld_bytes) {
+  constexpr uint32_t ROWS = MC ? 2u : (uint32_t)(1024 / (BK * 2));   // global rows covered by one instruction
 #pragma unroll
   for (int q = 0; q < INSTRS / WAVES; ++q) {
     const int j = wave + q * WAVES;
-    const uint32_t off = lane_off + tile_off + (uint32_t)j * (MC ? 2u : 16u) * ld_bytes;
+    const uint32_t off = lane_off + tile_off + (uint32_t)j * ROWS * ld_bytes;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(tile + j * 1024), 16, (int)off, 0, 0, 0);
   }
-}
-
-// Warm-up load: lane l of the wave's q-th instruction touches the 64-byte piece number
-// (wave + q * WAVES) * 64 + l of the operand tile.
-template <bool MC>
-__device__ __forceinline__ uint32_t touch_lane_offset(int piece, int r0, uint32_t ld_bytes) {
-  if (!MC) return (uint32_t)(r0 + piece) * ld_bytes;                                  // piece = row (64 bytes of k)
-  return (uint32_t)(piece >> 3) * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)((piece & 7) << 6);  // 8 pieces per k-row
 }
 
 struct Args {
@@ -156,148 +160,231 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const uint32_t a_lane = load_lane_offset<A_MC>(wave, g.a_r0, g.a_ld_bytes);
-  const uint32_t b_lane = load_lane_offset<B_MC>(wave, g.b_r0, g.b_ld_bytes);
+  constexpr int BK = T::BK, STAGES = T::STAGES, KS = T::KS;
+  const uint32_t a_lane = load_lane_offset<A_MC, BK>(wave, g.a_r0, g.a_ld_bytes);
+  const uint32_t b_lane = load_lane_offset<B_MC, BK>(wave, g.b_r0, g.b_ld_bytes);
   const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
   const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
-  uint32_t a_touch[T::PF_INSTRS_A / T::WAVES > 0 ? T::PF_INSTRS_A / T::WAVES : 1], b_touch[T::PF_INSTRS_B / T::WAVES > 0 ? T::PF_INSTRS_B / T::WAVES : 1];
-  if (T::PREFETCH > 0) {
-#pragma unroll
-    for (int q = 0; q < T::PF_INSTRS_A / T::WAVES; ++q) a_touch[q] = touch_lane_offset<A_MC>((wave + q * T::WAVES) * kWave + lane, g.a_r0, g.a_ld_bytes);
-#pragma unroll
-    for (int q = 0; q < T::PF_INSTRS_B / T::WAVES; ++q) b_touch[q] = touch_lane_offset<B_MC>((wave + q * T::WAVES) * kWave + lane, g.b_r0, g.b_ld_bytes);
-  }
-  auto issue = [&](int kt) {
-#ifdef MBX_TUNE_NO_GLOBAL
-    return;
-#endif
+  // q-th wave-wide load (of LOADS_PER_WAVE) of K tile kt: first the wave's share of A, then of B
+  // A tile index at or past nk is turned into an out-of-range offset: the load then fetches nothing
+  // and writes zeros into a stage nobody reads, which keeps the loop and its vmcnt bookkeeping uniform.
+  auto issue_one = [&](int kt, int q) {
     const lds_ptr stage = lds + (kt % STAGES) * T::STAGE_BYTES;
-    issue_operand<A_MC, T::A_INSTRS, T::WAVES>(g.rsrc_a, stage, wave, a_lane, (uint32_t)kt * a_step, g.a_ld_bytes);
-    issue_operand<B_MC, T::B_INSTRS, T::WAVES>(g.rsrc_b, stage + T::A_BYTES, wave, b_lane, (uint32_t)kt * b_step, g.b_ld_bytes);
-    if (T::PREFETCH > 0) {
-      // pull tile kt + PREFETCH into L2; the 4 bytes per lane land in a scratch corner of LDS nobody reads
-      const lds_ptr dump = lds + STAGES * T::STAGE_BYTES + wave * 256;
-      const uint32_t ka = (uint32_t)(kt + T::PREFETCH) * a_step, kb = (uint32_t)(kt + T::PREFETCH) * b_step;
-#pragma unroll
-      for (int q = 0; q < T::PF_INSTRS_A / T::WAVES; ++q)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_a, (__attribute__((address_space(3))) void*)dump, 4, (int)(a_touch[q] + ka), 0, 0, 0);
-#pragma unroll
-      for (int q = 0; q < T::PF_INSTRS_B / T::WAVES; ++q)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_b, (__attribute__((address_space(3))) void*)dump, 4, (int)(b_touch[q] + kb), 0, 0, 0);
+    const uint32_t past = kt < g.nk ? 0u : 0x80000000u;
+    constexpr int QA = T::A_INSTRS / T::WAVES;
+    if (q < QA) {
+      constexpr uint32_t ROWS = A_MC ? 2u : (uint32_t)(1024 / (BK * 2));
+      const int j = wave + q * T::WAVES;
+      const uint32_t off = (a_lane + (uint32_t)kt * a_step + (uint32_t)j * ROWS * g.a_ld_bytes) | past;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_a, (__attribute__((address_space(3))) void*)(stage + j * 1024), 16, (int)off, 0, 0, 0);
+    } else {
+      constexpr uint32_t ROWS = B_MC ? 2u : (uint32_t)(1024 / (BK * 2));
+      const int j = wave + (q - QA) * T::WAVES;
+      const uint32_t off = (b_lane + (uint32_t)kt * b_step + (uint32_t)j * ROWS * g.b_ld_bytes) | past;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_b, (__attribute__((address_space(3))) void*)(stage + T::A_BYTES + j * 1024), 16, (int)off, 0, 0, 0);
     }
   };
 
-  // per-lane LDS offsets of the MFMA operands (KC: one base, tiles at +i*2048; MC: one per tile)
+  // per-lane LDS offsets of the MFMA operands (KC: one base, 32-row tiles at +32 rows; MC: one per tile)
+  constexpr int KC_TILE = 32 * BK * 2;
   uint32_t fa_off[A_MC ? T::TM : 1], fb_off[B_MC ? T::TN : 1];
   if (A_MC) {
 #pragma unroll
-    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true>(wm + i * 32);
+    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true, BK>(wm + i * 32);
   } else {
-    fa_off[0] = frag_lane_offset<false>(wm);
+    fa_off[0] = frag_lane_offset<false, BK>(wm);
   }
   if (B_MC) {
 #pragma unroll
-    for (int j = 0; j < T::TN; ++j) fb_off[j] = T::A_BYTES + frag_lane_offset<true>(wn + j * 32);
+    for (int j = 0; j < T::TN; ++j) fb_off[j] = T::A_BYTES + frag_lane_offset<true, BK>(wn + j * 32);
   } else {
-    fb_off[0] = T::A_BYTES + frag_lane_offset<false>(wn);
+    fb_off[0] = T::A_BYTES + frag_lane_offset<false, BK>(wn);
   }
 
   u32x4 fa[2][T::TM], fb[2][T::TN];
-#ifdef MBX_TUNE_NO_LDS
-#define MBX_READ_FRAGS(KS, BUF, STAGE_ADDR) do { } while (0)
-#else
-#define MBX_READ_FRAGS(KS, BUF, STAGE_ADDR)                                                                      \
+  // m-th operand read (of TM + TN) of k-step KSTEP of the tile at STAGE_ADDR into register buffer BUF
+#define MBX_READ_ONE(KSTEP, BUF, STAGE_ADDR, M)                                                                  \
   do {                                                                                                           \
-    _Pragma("unroll") for (int i = 0; i < T::TM; ++i)                                                            \
-        fa[BUF][i] = A_MC ? read_frag<true, KS>(STAGE_ADDR, fa_off[A_MC ? i : 0])                                \
-                          : read_frag<false, KS>(STAGE_ADDR + i * 2048, fa_off[0]);                              \
-    _Pragma("unroll") for (int j = 0; j < T::TN; ++j)                                                            \
-        fb[BUF][j] = B_MC ? read_frag<true, KS>(STAGE_ADDR, fb_off[B_MC ? j : 0])                                \
-                          : read_frag<false, KS>(STAGE_ADDR + j * 2048, fb_off[0]);                              \
+    if ((M) < T::TM) {                                                                                           \
+      fa[BUF][(M) % T::TM] = A_MC ? read_frag<true, KSTEP>(STAGE_ADDR, fa_off[A_MC ? (M) % T::TM : 0])           \
+                                  : read_frag<false, KSTEP>(STAGE_ADDR + ((M) % T::TM) * KC_TILE, fa_off[0]);    \
+    } else if ((M) < T::TM + T::TN) {                                                                            \
+      fb[BUF][((M) - T::TM) % T::TN] =                                                                           \
+          B_MC ? read_frag<true, KSTEP>(STAGE_ADDR, fb_off[B_MC ? ((M) - T::TM) % T::TN : 0])                    \
+               : read_frag<false, KSTEP>(STAGE_ADDR + (((M) - T::TM) % T::TN) * KC_TILE, fb_off[0]);             \
+    }                                                                                                            \
   } while (0)
-#endif
+#define MBX_READ_FRAGS(KSTEP, BUF, STAGE_ADDR)                                                                   \
+  do {                                                                                                           \
+    _Pragma("unroll") for (int m_ = 0; m_ < T::TM + T::TN; ++m_) MBX_READ_ONE(KSTEP, BUF, STAGE_ADDR, m_);       \
+  } while (0)
   // the MFMAs may only start once the operands have arrived: tie them to the wait through "+v"
 #define MBX_WAIT_FRAGS(BUF)                                                                                      \
   do {                                                                                                           \
     _Pragma("unroll") for (int i = 0; i < T::TM; ++i) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[BUF][i]));    \
     _Pragma("unroll") for (int j = 0; j < T::TN; ++j) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[BUF][j]));    \
   } while (0)
-  // operands swapped: the accumulator tile is c^T, so a lane owns runs of four consecutive
-  // columns of one row of c and can store them as one 8-byte word
-#define MBX_MULTIPLY(BUF)                                                                                        \
+  // One k-step: TM x TN MFMAs on register buffer CUR_BUF.  Interleaved with them, so that neither
+  // the LDS nor the texture-address unit makes the wave wait with the matrix core idle:
+  //   * the operand reads of the next k-step (NEXT_KSTEP of the tile at NEXT_ADDR) into the other buffer,
+  //   * NLOADS global->LDS loads of K tile LOAD_KT, starting with the wave's LOAD_Q0-th.
+  // The accumulator tile is c^T (operands swapped): a lane owns runs of four consecutive columns
+  // of one row of c and can store them as one 8-byte word.
+#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_ADDR, LOAD_KT, LOAD_Q0, NLOADS)                                       \
   do {                                                                                                           \
-    _Pragma("unroll") for (int i = 0; i < T::TM; ++i)                                                            \
-      _Pragma("unroll") for (int j = 0; j < T::TN; ++j) acc[i][j] = mfma32<DT>(fb[BUF][j], fa[BUF][i], acc[i][j]); \
+    MBX_WAIT_FRAGS(CUR_BUF);                                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                                           \
+    _Pragma("unroll") for (int m_ = 0; m_ < T::TM * T::TN; ++m_) {                                               \
+      acc[m_ / T::TN][m_ % T::TN] =                                                                              \
+          mfma32<DT>(fb[CUR_BUF][m_ % T::TN], fa[CUR_BUF][m_ / T::TN], acc[m_ / T::TN][m_ % T::TN]);             \
+      MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_ADDR, m_);                                                    \
+      if ((NLOADS) > 0 && m_ % LOAD_EVERY == LOAD_EVERY - 1 && m_ / LOAD_EVERY < (NLOADS))                       \
+        issue_one(LOAD_KT, (LOAD_Q0) + m_ / LOAD_EVERY);                                                         \
+      __builtin_amdgcn_sched_barrier(0);                                                                         \
+    }                                                                                                            \
   } while (0)
 
   const int nk = g.nk;
+#ifdef MBX_TUNE_TIMING
+  long long tune_vm = 0, tune_bar = 0, tune_issue = 0;
+  const long long tune_t0 = __builtin_readcyclecounter();
+#endif
   if (nk > 0) {
-    // prologue: fill the ring, wait for tile 0
-#pragma unroll
-    for (int t = 0; t < STAGES; ++t)
-      if (t < nk) issue(t);
     constexpr int L = T::LOADS_PER_WAVE;
-    if (nk >= 4) wait_vmcnt<3 * L>();
-    else if (nk == 3) wait_vmcnt<2 * L>();
-    else if (nk == 2) wait_vmcnt<L>();
-    else wait_vmcnt<0>();
+    // The loads of a K tile are issued in two halves: the first during the last k-step of the tile
+    // whose stage it takes over (right after that stage became free), the second during the first
+    // k-step of the following tile.
+    constexpr int HALF = L / 2;
+    constexpr int LOAD_EVERY = (T::TM * T::TN) / (L - HALF) > 0 ? (T::TM * T::TN) / (L - HALF) : 1;
+    static_assert((L - HALF) * LOAD_EVERY <= T::TM * T::TN, "not enough MFMAs per k-step to hide the loads behind");
+    static_assert((STAGES - 1) * L < 64, "vmcnt is a 6-bit counter");
+    // prologue: tiles 0 .. STAGES-2 and the first half of tile STAGES-1, then wait for tile 0
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t)
+#pragma unroll
+      for (int q = 0; q < L; ++q) issue_one(t, q);
+#pragma unroll
+    for (int q = 0; q < HALF; ++q) issue_one(STAGES - 1, q);
+    wait_vmcnt<(STAGES - 2) * L + HALF>();
     __builtin_amdgcn_s_barrier();
     MBX_READ_FRAGS(0, 0, lds_base);
 
     for (int kt = 0; kt < nk; ++kt) {
       const uint32_t cur = lds_base + (uint32_t)(kt % STAGES) * T::STAGE_BYTES;
       const uint32_t nxt = lds_base + (uint32_t)((kt + 1) % STAGES) * T::STAGE_BYTES;
-      MBX_WAIT_FRAGS(0);            // operands of k-step 0, read half an iteration ago
-      MBX_READ_FRAGS(1, 1, cur);    // k-step 1 arrives under the MFMAs of k-step 0
-      __builtin_amdgcn_sched_barrier(0);
-      MBX_MULTIPLY(0);
-      __builtin_amdgcn_sched_barrier(0);
-      MBX_WAIT_FRAGS(1);
-      // Tile kt is now entirely in registers.  Once every wave is here and tile kt+1 has landed, the
-      // stage of tile kt can be refilled with tile kt+4.
-      const int ahead = nk - 2 - kt;  // tiles issued beyond kt+1
-      if (ahead >= 2) wait_vmcnt<2 * L>();
-      else if (ahead == 1) wait_vmcnt<L>();
-      else wait_vmcnt<0>();
+      MBX_STEP(0, 1, cur, kt - 1 + STAGES, HALF, L - HALF);
+      if (KS == 4) {
+        MBX_STEP(1, 2, cur, 0, 0, 0);
+        MBX_STEP(0, 3, cur, 0, 0, 0);
+      }
+      MBX_WAIT_FRAGS((KS - 1) & 1);
+#ifdef MBX_TUNE_TIMING
+      const long long tt0 = __builtin_readcyclecounter();
+#endif
+      // Tile kt is now entirely in registers.  Once every wave is here and tile kt+1 has landed
+      // (everything but the STAGES-2 tiles issued after it), the stage of tile kt can be refilled.
+      wait_vmcnt<(STAGES - 2) * L>();
+#ifdef MBX_TUNE_TIMING
+      const long long tt1 = __builtin_readcyclecounter();
+#endif
       __builtin_amdgcn_s_barrier();
-      if (kt + STAGES < nk) issue(kt + STAGES);
-      if (kt + 1 < nk) MBX_READ_FRAGS(0, 0, nxt);
-      __builtin_amdgcn_sched_barrier(0);
-      MBX_MULTIPLY(1);
-      __builtin_amdgcn_sched_barrier(0);
+#ifdef MBX_TUNE_TIMING
+      const long long tt2 = __builtin_readcyclecounter();
+      tune_vm += tt1 - tt0; tune_bar += tt2 - tt1;
+#endif
+      MBX_STEP((KS - 1) & 1, 0, nxt, kt + STAGES, 0, HALF);   // past the last tile this reads stale LDS into dead registers
     }
+    wait_vmcnt<0>();   // no load may still be writing LDS when the workgroup's LDS is handed on
   }
+#ifdef MBX_TUNE_TIMING
+  const long long tune_t1 = __builtin_readcyclecounter();
+#endif
+
 #undef MBX_READ_FRAGS
 #undef MBX_WAIT_FRAGS
-#undef MBX_MULTIPLY
+#undef MBX_READ_ONE
+#undef MBX_STEP
 
   // accumulator (i, j), register r of lane l holds c[m][n] with
   //   m = m_base + wm + 32 i + (l % 32),  n = n_base + wn + 32 j + 8 (r / 4) + 4 (l / 32) + (r % 4)
-  const bool n_vec = (ldc % 4 == 0) && (((uintptr_t)c & 7u) == 0);
+  if ((ldc % 8 == 0) && (((uintptr_t)c & 15u) == 0)) {
+    // Staged through LDS (free by now) so that every global store instruction writes whole rows of the
+    // tile: 64 lanes x 16 bytes = two 512-byte row segments, instead of 32 scattered 16-byte pieces.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    constexpr int ROW = T::BN * 2 + 16;   // bytes; the 16-byte pad spreads the rows of a column over the banks
 #pragma unroll
-  for (int i = 0; i < T::TM; ++i) {
-    const int m = m_base + wm + i * 32 + (lane & 31);
-    if (m >= m_lim) continue;
-    uint16_t* crow = c + (int64_t)m * ldc;
+    for (int i = 0; i < T::TM; ++i) {
+      const int ml = wm + i * 32 + (lane & 31);
 #pragma unroll
-    for (int j = 0; j < T::TN; ++j) {
+      for (int j = 0; j < T::TN; ++j) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n_base + wn + j * 32 + q * 8 + (lane >> 5) * 4;
-        const f32x16& v = acc[i][j];
-        if (n + 3 < n_lim && n_vec) {
+        for (int q = 0; q < 4; ++q) {
+          const int nl = wn + j * 32 + q * 8 + (lane >> 5) * 4;
+          const f32x16& v = acc[i][j];
           u32x2 w;
           w[0] = pack2<DT>(v[q * 4 + 0], v[q * 4 + 1]);
           w[1] = pack2<DT>(v[q * 4 + 2], v[q * 4 + 3]);
-          *(u32x2*)(crow + n) = w;
-        } else {
+          *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
+        }
+      }
+    }
+    __syncthreads();
+    constexpr int CHUNKS = T::BN / 8;                 // 16-byte chunks per tile row
+    constexpr int ROWS_PER_INSTR = kWave / CHUNKS;    // 2 for 256-wide tiles
+    const int rl = lane / CHUNKS, ch = lane % CHUNKS;
+    const int n = n_base + ch * 8;
+#pragma unroll 4
+    for (int it = wave; it < T::BM / ROWS_PER_INSTR; it += T::WAVES) {
+      const int ml = it * ROWS_PER_INSTR + rl, m = m_base + ml;
+      if (m >= m_lim || n >= n_lim) continue;
+      const u32x4 v = *(const __attribute__((address_space(3))) u32x4*)(lds + ml * ROW + ch * 16);
+      uint16_t* dst = c + (int64_t)m * ldc + n;
+      if (n + 8 <= n_lim) {
+        *(u32x4*)dst = v;
+      } else {
 #pragma unroll
-          for (int t = 0; t < 4; ++t)
-            if (n + t < n_lim) crow[n + t] = (uint16_t)(pack2<DT>(v[q * 4 + t], 0.f) & 0xffffu);
+        for (int t = 0; t < 8; ++t)
+          if (n + t < n_lim) dst[t] = (uint16_t)(v[t >> 1] >> ((t & 1) * 16));
+      }
+    }
+  } else {
+    const bool n_vec = (ldc % 4 == 0) && (((uintptr_t)c & 7u) == 0);
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i) {
+      const int m = m_base + wm + i * 32 + (lane & 31);
+      if (m >= m_lim) continue;
+      uint16_t* crow = c + (int64_t)m * ldc;
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n_base + wn + j * 32 + q * 8 + (lane >> 5) * 4;
+          const f32x16& v = acc[i][j];
+          if (n + 3 < n_lim && n_vec) {
+            u32x2 w;
+            w[0] = pack2<DT>(v[q * 4 + 0], v[q * 4 + 1]);
+            w[1] = pack2<DT>(v[q * 4 + 2], v[q * 4 + 3]);
+            *(u32x2*)(crow + n) = w;
+          } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              if (n + t < n_lim) crow[n + t] = (uint16_t)(pack2<DT>(v[q * 4 + t], 0.f) & 0xffffu);
+          }
         }
       }
     }
   }
+#ifdef MBX_TUNE_TIMING
+  if (lane == 0) {
+    const long long tune_t2 = __builtin_readcyclecounter();
+    atomicAdd((unsigned long long*)&mbx_tune_counters[0], (unsigned long long)(tune_t1 - tune_t0));
+    atomicAdd((unsigned long long*)&mbx_tune_counters[1], (unsigned long long)tune_vm);
+    atomicAdd((unsigned long long*)&mbx_tune_counters[2], (unsigned long long)tune_bar);
+    atomicAdd((unsigned long long*)&mbx_tune_counters[3], 1ull);
+    atomicAdd((unsigned long long*)&mbx_tune_counters[4], (unsigned long long)(tune_t2 - tune_t1));
+  }
+#endif
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
@@ -329,22 +416,32 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
   g.b_ld_bytes = (uint32_t)(B_MC ? n : k) * 2;
   g.b_r0 = tn * T::BN;
-  g.nk = k / BK;
+  g.nk = k / T::BK;
   block_gemm<DT, false, B_MC, T>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
 }
 
 // ---- TN ----
+// Tiles of one expert's [k, n] product are enumerated in 8 x 4 blocks (8 row tiles x 4 column
+// tiles), matching the run of 32 tiles an XCD works on at a time: 12 operand panels per 32 tiles.
+constexpr int kTnBlockM = 8, kTnBlockN = 4;
+static inline int64_t tn_tiles_per_group(int tiles_m, int tiles_n) {
+  return (int64_t)((tiles_m + kTnBlockM - 1) / kTnBlockM) * ((tiles_n + kTnBlockN - 1) / kTnBlockN) * (kTnBlockM * kTnBlockN);
+}
+
 template <int DT, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int id = xcd_tile_id(blockIdx.x);
-  const int per_group = tiles_m * tiles_n;
+  const int blocks_m = (tiles_m + kTnBlockM - 1) / kTnBlockM, blocks_n = (tiles_n + kTnBlockN - 1) / kTnBlockN;
+  const int per_group = blocks_m * blocks_n * (kTnBlockM * kTnBlockN);
   const int e = id / per_group;
   if (e >= num_groups) return;
   const int t = id % per_group;
-  const int tm = t % tiles_m, tn = t / tiles_m;
+  const int blk = t / (kTnBlockM * kTnBlockN), in = t % (kTnBlockM * kTnBlockN);
+  const int tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
+  if (tm >= tiles_m || tn >= tiles_n) return;   // padding of the 8 x 4 enumeration (uniform over the workgroup)
   const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
   const int64_t group_rows = end - start;
   Args g;
@@ -355,7 +452,7 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
   g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
   g.b_ld_bytes = (uint32_t)n * 2;
   g.b_r0 = tn * T::BN;
-  g.nk = (int)((group_rows + BK - 1) / BK);
+  g.nk = (int)((group_rows + T::BK - 1) / T::BK);
   block_gemm<DT, true, true, T>(g, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
 }
 
