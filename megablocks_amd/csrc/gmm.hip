@@ -184,11 +184,7 @@ __device__ __forceinline__ void block_gemm(const Operand& opa, const Operand& op
     for (int i = 0; i < T::TM; ++i)
 #pragma unroll
       for (int j = 0; j < T::TN; ++j) {
-#ifndef MBX_TUNE_NO_MFMA
         acc[i][j] = mfma32<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
-#else
-        acc[i][j][0] += __uint_as_float(fb[buf][j][0] ^ fa[buf][i][0]);
-#endif
       }
   };
 
@@ -208,10 +204,8 @@ __device__ __forceinline__ void block_gemm(const Operand& opa, const Operand& op
   for (int kt = 0; kt < nk; ++kt) {
     uint16_t* cur = lds + (kt & 1) * STAGE;
     uint16_t* nxt = lds + ((kt + 1) & 1) * STAGE;
-#ifndef MBX_TUNE_NO_GLOBAL
     SA::load(opa, k_begin + (kt + 1) * T::BK, k_begin, k_end, ra);
     SB::load(opb, k_begin + (kt + 1) * T::BK, k_begin, k_end, rb);
-#endif
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < KS - 1; ++ks) {

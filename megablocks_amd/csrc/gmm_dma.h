@@ -25,9 +25,6 @@
 #pragma once
 
 namespace dma {
-#ifdef MBX_TUNE_TIMING
-__device__ unsigned long long mbx_tune_counters[8];
-#endif
 
 template <int BM_, int BN_, int WM_, int WN_, int BK_, int STAGES_>
 struct Tile {
@@ -245,18 +242,15 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   } while (0)
 
   const int nk = g.nk;
-#ifdef MBX_TUNE_TIMING
-  long long tune_vm = 0, tune_bar = 0, tune_issue = 0;
-  const long long tune_t0 = __builtin_readcyclecounter();
-#endif
   if (nk > 0) {
     constexpr int L = T::LOADS_PER_WAVE;
     // The loads of a K tile are issued in two halves: the first during the last k-step of the tile
     // whose stage it takes over (right after that stage became free), the second during the first
     // k-step of the following tile.
     constexpr int HALF = L / 2;
-    constexpr int LOAD_EVERY = (T::TM * T::TN) / (L - HALF) > 0 ? (T::TM * T::TN) / (L - HALF) : 1;
-    static_assert((L - HALF) * LOAD_EVERY <= T::TM * T::TN, "not enough MFMAs per k-step to hide the loads behind");
+    constexpr int MAXPART = HALF > L - HALF ? HALF : L - HALF;
+    constexpr int LOAD_EVERY = (T::TM * T::TN) / MAXPART > 0 ? (T::TM * T::TN) / MAXPART : 1;
+    static_assert(MAXPART * LOAD_EVERY <= T::TM * T::TN, "not enough MFMAs per k-step to hide the loads behind");
     static_assert((STAGES - 1) * L < 64, "vmcnt is a 6-bit counter");
     // prologue: tiles 0 .. STAGES-2 and the first half of tile STAGES-1, then wait for tile 0
 #pragma unroll
@@ -278,27 +272,15 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
         MBX_STEP(0, 3, cur, 0, 0, 0);
       }
       MBX_WAIT_FRAGS((KS - 1) & 1);
-#ifdef MBX_TUNE_TIMING
-      const long long tt0 = __builtin_readcyclecounter();
-#endif
       // Tile kt is now entirely in registers.  Once every wave is here and tile kt+1 has landed
       // (everything but the STAGES-2 tiles issued after it), the stage of tile kt can be refilled.
       wait_vmcnt<(STAGES - 2) * L>();
-#ifdef MBX_TUNE_TIMING
-      const long long tt1 = __builtin_readcyclecounter();
-#endif
       __builtin_amdgcn_s_barrier();
-#ifdef MBX_TUNE_TIMING
-      const long long tt2 = __builtin_readcyclecounter();
-      tune_vm += tt1 - tt0; tune_bar += tt2 - tt1;
-#endif
       MBX_STEP((KS - 1) & 1, 0, nxt, kt + STAGES, 0, HALF);   // past the last tile this reads stale LDS into dead registers
     }
     wait_vmcnt<0>();   // no load may still be writing LDS when the workgroup's LDS is handed on
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // nor an LDS read still be landing in a register the epilogue reuses
   }
-#ifdef MBX_TUNE_TIMING
-  const long long tune_t1 = __builtin_readcyclecounter();
-#endif
 
 #undef MBX_READ_FRAGS
 #undef MBX_WAIT_FRAGS
@@ -310,7 +292,6 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   if ((ldc % 8 == 0) && (((uintptr_t)c & 15u) == 0)) {
     // Staged through LDS (free by now) so that every global store instruction writes whole rows of the
     // tile: 64 lanes x 16 bytes = two 512-byte row segments, instead of 32 scattered 16-byte pieces.
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __syncthreads();
     constexpr int ROW = T::BN * 2 + 16;   // bytes; the 16-byte pad spreads the rows of a column over the banks
 #pragma unroll
@@ -375,16 +356,6 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
       }
     }
   }
-#ifdef MBX_TUNE_TIMING
-  if (lane == 0) {
-    const long long tune_t2 = __builtin_readcyclecounter();
-    atomicAdd((unsigned long long*)&mbx_tune_counters[0], (unsigned long long)(tune_t1 - tune_t0));
-    atomicAdd((unsigned long long*)&mbx_tune_counters[1], (unsigned long long)tune_vm);
-    atomicAdd((unsigned long long*)&mbx_tune_counters[2], (unsigned long long)tune_bar);
-    atomicAdd((unsigned long long*)&mbx_tune_counters[3], 1ull);
-    atomicAdd((unsigned long long*)&mbx_tune_counters[4], (unsigned long long)(tune_t2 - tune_t1));
-  }
-#endif
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {

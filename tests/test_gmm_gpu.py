@@ -151,3 +151,32 @@ def test_gelu_backward_inplace():
         gd = g.cuda()
         out = gelu_backward_(gd, x.cuda())
         assert out is gd and rel_err(gd.cpu().float(), want) < (1e-5 if dtype == torch.float32 else 1e-2)
+
+
+DMA_EDGE = [  # groups, rows, k, n: shapes that take the direct-to-LDS kernels, off every tile boundary
+    (3, 700, 64, 8), (5, 1030, 128, 264), (2, 255, 192, 1408), (7, 3001, 320, 520), (1, 257, 64, 248),
+    (4, 513, 1024, 72), (6, 40, 64, 40),
+]
+
+
+@pytest.mark.parametrize('groups,rows,k,n', DMA_EDGE)
+@pytest.mark.parametrize('mode', ['nn', 'nt', 'tn'])
+def test_gmm_ragged_shapes_on_the_pipelined_path(gg, groups, rows, k, n, mode):
+    sizes = _sizes(groups, rows, seed=rows, empty=(0,) if groups > 2 else ())
+    a = torch.randn(rows, k).bfloat16()
+    if mode == 'tn':
+        b = torch.randn(rows, n).bfloat16()
+    elif mode == 'nt':
+        b = (torch.randn(groups, n, k) * 0.1).bfloat16()
+    else:
+        b = (torch.randn(groups, k, n) * 0.1).bfloat16()
+    want = oracle.gmm(a, b, sizes, trans_a=mode == 'tn', trans_b=mode == 'nt')
+    guard = torch.full((want.numel() + 4096,), 3.0).bfloat16().cuda()       # canary around the output
+    c = guard[2048:2048 + want.numel()].view(want.shape)
+    got = gg.backend.gmm(a.cuda(), b.cuda(), sizes, trans_a=mode == 'tn', trans_b=mode == 'nt', c=c)
+    assert rel_err(got.cpu(), want) < TOL
+    assert bool((guard[:2048] == 3.0).all()) and bool((guard[2048 + want.numel():] == 3.0).all())
+    if mode == 'tn':
+        for e, s in enumerate(sizes.tolist()):
+            if s == 0:
+                assert torch.count_nonzero(got[e]) == 0
