@@ -24,7 +24,11 @@ MFMA_PEAK = {'bf16': 2.5e15, 'f16': 2.5e15, 'f32': 157.3e12}
 HBM_PEAK = 8e12
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
 # keyed by (workload, kernel); None until measured for the workload at hand.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # workload c3, rocprofv3 FETCH_SIZE (x2.00, the factor a plain 1 GiB copy shows) + WRITE_SIZE, bytes per launch;
+    # see profiles/gmm_dmoe_c3_mixtral_hbm_traffic.txt
+    ('c3', 'gmm_nn'): 3.43e9, ('c3', 'gmm_nt'): 3.90e9, ('c3', 'gmm_tn'): 3.77e9,
+}
 
 
 def parse():
