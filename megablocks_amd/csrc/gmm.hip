@@ -257,13 +257,13 @@ __device__ __forceinline__ void block_gemm(const Operand& opa, const Operand& op
 constexpr int kXcds = 8;
 constexpr int kXcdRun = 32;
 
-__device__ __forceinline__ int xcd_tile_id(int block) {
+__device__ __forceinline__ int xcd_tile_id(int block, int run = kXcdRun) {
   const int xcd = block % kXcds, l = block / kXcds;
-  return ((l / kXcdRun) * kXcds + xcd) * kXcdRun + (l % kXcdRun);
+  return ((l / run) * kXcds + xcd) * run + (l % run);
 }
 
-static inline int64_t xcd_grid(int64_t tiles) {
-  const int64_t q = (int64_t)kXcds * kXcdRun;
+static inline int64_t xcd_grid(int64_t tiles, int run = kXcdRun) {
+  const int64_t q = (int64_t)kXcds * run;
   return (tiles + q - 1) / q * q;
 }
 
@@ -452,7 +452,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     auto kern = dma::gmm_tn_kernel<DT, T>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    const int64_t grid = xcd_grid(dma::tn_tiles_per_group(tiles_m, tiles_n) * num_groups);
+    const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups);
     if (grid > 0x7fffffff) return MBX_ERANGE;
     kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n);
     return launch_status();

@@ -392,11 +392,18 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
 }
 
 // ---- TN ----
-// Tiles of one expert's [k, n] product are enumerated in 8 x 4 blocks (8 row tiles x 4 column
-// tiles), matching the run of 32 tiles an XCD works on at a time: 12 operand panels per 32 tiles.
+// Tiles of one expert's [k, n] product are enumerated in 8 x 4 blocks (8 row tiles x 4 column tiles:
+// 12 operand panels per 32 tiles), and that sequence is cut into 8 equal pieces, one per XCD: XCD x
+// works through piece x of the first expert, piece x of the second, and so on.  The cost of a tile
+// is proportional to its expert's row count, so with skewed routing any coarser dealing of tiles to
+// XCDs (whose queues are fixed by the workgroup id) leaves some XCDs with several times the work.
 constexpr int kTnBlockM = 8, kTnBlockN = 4;
 static inline int64_t tn_tiles_per_group(int tiles_m, int tiles_n) {
   return (int64_t)((tiles_m + kTnBlockM - 1) / kTnBlockM) * ((tiles_n + kTnBlockN - 1) / kTnBlockN) * (kTnBlockM * kTnBlockN);
+}
+static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups) {
+  const int64_t per_xcd = (tn_tiles_per_group(tiles_m, tiles_n) + kXcds - 1) / kXcds;
+  return per_xcd * kXcds * num_groups;
 }
 
 template <int DT, typename T>
@@ -404,12 +411,28 @@ __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  const int id = xcd_tile_id(blockIdx.x);
   const int blocks_m = (tiles_m + kTnBlockM - 1) / kTnBlockM, blocks_n = (tiles_n + kTnBlockN - 1) / kTnBlockN;
   const int per_group = blocks_m * blocks_n * (kTnBlockM * kTnBlockN);
-  const int e = id / per_group;
-  if (e >= num_groups) return;
-  const int t = id % per_group;
+  const int per_xcd = (per_group + kXcds - 1) / kXcds;
+  const int xcd = blockIdx.x % kXcds, local = blockIdx.x / kXcds;
+  const int slot = local / per_xcd;                      // position of the expert in the longest-first order
+  const int t = xcd * per_xcd + local % per_xcd;         // tile slot inside the expert
+  if (slot >= num_groups || t >= per_group) return;
+  // Experts are taken in order of decreasing row count (longest reduction first), so that the tiles
+  // of a heavily loaded expert do not start last and leave most of the chip idle at the end.  With at
+  // most 64 experts every workgroup ranks them itself: lane e holds expert e's row count.
+  int e = slot;
+  if (num_groups <= kWave) {
+    const int lane = lane_id();
+    const int mine = lane < num_groups ? bins[lane] - (lane > 0 ? bins[lane - 1] : 0) : -1;
+    int rank = 0;
+    for (int o = 0; o < num_groups; ++o) {
+      const int other = __shfl(mine, o, kWave);
+      rank += (other > mine || (other == mine && o < lane)) ? 1 : 0;
+    }
+    const uint64_t hit = __ballot(lane < num_groups && rank == slot);
+    e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
+  }
   const int blk = t / (kTnBlockM * kTnBlockN), in = t % (kTnBlockM * kTnBlockN);
   const int tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
   if (tm >= tiles_m || tn >= tiles_n) return;   // padding of the 8 x 4 enumeration (uniform over the workgroup)
