@@ -145,6 +145,19 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
 int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel,
                               mbx_stream_t stream);
 
+/* The gated activation of the GLU experts, megablocks/layers/glu.py:89,204
+ * (`activation_fn(x1) * x2`) in one pass: out = round(round(act(a)) * b), i.e. with the same two
+ * roundings as the reference's two element-wise ops.  act: 0 = SiLU, 1 = tanh-GELU.  numel must be a
+ * multiple of 16 bytes' worth of elements and the buffers 16-byte aligned (else MBX_EINVAL). */
+enum mbx_activation { MBX_ACT_SILU = 0, MBX_ACT_GELU_TANH = 1 };
+int mbx_glu_forward(const void* a, const void* b, void* out, int dtype, int act, int64_t numel,
+                    mbx_stream_t stream);
+
+/* Backward of the above as autograd derives it for glu.py:89 / glu.py:120-151:
+ * db = g * round(act(a)), da = round(g * b) * act'(a). */
+int mbx_glu_backward(const void* g, const void* a, const void* b, void* da, void* db, int dtype,
+                     int act, int64_t numel, mbx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

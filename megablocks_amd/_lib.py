@@ -38,13 +38,15 @@ _SIGNATURES = {
     'mbx_binned_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _vp]),
     'mbx_gmm': (_i, [_vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gelu_backward_inplace': (_i, [_vp, _vp, _i, _i64, _vp]),
+    'mbx_glu_forward': (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp]),
+    'mbx_glu_backward': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _vp]),
 }
 
 
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f'{LIB_PATH} is missing: build the HIP kernels first with `python -m megablocks_amd.build` '
+            f'{LIB_PATH} is missing: build the HIP kernels first with `python megablocks_amd/build.py` '
             '(needs hipcc; cross-compiles for gfx950 without a GPU).')
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in _SIGNATURES.items():

@@ -1,7 +1,10 @@
 """Builds libmbx.so (the HIP kernels + C ABI) in-tree for gfx950 with hipcc.
 
-    python -m megablocks_amd.build            # compile what is out of date
-    python -m megablocks_amd.build --force    # recompile everything
+    python megablocks_amd/build.py            # compile what is out of date
+    python megablocks_amd/build.py --force    # recompile everything
+
+(run it as a script: `python -m megablocks_amd.build` would import the package, which needs the
+library to exist already)
 """
 import os
 import subprocess
@@ -11,8 +14,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
 BUILD = os.path.join(HERE, 'build')
 LIB = os.path.join(HERE, 'libmbx.so')
-SOURCES = ['routing.hip', 'permute.hip', 'gmm.hip']
-HEADERS = [os.path.join(CSRC, 'common.h'), os.path.join(os.path.dirname(HERE), 'include', 'mbx.h')]
+SOURCES = ['routing.hip', 'permute.hip', 'gmm.hip', 'elementwise.hip']
+HEADERS = [os.path.join(CSRC, 'common.h'), os.path.join(CSRC, 'gmm_dma.h'),
+           os.path.join(os.path.dirname(HERE), 'include', 'mbx.h')]
 ARCH = 'gfx950'
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from scalar float code.
 FLAGS = ['-O3', '-fPIC', '-std=c++17', f'--offload-arch={ARCH}', '-Xclang', '-target-feature', '-Xclang',

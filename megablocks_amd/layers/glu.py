@@ -1,10 +1,85 @@
 """Gated expert MLPs: megablocks/layers/glu.py.  y = (act(x @ w1.T) * (x @ v1.T)) @ w2 per expert."""
 import torch
 
+from functools import partial
+
+import torch.nn.functional as F
+
+from megablocks_amd import _lib
 from megablocks_amd import grouped_gemm_util as gg
+from megablocks_amd._lib import lib
 from megablocks_amd.layers import common, mpu
-from megablocks_amd.layers.arguments import Arguments
+from megablocks_amd.layers.arguments import DEFAULT_ACTIVATION_FN, Arguments
 from megablocks_amd.layers.mlp import SparseMLP, Topology, create_dmoe_expert_weights
+
+_ACT_SILU, _ACT_GELU_TANH = 0, 1
+
+
+def _activation_code(fn):
+    """Code of an activation the fused gated-activation kernels implement, else None."""
+    if fn is F.silu:
+        return _ACT_SILU
+    if fn is DEFAULT_ACTIVATION_FN:
+        return _ACT_GELU_TANH
+    if isinstance(fn, partial) and fn.func is F.gelu and not fn.args and fn.keywords == {'approximate': 'tanh'}:
+        return _ACT_GELU_TANH
+    return None
+
+
+def _fusable(*tensors):
+    t0 = tensors[0]
+    per = 16 // t0.element_size()
+    return (t0.is_cuda and t0.dtype in _lib.DTYPE and t0.numel() % per == 0 and
+            all(t.is_contiguous() and t.dtype == t0.dtype and t.shape == t0.shape and t.data_ptr() % 16 == 0
+                for t in tensors))
+
+
+def _glu_forward(a, b, act):
+    out = torch.empty_like(a)
+    with torch.cuda.device_of(a):
+        _lib.check(lib.mbx_glu_forward(_lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.dtype_of(a), act, a.numel(),
+                                       _lib.stream()), 'glu_forward')
+    return out
+
+
+def _glu_backward(g, a, b, act):
+    da, db = torch.empty_like(a), torch.empty_like(a)
+    with torch.cuda.device_of(a):
+        _lib.check(lib.mbx_glu_backward(_lib.ptr(g), _lib.ptr(a), _lib.ptr(b), _lib.ptr(da), _lib.ptr(db),
+                                        _lib.dtype_of(a), act, a.numel(), _lib.stream()), 'glu_backward')
+    return da, db
+
+
+class GatedActivation(torch.autograd.Function):
+    """`activation_fn(a) * b` (glu.py:89,204) and its gradient, one kernel each instead of two and
+    three element-wise passes; same values (each intermediate is rounded as the separate ops round it)."""
+
+    @staticmethod
+    def forward(ctx, a, b, act):
+        ctx.save_for_backward(a, b)
+        ctx.act = act
+        return _glu_forward(a, b, act)
+
+    @staticmethod
+    def backward(ctx, g):
+        a, b = ctx.saved_tensors
+        g = g.contiguous()
+        if not _fusable(g, a, b):
+            with torch.enable_grad():
+                a_, b_ = a.detach().requires_grad_(True), b.detach().requires_grad_(True)
+                fn = F.silu if ctx.act == _ACT_SILU else DEFAULT_ACTIVATION_FN
+                (fn(a_) * b_).backward(g)
+            return a_.grad, b_.grad, None
+        da, db = _glu_backward(g, a, b, ctx.act)
+        return da, db, None
+
+
+def gated_activation(activation_fn, a, b):
+    """activation_fn(a) * b, fused when the activation is SiLU or tanh-GELU and the layout allows."""
+    act = _activation_code(activation_fn)
+    if act is not None and _fusable(a, b):
+        return GatedActivation.apply(a, b, act)
+    return activation_fn(a) * b
 
 
 class MemoryOptimizedGroupedGLU(torch.autograd.Function):
@@ -19,7 +94,11 @@ class MemoryOptimizedGroupedGLU(torch.autograd.Function):
             raise ValueError("Expected contiguous 'x', 'w1', 'v1' and 'w2'.")
         sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
         v1_out = gg.backend.gmm(x, v1, batch_sizes, trans_b=True)
-        activation_fn_out = activation_fn(sdd_out) * v1_out
+        act = _activation_code(activation_fn)
+        if act is not None and _fusable(sdd_out, v1_out):
+            activation_fn_out = _glu_forward(sdd_out, v1_out, act)
+        else:
+            activation_fn_out = activation_fn(sdd_out) * v1_out
         dsd_out = gg.backend.gmm(activation_fn_out, w2, batch_sizes)
         ctx.x_shape = x.shape
         ctx.sdd_out_shape = sdd_out.shape
@@ -36,15 +115,25 @@ class MemoryOptimizedGroupedGLU(torch.autograd.Function):
         w1, v1, w2, batch_sizes, x, sdd_out, v1_out = ctx.saved_tensors
         ddsd_out = ddsd_out.contiguous()
         activation_fn = ctx.activation_fn
-        with torch.set_grad_enabled(True):
-            sdd_out = sdd_out.detach().requires_grad_(True)
-            v1_out = v1_out.detach().requires_grad_(True)
-            activation_fn_out = activation_fn(sdd_out) * v1_out
+        act = _activation_code(activation_fn)
+        fused = act is not None and _fusable(sdd_out, v1_out)
+        if fused:
+            activation_fn_out = _glu_forward(sdd_out, v1_out, act)       # recomputed, not saved
+        else:
+            with torch.set_grad_enabled(True):
+                sdd_out = sdd_out.detach().requires_grad_(True)
+                v1_out = v1_out.detach().requires_grad_(True)
+                activation_fn_out = activation_fn(sdd_out) * v1_out
 
         dw2 = gg.backend.gmm(activation_fn_out.detach(), ddsd_out, batch_sizes, trans_a=True)
-        dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True)
-        activation_fn_out.backward(dactivation_fn_out)
-        dsdd_out, dv1_out = sdd_out.grad, v1_out.grad
+        if fused:
+            # the gradient of the activation output overwrites the recomputed activation
+            dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True, c=activation_fn_out)
+            dsdd_out, dv1_out = _glu_backward(dactivation_fn_out, sdd_out, v1_out, act)
+        else:
+            dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True)
+            activation_fn_out.backward(dactivation_fn_out)
+            dsdd_out, dv1_out = sdd_out.grad, v1_out.grad
 
         dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
         dv1 = gg.backend.gmm(dv1_out, x, batch_sizes, trans_a=True)
@@ -77,7 +166,7 @@ class SparseGLU(SparseMLP):
             return memory_optimized_grouped_glu(x, w1, v1, w2, batch_sizes, self.args.activation_fn)
         x1 = gg.ops.gmm(x, w1, batch_sizes, trans_b=True)
         x2 = gg.ops.gmm(x, v1, batch_sizes, trans_b=True)
-        x1 = self.args.activation_fn(x1) * x2
+        x1 = gated_activation(self.args.activation_fn, x1, x2)
         return gg.ops.gmm(x1, w2, batch_sizes)
 
     def forward(self, x, topo: Topology):

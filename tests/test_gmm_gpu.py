@@ -180,3 +180,28 @@ def test_gmm_ragged_shapes_on_the_pipelined_path(gg, groups, rows, k, n, mode):
         for e, s in enumerate(sizes.tolist()):
             if s == 0:
                 assert torch.count_nonzero(got[e]) == 0
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('act_name', ['silu', 'gelu_tanh'])
+def test_fused_gated_activation_matches_the_two_step_formulation(dtype, act_name):
+    import torch.nn.functional as F
+    from megablocks_amd.layers.arguments import DEFAULT_ACTIVATION_FN
+    from megablocks_amd.layers.glu import gated_activation
+    fn = F.silu if act_name == 'silu' else DEFAULT_ACTIVATION_FN
+    a = (torch.randn(777, 1408) * 2).to(dtype).cuda().requires_grad_(True)
+    b = torch.randn(777, 1408).to(dtype).cuda().requires_grad_(True)
+    g = torch.randn(777, 1408).to(dtype).cuda()
+    out = gated_activation(fn, a, b)
+    out.backward(g)
+    a2, b2 = a.detach().clone().requires_grad_(True), b.detach().clone().requires_grad_(True)
+    want = fn(a2) * b2                                   # the reference's two element-wise ops (glu.py:89)
+    want.backward(g)
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    assert rel_err(out, want) < tol and rel_err(a.grad, a2.grad) < tol and rel_err(b.grad, b2.grad) < tol
+    if dtype != torch.float32:                           # forward: same roundings -> almost always the same bits
+        assert float((out != want).float().mean()) < 1e-3
+    wantf = fn(a.detach().float().cpu()) * b.detach().float().cpu()      # CPU fp32 check of the math itself
+    assert rel_err(out.cpu(), wantf) < (1e-5 if dtype == torch.float32 else 1e-2)
+    odd = torch.randn(5, 3).to(dtype).cuda()             # not a multiple of 16 bytes: plain torch ops
+    assert torch.equal(gated_activation(fn, odd, odd), fn(odd) * odd)
