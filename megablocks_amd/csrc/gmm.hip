@@ -390,6 +390,9 @@ __global__ void gelu_backward_kernel(void* __restrict__ g_, const void* __restri
 // 256 registers per lane and needs 144 KiB of the 160 KiB LDS for two stages.
 typedef Tile<256, 256, 64, 2, 2, 8, 32> TileBig;
 typedef dma::Tile<256, 256, 2, 2, 64, 2> TileDma;
+// For small experts (NN / NT only: the row tile follows the expert's row count) a 128-row tile wastes
+// fewer rows of the last tile of every expert; its smaller stages allow a three-deep ring.
+typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;
 
 template <int DT, bool A_MC, bool B_MC, typename T>
 constexpr size_t lds_bytes() {
@@ -447,7 +450,9 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const uint16_t* bp = (const uint16_t*)b;
   uint16_t* cp = (uint16_t*)c;
   constexpr size_t lds = T::LDS_BYTES;
+  static_assert(T::BN == 256, "the [k][cols] LDS layout of a strided operand is written for 256-column tiles");
   if (layout == MBX_TN) {
+    if (T::BM != 256) return MBX_EINVAL;   // both TN operands are strided
     const int tiles_m = (int)ceil_div(k, T::BM), tiles_n = (int)ceil_div(n, T::BN);
     auto kern = dma::gmm_tn_kernel<DT, T>;
     int rc = allow_lds(kern, lds);
@@ -523,6 +528,11 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     bool dma_ok = rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
     if (layout != MBX_TN) dma_ok = dma_ok && k % TileDma::BK == 0;
     if (dma_ok) {
+      const bool small_m = layout != MBX_TN && rows <= (int64_t)num_groups * 320;   // average rows per expert
+      if (small_m) {
+        if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+        return gmm_dma<MBX_F16, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+      }
       if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);
       return gmm_dma<MBX_F16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);
     }
