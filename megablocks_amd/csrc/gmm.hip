@@ -442,39 +442,60 @@ int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num
   return launch_status();
 }
 
-// Launch of the direct-to-LDS kernels (k a multiple of 32 for NN / NT, operands below 2 GiB).
-template <int DT, typename T>
+// One persistent workgroup per compute unit (a multiple of 8, so that every XCD gets the same number),
+// fewer when there are not that many tiles.
+static inline int persistent_grid(int64_t tiles_upper_bound) {
+  static int cus[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < kXcds) n = 256;
+    cus[dev] = n / kXcds * kXcds;
+  }
+  const int64_t need = (tiles_upper_bound + kXcds - 1) / kXcds * kXcds;
+  return (int)(need < cus[dev] ? need : cus[dev]);
+}
+
+// Launch of the direct-to-LDS kernels (k a multiple of 64 for NN / NT, operands below 2 GiB).
+// TS is the tile the tail of an NN / NT launch is cut into (TS = T: never cut).
+template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
             int layout, hipStream_t s) {
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
   uint16_t* cp = (uint16_t*)c;
-  constexpr size_t lds = T::LDS_BYTES;
   static_assert(T::BN == 256, "the [k][cols] LDS layout of a strided operand is written for 256-column tiles");
   if (layout == MBX_TN) {
     if (T::BM != 256) return MBX_EINVAL;   // both TN operands are strided
+    constexpr size_t lds = T::LDS_BYTES;
     const int tiles_m = (int)ceil_div(k, T::BM), tiles_n = (int)ceil_div(n, T::BN);
     auto kern = dma::gmm_tn_kernel<DT, T>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups);
+    // short reductions (few rows per expert): several tiles per workgroup
+    const int64_t avg_rows = rows / (num_groups > 0 ? num_groups : 1);
+    const int chunk = avg_rows >= 1024 ? 1 : avg_rows >= 512 ? 2 : 4;
+    const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups, chunk);
     if (grid > 0x7fffffff) return MBX_ERANGE;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n);
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n, chunk);
     return launch_status();
   }
+  constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
   const int tiles_n = (int)ceil_div(n, T::BN);
-  const int64_t grid = xcd_grid((ceil_div(rows, T::BM) + num_groups) * tiles_n);
-  if (grid > 0x7fffffff) return MBX_ERANGE;
+  const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
+  if (tiles > 0x7fffffff) return MBX_ERANGE;
+  const unsigned grid = (unsigned)persistent_grid(tiles);
   if (layout == MBX_NT) {
-    auto kern = dma::gmm_rows_kernel<DT, false, T>;
+    auto kern = dma::gmm_rows_kernel<DT, false, T, TS>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
+    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
   } else {
-    auto kern = dma::gmm_rows_kernel<DT, true, T>;
+    auto kern = dma::gmm_rows_kernel<DT, true, T, TS>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
+    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
   }
   return launch_status();
 }
@@ -530,11 +551,11 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     if (dma_ok) {
       const bool small_m = layout != MBX_TN && rows <= (int64_t)num_groups * 320;   // average rows per expert
       if (small_m) {
-        if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-        return gmm_dma<MBX_F16, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+        if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+        return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
       }
-      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-      return gmm_dma<MBX_F16, TileDma>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+      return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
     }
     if (dtype == MBX_BF16) return gmm_mfma<MBX_BF16, TileBig>(a, b, c, bins, num_groups, rows, k, n, layout, s);
     return gmm_mfma<MBX_F16, TileBig>(a, b, c, bins, num_groups, rows, k, n, layout, s);

@@ -362,33 +362,137 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
 }
 
+// ---- workgroups that compute several tiles ----
+// An NN / NT launch has one workgroup per compute unit (P of them, a multiple of 8); each walks a
+// fixed list of tiles (all tiles of such a launch cost the same).  Workgroup w sits on XCD w % 8 and
+// is that XCD's member w / 8; the P / 8 members of an XCD take one run of P / 8 consecutive tiles per
+// round, so the tiles an XCD works on at any time are a compact block that shares operand panels in
+// that XCD's L2.  Walking the list inside the kernel spares a workgroup launch and an expert lookup
+// from scratch per tile, and makes the last, partly filled round visible to the kernel.
+
+// The LDS and the operand registers of the finished tile are dead once every wave is here.
+__device__ __forceinline__ void tile_done() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+}
+
 // ---- NN / NT ----
-template <int DT, bool B_MC, typename T>
+// Logical tile id -> (expert, column tile, row tile inside the expert), row tiles fastest.  With at
+// most 64 experts lane e of every wave keeps expert e's row range and the inclusive count of tiles
+// up to it, and a tile id is resolved with one ballot; with more, by a scan over the bins.
+template <int BM>
+struct RowTiles {
+  int lane_start = 0, lane_end = 0, lane_mt = 0, lane_incl = 0;
+  int total = 0;
+  bool table;
+  const int32_t* bins;
+  int num_groups, tiles_n;
+
+  __device__ __forceinline__ RowTiles(const int32_t* bins_, int num_groups_, int tiles_n_)
+      : bins(bins_), num_groups(num_groups_), tiles_n(tiles_n_) {
+    table = num_groups <= kWave;
+    if (table) {
+      const int lane = lane_id();
+      if (lane < num_groups) {
+        lane_end = bins[lane];
+        lane_start = lane > 0 ? bins[lane - 1] : 0;
+        const int mt = (lane_end - lane_start + BM - 1) / BM;
+        lane_mt = mt > 0 ? mt : 0;
+      }
+      int incl = lane_mt * tiles_n;
+#pragma unroll
+      for (int o = 1; o < kWave; o <<= 1) {
+        const int v = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += v;
+      }
+      lane_incl = incl;
+      total = __builtin_amdgcn_readlane(incl, kWave - 1);
+    } else {
+      int start = 0;
+      for (int e = 0; e < num_groups; ++e) {
+        const int end = bins[e];
+        const int mt = (end - start + BM - 1) / BM;
+        total += (mt > 0 ? mt : 0) * tiles_n;
+        start = end;
+      }
+    }
+  }
+
+  // id in [0, total) -> expert, its row range, the row tile and the column tile
+  __device__ __forceinline__ void find(int id, int& e, int& start, int& end, int& tm, int& tn) const {
+    int mt;
+    if (table) {
+      const uint64_t hit = __ballot(id < lane_incl);
+      e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
+      start = __builtin_amdgcn_readlane(lane_start, e);
+      end = __builtin_amdgcn_readlane(lane_end, e);
+      mt = __builtin_amdgcn_readlane(lane_mt, e);
+      id -= __builtin_amdgcn_readlane(lane_incl, e) - mt * tiles_n;
+    } else {
+      start = 0; end = 0; mt = 0;
+      for (e = 0; e < num_groups; ++e) {
+        end = bins[e];
+        mt = (end - start + BM - 1) / BM;
+        mt = mt > 0 ? mt : 0;
+        const int span = mt * tiles_n;
+        if (id < span) break;
+        id -= span;
+        start = end;
+      }
+    }
+    tn = id / mt;
+    tm = id % mt;
+  }
+};
+
+// T is the main tile.  When the last round would leave at least half of the compute units idle, its
+// R tiles are cut into 2 R half tiles of TS (BM / 2 rows, same columns), spread over all XCDs:
+// the tail then costs little more than half a round.  TS = T switches this off.
+template <int DT, bool B_MC, typename T, typename TS>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  int id = xcd_tile_id(blockIdx.x);
-  int e = 0, start = 0, end = 0, mt = 0;
-  for (; e < num_groups; ++e) {
-    end = bins[e];
-    mt = (end - start + T::BM - 1) / T::BM;
-    const int span = mt * tiles_n;
-    if (id < span) break;
-    id -= span;
-    start = end;
-  }
-  if (e >= num_groups) return;
-  const int tn = id / mt, tm = id % mt;
+  static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "tail tile");
+  constexpr bool kSplit = T::BM != TS::BM;
+  static_assert(!kSplit || T::BM == 2 * TS::BM, "tail tile");
+  const int P = gridDim.x, run = P / kXcds;
+  const int xcd = blockIdx.x % kXcds, member = blockIdx.x / kXcds;
+  const RowTiles<T::BM> tiles(bins, num_groups, tiles_n);
+  const int total = tiles.total;
+  const int full_rounds = total / P, rest = total - full_rounds * P;
+  const bool split = kSplit && rest > 0 && 2 * rest <= P;
+  const int big_rounds = full_rounds + ((rest > 0 && !split) ? 1 : 0);
+
   Args g;
   g.rsrc_a = make_rsrc(a, (uint32_t)(rows * k * 2));
   g.a_ld_bytes = (uint32_t)k * 2;
-  g.a_r0 = start + tm * T::BM;
-  g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
   g.b_ld_bytes = (uint32_t)(B_MC ? n : k) * 2;
-  g.b_r0 = tn * T::BN;
   g.nk = k / T::BK;
-  block_gemm<DT, false, B_MC, T>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+  for (int r = 0; r < big_rounds; ++r) {
+    const int id = (r * kXcds + xcd) * run + member;
+    if (id >= total) break;
+    int e, start, end, tm, tn;
+    tiles.find(id, e, start, end, tm, tn);
+    g.a_r0 = start + tm * T::BM;
+    g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
+    g.b_r0 = tn * T::BN;
+    block_gemm<DT, false, B_MC, T>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+    tile_done();
+  }
+  if (kSplit && split) {
+    const int j = xcd * run + member;     // half tile j: tile j / 2 of the tail, rows half j % 2
+    if (j < 2 * rest) {
+      int e, start, end, tm, tn;
+      tiles.find(full_rounds * P + j / 2, e, start, end, tm, tn);
+      g.a_r0 = start + tm * T::BM + (j & 1) * TS::BM;
+      if (g.a_r0 < end) {
+        g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
+        g.b_r0 = tn * TS::BN;
+        block_gemm<DT, false, B_MC, TS>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+      }
+    }
+  }
 }
 
 // ---- TN ----
@@ -397,57 +501,67 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
 // works through piece x of the first expert, piece x of the second, and so on.  The cost of a tile
 // is proportional to its expert's row count, so with skewed routing any coarser dealing of tiles to
 // XCDs (whose queues are fixed by the workgroup id) leaves some XCDs with several times the work.
+// For the same reason the tiles of an XCD are not dealt to workgroups statically: a workgroup takes
+// `chunk` consecutive tiles of its XCD's list and the hardware hands out workgroups as compute units
+// become free (chunk > 1 when the reductions are short and the per-workgroup overhead shows).
 constexpr int kTnBlockM = 8, kTnBlockN = 4;
 static inline int64_t tn_tiles_per_group(int tiles_m, int tiles_n) {
   return (int64_t)((tiles_m + kTnBlockM - 1) / kTnBlockM) * ((tiles_n + kTnBlockN - 1) / kTnBlockN) * (kTnBlockM * kTnBlockN);
 }
-static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups) {
+static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chunk) {
   const int64_t per_xcd = (tn_tiles_per_group(tiles_m, tiles_n) + kXcds - 1) / kXcds;
-  return per_xcd * kXcds * num_groups;
+  return (per_xcd * num_groups + chunk - 1) / chunk * kXcds;
 }
 
 template <int DT, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
-              const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n) {
+              const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int blocks_m = (tiles_m + kTnBlockM - 1) / kTnBlockM, blocks_n = (tiles_n + kTnBlockN - 1) / kTnBlockN;
   const int per_group = blocks_m * blocks_n * (kTnBlockM * kTnBlockN);
   const int per_xcd = (per_group + kXcds - 1) / kXcds;
-  const int xcd = blockIdx.x % kXcds, local = blockIdx.x / kXcds;
-  const int slot = local / per_xcd;                      // position of the expert in the longest-first order
-  const int t = xcd * per_xcd + local % per_xcd;         // tile slot inside the expert
-  if (slot >= num_groups || t >= per_group) return;
+  const int xcd = blockIdx.x % kXcds;
   // Experts are taken in order of decreasing row count (longest reduction first), so that the tiles
   // of a heavily loaded expert do not start last and leave most of the chip idle at the end.  With at
-  // most 64 experts every workgroup ranks them itself: lane e holds expert e's row count.
-  int e = slot;
-  if (num_groups <= kWave) {
+  // most 64 experts every wave ranks them itself: lane e holds expert e's row count and its rank.
+  const bool ranked = num_groups <= kWave;
+  int rank = -1;
+  if (ranked) {
     const int lane = lane_id();
     const int mine = lane < num_groups ? bins[lane] - (lane > 0 ? bins[lane - 1] : 0) : -1;
-    int rank = 0;
+    rank = 0;
     for (int o = 0; o < num_groups; ++o) {
       const int other = __shfl(mine, o, kWave);
       rank += (other > mine || (other == mine && o < lane)) ? 1 : 0;
     }
-    const uint64_t hit = __ballot(lane < num_groups && rank == slot);
-    e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
+    if (lane >= num_groups) rank = -1;
   }
-  const int blk = t / (kTnBlockM * kTnBlockN), in = t % (kTnBlockM * kTnBlockN);
-  const int tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
-  if (tm >= tiles_m || tn >= tiles_n) return;   // padding of the 8 x 4 enumeration (uniform over the workgroup)
-  const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
-  const int64_t group_rows = end - start;
   Args g;
-  // the buffers cover exactly the rows of this expert: later rows read as zero
-  g.rsrc_a = make_rsrc(a + (int64_t)start * k, (uint32_t)(group_rows * k * 2));
   g.a_ld_bytes = (uint32_t)k * 2;
-  g.a_r0 = tm * T::BM;
-  g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
   g.b_ld_bytes = (uint32_t)n * 2;
-  g.b_r0 = tn * T::BN;
-  g.nk = (int)((group_rows + T::BK - 1) / T::BK);
-  block_gemm<DT, true, true, T>(g, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
+  const int64_t items = (int64_t)per_xcd * num_groups;   // per XCD
+  const int64_t first = (int64_t)(blockIdx.x / kXcds) * chunk;
+  for (int64_t i = first; i < first + chunk && i < items; ++i) {
+    const int slot = (int)(i / per_xcd);                  // position of the expert in the longest-first order
+    const int t = xcd * per_xcd + (int)(i % per_xcd);     // tile slot inside the expert
+    if (t >= per_group) continue;
+    const int blk = t / (kTnBlockM * kTnBlockN), in = t % (kTnBlockM * kTnBlockN);
+    const int tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
+    if (tm >= tiles_m || tn >= tiles_n) continue;   // padding of the 8 x 4 enumeration (uniform over the workgroup)
+    int e = slot;
+    if (ranked) e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(__ballot(rank == slot)));
+    const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
+    const int64_t group_rows = end - start;
+    // the buffers cover exactly the rows of this expert: later rows read as zero
+    g.rsrc_a = make_rsrc(a + (int64_t)start * k, (uint32_t)(group_rows * k * 2));
+    g.a_r0 = tm * T::BM;
+    g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
+    g.b_r0 = tn * T::BN;
+    g.nk = (int)((group_rows + T::BK - 1) / T::BK);
+    block_gemm<DT, true, true, T>(g, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
+    tile_done();
+  }
 }
 
 }  // namespace dma
