@@ -392,7 +392,7 @@ typedef Tile<256, 256, 64, 2, 2, 8, 32> TileBig;
 typedef dma::Tile<256, 256, 2, 2, 64, 2> TileDma;
 // For small experts (NN / NT only: the row tile follows the expert's row count) a 128-row tile wastes
 // fewer rows of the last tile of every expert; its smaller stages allow a three-deep ring.
-typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;
+typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;   // 4 x 16 KiB + 3 x 32 KiB
 
 template <int DT, bool A_MC, bool B_MC, typename T>
 constexpr size_t lds_bytes() {

@@ -24,28 +24,48 @@
 // compiler would otherwise wait for ALL outstanding LDS-DMA loads before any LDS read.
 #pragma once
 
+#include <type_traits>
+#include <utility>
+
 namespace dma {
 
-template <int BM_, int BN_, int WM_, int WN_, int BK_, int STAGES_>
+// The two operands have separate LDS rings: SB stages for the B operand and SA = SB + 1 for the A
+// operand.  The extra A stage lets the A loads of a K tile be issued during the k-steps in which no
+// B load can be (the B stage to refill is still being read), so that global -> LDS loads leave the
+// compute unit at an even rate: the texture-address unit takes some 20 cycles per wave-wide load, is
+// shared by the four waves, and a wave whose load has to queue cannot issue its next MFMA either.
+template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, STAGES = STAGES_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1;
   static constexpr int KS = BK / 16;                                           // MFMA k-steps per tile
   static constexpr int WAVES = WM * WN, THREADS = WAVES * kWave;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
-  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int A_INSTRS = A_BYTES / 1024, B_INSTRS = B_BYTES / 1024;  // wave-wide 1 KiB loads per tile
-  static constexpr int LOADS_PER_WAVE = (A_INSTRS + B_INSTRS) / WAVES;
-  static constexpr size_t RING_BYTES = (size_t)STAGES * STAGE_BYTES, EPILOGUE_BYTES = (size_t)BM * (BN * 2 + 16);
+  static constexpr int LA = A_INSTRS / WAVES, LB = B_INSTRS / WAVES;          // ... per wave
+  static constexpr size_t RING_BYTES = (size_t)SA * A_BYTES + (size_t)SB * B_BYTES, EPILOGUE_BYTES = (size_t)BM * (BN * 2 + 16);
   static constexpr size_t LDS_BYTES = RING_BYTES > EPILOGUE_BYTES ? RING_BYTES : EPILOGUE_BYTES;
-  static_assert(BK == 32 || BK == 64, "K tile");
-  static_assert(STAGES >= 2 && LDS_BYTES <= 160 * 1024, "LDS ring");
+  static_assert(BK == 64, "K tile");
+  static_assert(SB >= 2 && LDS_BYTES <= 160 * 1024, "LDS rings");
   static_assert(A_INSTRS % WAVES == 0 && B_INSTRS % WAVES == 0, "loads must split evenly over the waves");
+  static_assert(LA % 2 == 0 && LB % 2 == 0, "the loads of an operand tile are issued in two halves");
   static_assert(WAVES % 2 == 0, "the swizzles need the parity of a wave's load index to be fixed");
-  static_assert((STAGES - 1) * LOADS_PER_WAVE < 64, "vmcnt is a 6-bit counter");
+  static_assert((SB - 1) * (LA + LB) + LA + LB / 2 < 64, "vmcnt is a 6-bit counter");
 };
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
+// expression in the body (it selects instruction immediates).
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {  // at most N vector-memory loads of this wave still in flight
@@ -83,10 +103,11 @@ __device__ __forceinline__ uint32_t frag_lane_offset(int r) {
   }
 }
 
-template <bool MC, int KS>
+// IMM: constant byte offset of the 32-row tile inside a KC operand tile (goes into the instruction).
+template <bool MC, int KS, int IMM = 0>
 __device__ __forceinline__ u32x4 read_frag(uint32_t tile_addr, uint32_t lane_off) {
   if (!MC) {
-    return lds_read_b128<0>(tile_addr + (lane_off ^ (KS * 32)));
+    return lds_read_b128<IMM>(tile_addr + (lane_off ^ (KS * 32)));
   } else {
     const u32x2 lo = lds_read_tr16_b64<KS * 8192>(tile_addr + lane_off);
     const u32x2 hi = lds_read_tr16_b64<KS * 8192 + 2048>(tile_addr + lane_off);
@@ -157,29 +178,29 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  constexpr int BK = T::BK, STAGES = T::STAGES, KS = T::KS;
+  constexpr int BK = T::BK, SA = T::SA, SB = T::SB, LA = T::LA, LB = T::LB;
+  static_assert(T::KS == 4, "the schedule below is written for four k-steps per K tile");
+  constexpr uint32_t B_RING = (uint32_t)SA * T::A_BYTES;   // the B stages follow the A stages
   const uint32_t a_lane = load_lane_offset<A_MC, BK>(wave, g.a_r0, g.a_ld_bytes);
   const uint32_t b_lane = load_lane_offset<B_MC, BK>(wave, g.b_r0, g.b_ld_bytes);
   const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
   const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
-  // q-th wave-wide load (of LOADS_PER_WAVE) of K tile kt: first the wave's share of A, then of B
+  // q-th wave-wide load of the wave's share of the A (B) part of K tile kt into ring stage `stage`.
   // A tile index at or past nk is turned into an out-of-range offset: the load then fetches nothing
   // and writes zeros into a stage nobody reads, which keeps the loop and its vmcnt bookkeeping uniform.
-  auto issue_one = [&](int kt, int q) {
-    const lds_ptr stage = lds + (kt % STAGES) * T::STAGE_BYTES;
+  auto issue_a = [&](int kt, int stage, int q) {
+    constexpr uint32_t ROWS = A_MC ? 2u : (uint32_t)(1024 / (BK * 2));
     const uint32_t past = kt < g.nk ? 0u : 0x80000000u;
-    constexpr int QA = T::A_INSTRS / T::WAVES;
-    if (q < QA) {
-      constexpr uint32_t ROWS = A_MC ? 2u : (uint32_t)(1024 / (BK * 2));
-      const int j = wave + q * T::WAVES;
-      const uint32_t off = (a_lane + (uint32_t)kt * a_step + (uint32_t)j * ROWS * g.a_ld_bytes) | past;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_a, (__attribute__((address_space(3))) void*)(stage + j * 1024), 16, (int)off, 0, 0, 0);
-    } else {
-      constexpr uint32_t ROWS = B_MC ? 2u : (uint32_t)(1024 / (BK * 2));
-      const int j = wave + (q - QA) * T::WAVES;
-      const uint32_t off = (b_lane + (uint32_t)kt * b_step + (uint32_t)j * ROWS * g.b_ld_bytes) | past;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_b, (__attribute__((address_space(3))) void*)(stage + T::A_BYTES + j * 1024), 16, (int)off, 0, 0, 0);
-    }
+    const int j = wave + q * T::WAVES;
+    const uint32_t off = a_lane + (((uint32_t)kt * a_step + (uint32_t)j * ROWS * g.a_ld_bytes) | past);   // operands are below 2 GiB
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_a, (__attribute__((address_space(3))) void*)(lds + stage * T::A_BYTES + j * 1024), 16, (int)off, 0, 0, 0);
+  };
+  auto issue_b = [&](int kt, int stage, int q) {
+    constexpr uint32_t ROWS = B_MC ? 2u : (uint32_t)(1024 / (BK * 2));
+    const uint32_t past = kt < g.nk ? 0u : 0x80000000u;
+    const int j = wave + q * T::WAVES;
+    const uint32_t off = b_lane + (((uint32_t)kt * b_step + (uint32_t)j * ROWS * g.b_ld_bytes) | past);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_b, (__attribute__((address_space(3))) void*)(lds + B_RING + stage * T::B_BYTES + j * 1024), 16, (int)off, 0, 0, 0);
   };
 
   // per-lane LDS offsets of the MFMA operands (KC: one base, 32-row tiles at +32 rows; MC: one per tile)
@@ -193,27 +214,27 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   }
   if (B_MC) {
 #pragma unroll
-    for (int j = 0; j < T::TN; ++j) fb_off[j] = T::A_BYTES + frag_lane_offset<true, BK>(wn + j * 32);
+    for (int j = 0; j < T::TN; ++j) fb_off[j] = frag_lane_offset<true, BK>(wn + j * 32);
   } else {
-    fb_off[0] = T::A_BYTES + frag_lane_offset<false, BK>(wn);
+    fb_off[0] = frag_lane_offset<false, BK>(wn);
   }
 
   u32x4 fa[2][T::TM], fb[2][T::TN];
-  // m-th operand read (of TM + TN) of k-step KSTEP of the tile at STAGE_ADDR into register buffer BUF
-#define MBX_READ_ONE(KSTEP, BUF, STAGE_ADDR, M)                                                                  \
+  // m-th operand read (of TM + TN) of k-step KSTEP of the tiles at A_ADDR / B_ADDR into register buffer BUF
+#define MBX_READ_ONE(KSTEP, BUF, A_ADDR, B_ADDR, M)                                                              \
   do {                                                                                                           \
     if ((M) < T::TM) {                                                                                           \
-      fa[BUF][(M) % T::TM] = A_MC ? read_frag<true, KSTEP>(STAGE_ADDR, fa_off[A_MC ? (M) % T::TM : 0])           \
-                                  : read_frag<false, KSTEP>(STAGE_ADDR + ((M) % T::TM) * KC_TILE, fa_off[0]);    \
+      fa[BUF][(M) % T::TM] = A_MC ? read_frag<true, KSTEP>(A_ADDR, fa_off[A_MC ? (M) % T::TM : 0])               \
+                                  : read_frag<false, KSTEP, ((M) % T::TM) * KC_TILE>(A_ADDR, fa_off[0]);         \
     } else if ((M) < T::TM + T::TN) {                                                                            \
       fb[BUF][((M) - T::TM) % T::TN] =                                                                           \
-          B_MC ? read_frag<true, KSTEP>(STAGE_ADDR, fb_off[B_MC ? ((M) - T::TM) % T::TN : 0])                    \
-               : read_frag<false, KSTEP>(STAGE_ADDR + (((M) - T::TM) % T::TN) * KC_TILE, fb_off[0]);             \
+          B_MC ? read_frag<true, KSTEP>(B_ADDR, fb_off[B_MC ? ((M) - T::TM) % T::TN : 0])                        \
+               : read_frag<false, KSTEP, (((M) - T::TM) % T::TN) * KC_TILE>(B_ADDR, fb_off[0]);                  \
     }                                                                                                            \
   } while (0)
-#define MBX_READ_FRAGS(KSTEP, BUF, STAGE_ADDR)                                                                   \
+#define MBX_READ_FRAGS(KSTEP, BUF, A_ADDR, B_ADDR)                                                               \
   do {                                                                                                           \
-    _Pragma("unroll") for (int m_ = 0; m_ < T::TM + T::TN; ++m_) MBX_READ_ONE(KSTEP, BUF, STAGE_ADDR, m_);       \
+    static_for<T::TM + T::TN>([&](auto mi_) { constexpr int m_ = decltype(mi_)::value; MBX_READ_ONE(KSTEP, BUF, A_ADDR, B_ADDR, m_); }); \
   } while (0)
   // the MFMAs may only start once the operands have arrived: tie them to the wait through "+v"
 #define MBX_WAIT_FRAGS(BUF)                                                                                      \
@@ -223,60 +244,69 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   } while (0)
   // One k-step: TM x TN MFMAs on register buffer CUR_BUF.  Interleaved with them, so that neither
   // the LDS nor the texture-address unit makes the wave wait with the matrix core idle:
-  //   * the operand reads of the next k-step (NEXT_KSTEP of the tile at NEXT_ADDR) into the other buffer,
-  //   * NLOADS global->LDS loads of K tile LOAD_KT, starting with the wave's LOAD_Q0-th.
+  //   * the operand reads of the next k-step (NEXT_KSTEP of the tiles at NEXT_A / NEXT_B) into the other buffer,
+  //   * NLOADS global->LDS loads (ISSUE = issue_a or issue_b) of K tile LOAD_KT into stage LOAD_STAGE,
+  //     starting with the wave's LOAD_Q0-th, one after every (TM TN / NLOADS)-th MFMA.
   // The accumulator tile is c^T (operands swapped): a lane owns runs of four consecutive columns
   // of one row of c and can store them as one 8-byte word.
-#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_ADDR, LOAD_KT, LOAD_Q0, NLOADS)                                       \
+#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, ISSUE, LOAD_KT, LOAD_STAGE, LOAD_Q0, NLOADS)               \
   do {                                                                                                           \
+    constexpr int every_ = (T::TM * T::TN) / (NLOADS);                                                           \
+    static_assert(every_ >= 1, "not enough MFMAs per k-step to hide the loads behind");                          \
     MBX_WAIT_FRAGS(CUR_BUF);                                                                                     \
     __builtin_amdgcn_sched_barrier(0);                                                                           \
-    _Pragma("unroll") for (int m_ = 0; m_ < T::TM * T::TN; ++m_) {                                               \
+    static_for<T::TM * T::TN>([&](auto mi_) {                                                                    \
+      constexpr int m_ = decltype(mi_)::value;                                                                   \
       acc[m_ / T::TN][m_ % T::TN] =                                                                              \
           mfma32<DT>(fb[CUR_BUF][m_ % T::TN], fa[CUR_BUF][m_ / T::TN], acc[m_ / T::TN][m_ % T::TN]);             \
-      MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_ADDR, m_);                                                    \
-      if ((NLOADS) > 0 && m_ % LOAD_EVERY == LOAD_EVERY - 1 && m_ / LOAD_EVERY < (NLOADS))                       \
-        issue_one(LOAD_KT, (LOAD_Q0) + m_ / LOAD_EVERY);                                                         \
+      MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                               \
+      if (m_ % every_ == every_ - 1 && m_ / every_ < (NLOADS)) ISSUE(LOAD_KT, LOAD_STAGE, (LOAD_Q0) + m_ / every_); \
       __builtin_amdgcn_sched_barrier(0);                                                                         \
-    }                                                                                                            \
+    });                                                                                                          \
   } while (0)
 
   const int nk = g.nk;
   if (nk > 0) {
-    constexpr int L = T::LOADS_PER_WAVE;
-    // The loads of a K tile are issued in two halves: the first during the last k-step of the tile
-    // whose stage it takes over (right after that stage became free), the second during the first
-    // k-step of the following tile.
-    constexpr int HALF = L / 2;
-    constexpr int MAXPART = HALF > L - HALF ? HALF : L - HALF;
-    constexpr int LOAD_EVERY = (T::TM * T::TN) / MAXPART > 0 ? (T::TM * T::TN) / MAXPART : 1;
-    static_assert(MAXPART * LOAD_EVERY <= T::TM * T::TN, "not enough MFMAs per k-step to hide the loads behind");
-    static_assert((STAGES - 1) * L < 64, "vmcnt is a 6-bit counter");
-    // prologue: tiles 0 .. STAGES-2 and the first half of tile STAGES-1, then wait for tile 0
+    // Iteration kt multiplies K tile kt (A stage kt % SA, B stage kt % SB) and issues, spread evenly
+    // over its four k-steps:
+    //   k-step 0: the second half of B tile kt + SB - 1 -> B stage (kt - 1) % SB   (free since the barrier of kt - 1)
+    //   k-steps 1, 2: the halves of A tile kt + SB      -> A stage (kt - 1) % SA   (likewise)
+    //   barrier: every wave has tile kt in registers and tile kt + 1 has landed
+    //   k-step 3: the first half of B tile kt + SB      -> B stage kt % SB         (free since that barrier)
+    // Loads complete in order, so "tile kt + 1 has landed" is "at most WAIT_LOOP of my loads in flight".
+    constexpr int WAIT_PROLOGUE = (SB - 2) * (LA + LB) + LA + LB / 2;
+    constexpr int WAIT_LOOP = (SB - 1) * LA + (SB - 2) * LB;
+    // prologue: tiles 0 .. SB-2, the A part and half of the B part of tile SB-1, then wait for tile 0
 #pragma unroll
-    for (int t = 0; t < STAGES - 1; ++t)
+    for (int t = 0; t < SB - 1; ++t) {
 #pragma unroll
-      for (int q = 0; q < L; ++q) issue_one(t, q);
+      for (int q = 0; q < LA; ++q) issue_a(t, t, q);
 #pragma unroll
-    for (int q = 0; q < HALF; ++q) issue_one(STAGES - 1, q);
-    wait_vmcnt<(STAGES - 2) * L + HALF>();
+      for (int q = 0; q < LB; ++q) issue_b(t, t, q);
+    }
+#pragma unroll
+    for (int q = 0; q < LA; ++q) issue_a(SB - 1, SB - 1, q);
+#pragma unroll
+    for (int q = 0; q < LB / 2; ++q) issue_b(SB - 1, SB - 1, q);
+    wait_vmcnt<WAIT_PROLOGUE>();
     __builtin_amdgcn_s_barrier();
-    MBX_READ_FRAGS(0, 0, lds_base);
+    MBX_READ_FRAGS(0, 0, lds_base, lds_base + B_RING);
 
+    int sa = 0, sb = 0;   // kt % SA, kt % SB
     for (int kt = 0; kt < nk; ++kt) {
-      const uint32_t cur = lds_base + (uint32_t)(kt % STAGES) * T::STAGE_BYTES;
-      const uint32_t nxt = lds_base + (uint32_t)((kt + 1) % STAGES) * T::STAGE_BYTES;
-      MBX_STEP(0, 1, cur, kt - 1 + STAGES, HALF, L - HALF);
-      if (KS == 4) {
-        MBX_STEP(1, 2, cur, 0, 0, 0);
-        MBX_STEP(0, 3, cur, 0, 0, 0);
-      }
-      MBX_WAIT_FRAGS((KS - 1) & 1);
-      // Tile kt is now entirely in registers.  Once every wave is here and tile kt+1 has landed
-      // (everything but the STAGES-2 tiles issued after it), the stage of tile kt can be refilled.
-      wait_vmcnt<(STAGES - 2) * L>();
+      const int sa_prev = sa == 0 ? SA - 1 : sa - 1, sb_prev = sb == 0 ? SB - 1 : sb - 1;
+      const int sa_next = sa == SA - 1 ? 0 : sa + 1, sb_next = sb == SB - 1 ? 0 : sb + 1;
+      const uint32_t a_cur = lds_base + (uint32_t)sa * T::A_BYTES, b_cur = lds_base + B_RING + (uint32_t)sb * T::B_BYTES;
+      const uint32_t a_nxt = lds_base + (uint32_t)sa_next * T::A_BYTES, b_nxt = lds_base + B_RING + (uint32_t)sb_next * T::B_BYTES;
+      MBX_STEP(0, 1, a_cur, b_cur, issue_b, kt + SB - 1, sb_prev, LB / 2, LB / 2);
+      MBX_STEP(1, 2, a_cur, b_cur, issue_a, kt + SB, sa_prev, 0, LA / 2);
+      MBX_STEP(0, 3, a_cur, b_cur, issue_a, kt + SB, sa_prev, LA / 2, LA / 2);
+      MBX_WAIT_FRAGS(1);
+      wait_vmcnt<WAIT_LOOP>();
       __builtin_amdgcn_s_barrier();
-      MBX_STEP((KS - 1) & 1, 0, nxt, kt + STAGES, 0, HALF);   // past the last tile this reads stale LDS into dead registers
+      MBX_STEP(1, 0, a_nxt, b_nxt, issue_b, kt + SB, sb, 0, LB / 2);   // past the last tile this reads stale LDS into dead registers
+      sa = sa_next;
+      sb = sb_next;
     }
     wait_vmcnt<0>();   // no load may still be writing LDS when the workgroup's LDS is handed on
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // nor an LDS read still be landing in a register the epilogue reuses
