@@ -153,6 +153,21 @@ __device__ __forceinline__ void issue_operand(__amdgpu_buffer_rsrc_t rsrc, lds_p
   }
 }
 
+// One wait for all LDS reads in flight, tied to the operand registers of a k-step so that the MFMAs
+// that consume them cannot be scheduled above it.
+template <int NA, int NB>
+__device__ __forceinline__ void wait_frags(u32x4 (&a)[NA], u32x4 (&b)[NB]) {
+  static_assert(NA <= 4 && NB <= 4 && NA >= 2 && NB >= 2, "operand registers per k-step");
+  if constexpr (NA == 4 && NB == 4) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+  } else if constexpr (NA == 4 && NB == 2) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]));
+  } else {
+    static_for<NA>([&](auto i) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[decltype(i)::value])); });
+    static_for<NB>([&](auto i) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(b[decltype(i)::value])); });
+  }
+}
+
 struct Args {
   __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b;  // out-of-range bytes read as zero
   uint32_t a_ld_bytes, b_ld_bytes;
@@ -185,22 +200,36 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   const uint32_t b_lane = load_lane_offset<B_MC, BK>(wave, g.b_r0, g.b_ld_bytes);
   const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
   const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
-  // q-th wave-wide load of the wave's share of the A (B) part of K tile kt into ring stage `stage`.
-  // A tile index at or past nk is turned into an out-of-range offset: the load then fetches nothing
-  // and writes zeros into a stage nobody reads, which keeps the loop and its vmcnt bookkeeping uniform.
-  auto issue_a = [&](int kt, int stage, int q) {
-    constexpr uint32_t ROWS = A_MC ? 2u : (uint32_t)(1024 / (BK * 2));
-    const uint32_t past = kt < g.nk ? 0u : 0x80000000u;
-    const int j = wave + q * T::WAVES;
-    const uint32_t off = a_lane + (((uint32_t)kt * a_step + (uint32_t)j * ROWS * g.a_ld_bytes) | past);   // operands are below 2 GiB
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_a, (__attribute__((address_space(3))) void*)(lds + stage * T::A_BYTES + j * 1024), 16, (int)off, 0, 0, 0);
+  // The q-th wave-wide load of this wave's share of an operand tile is load number j = wave + q WAVES
+  // of the tile: 1 KiB of LDS at j KiB, global rows j ROWS onwards.  Byte offset into the operand =
+  // lane part (a_lane / b_lane) + scalar part; the scalar part of K tile kt, load j is
+  // kt a_step + j a_jstep.  A tile index at or past nk gets bit 31 set in the scalar part (operands are
+  // below 2 GiB): the load is then out of range, fetches nothing and writes zeros into a stage nobody
+  // reads, which keeps the loop and its vmcnt bookkeeping uniform.
+  constexpr uint32_t A_ROWS = A_MC ? 2u : (uint32_t)(1024 / (BK * 2)), B_ROWS = B_MC ? 2u : (uint32_t)(1024 / (BK * 2));
+  const uint32_t a_jstep = A_ROWS * g.a_ld_bytes, b_jstep = B_ROWS * g.b_ld_bytes;
+  auto scalar_off = [&](bool is_b, int kt, int q) -> uint32_t {
+    const uint32_t j = (uint32_t)(wave + q * T::WAVES);
+    const uint32_t v = is_b ? (uint32_t)kt * b_step + j * b_jstep : (uint32_t)kt * a_step + j * a_jstep;
+    return v | (kt < g.nk ? 0u : 0x80000000u);
   };
-  auto issue_b = [&](int kt, int stage, int q) {
-    constexpr uint32_t ROWS = B_MC ? 2u : (uint32_t)(1024 / (BK * 2));
-    const uint32_t past = kt < g.nk ? 0u : 0x80000000u;
-    const int j = wave + q * T::WAVES;
-    const uint32_t off = b_lane + (((uint32_t)kt * b_step + (uint32_t)j * ROWS * g.b_ld_bytes) | past);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_b, (__attribute__((address_space(3))) void*)(lds + B_RING + stage * T::B_BYTES + j * 1024), 16, (int)off, 0, 0, 0);
+  auto lds_off = [&](bool is_b, int stage, int q) -> uint32_t {
+    return (is_b ? B_RING + (uint32_t)stage * T::B_BYTES : (uint32_t)stage * T::A_BYTES) + (uint32_t)(wave + q * T::WAVES) * 1024u;
+  };
+  auto issue = [&](bool is_b, uint32_t sc, uint32_t dst) {
+    if (is_b) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_b, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(b_lane + sc), 0, 0, 0);
+    } else {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_a, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(a_lane + sc), 0, 0, 0);
+    }
+  };
+  auto issue_group = [&](bool is_b, int kt, int stage, int q0, int count) {   // prologue
+    uint32_t sc = scalar_off(is_b, kt, q0), dst = lds_off(is_b, stage, q0);
+    for (int i = 0; i < count; ++i) {
+      issue(is_b, sc, dst);
+      sc += T::WAVES * (is_b ? b_jstep : a_jstep);
+      dst += T::WAVES * 1024u;
+    }
   };
 
   // per-lane LDS offsets of the MFMA operands (KC: one base, 32-row tiles at +32 rows; MC: one per tile)
@@ -237,22 +266,22 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
     static_for<T::TM + T::TN>([&](auto mi_) { constexpr int m_ = decltype(mi_)::value; MBX_READ_ONE(KSTEP, BUF, A_ADDR, B_ADDR, m_); }); \
   } while (0)
   // the MFMAs may only start once the operands have arrived: tie them to the wait through "+v"
-#define MBX_WAIT_FRAGS(BUF)                                                                                      \
-  do {                                                                                                           \
-    _Pragma("unroll") for (int i = 0; i < T::TM; ++i) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[BUF][i]));    \
-    _Pragma("unroll") for (int j = 0; j < T::TN; ++j) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[BUF][j]));    \
-  } while (0)
+#define MBX_WAIT_FRAGS(BUF) wait_frags(fa[BUF], fb[BUF])
   // One k-step: TM x TN MFMAs on register buffer CUR_BUF.  Interleaved with them, so that neither
   // the LDS nor the texture-address unit makes the wave wait with the matrix core idle:
   //   * the operand reads of the next k-step (NEXT_KSTEP of the tiles at NEXT_A / NEXT_B) into the other buffer,
-  //   * NLOADS global->LDS loads (ISSUE = issue_a or issue_b) of K tile LOAD_KT into stage LOAD_STAGE,
-  //     starting with the wave's LOAD_Q0-th, one after every (TM TN / NLOADS)-th MFMA.
+  //   * NLOADS global->LDS loads of operand IS_B of K tile LOAD_KT into stage LOAD_STAGE, starting with
+  //     the wave's LOAD_Q0-th, one after every (TM TN / NLOADS)-th MFMA.
+  // A wave issues at most one instruction every four cycles, eight per MFMA: every instruction placed
+  // between the MFMAs counts, also the scalar ones, hence the running offsets.
   // The accumulator tile is c^T (operands swapped): a lane owns runs of four consecutive columns
   // of one row of c and can store them as one 8-byte word.
-#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, ISSUE, LOAD_KT, LOAD_STAGE, LOAD_Q0, NLOADS)               \
+#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, IS_B, LOAD_KT, LOAD_STAGE, LOAD_Q0, NLOADS)                \
   do {                                                                                                           \
     constexpr int every_ = (T::TM * T::TN) / (NLOADS);                                                           \
     static_assert(every_ >= 1, "not enough MFMAs per k-step to hide the loads behind");                          \
+    uint32_t sc_ = scalar_off(IS_B, LOAD_KT, LOAD_Q0), dst_ = lds_off(IS_B, LOAD_STAGE, LOAD_Q0);                \
+    const uint32_t sc_step_ = T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                           \
     MBX_WAIT_FRAGS(CUR_BUF);                                                                                     \
     __builtin_amdgcn_sched_barrier(0);                                                                           \
     static_for<T::TM * T::TN>([&](auto mi_) {                                                                    \
@@ -260,7 +289,11 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
       acc[m_ / T::TN][m_ % T::TN] =                                                                              \
           mfma32<DT>(fb[CUR_BUF][m_ % T::TN], fa[CUR_BUF][m_ / T::TN], acc[m_ / T::TN][m_ % T::TN]);             \
       MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                               \
-      if (m_ % every_ == every_ - 1 && m_ / every_ < (NLOADS)) ISSUE(LOAD_KT, LOAD_STAGE, (LOAD_Q0) + m_ / every_); \
+      if (m_ % every_ == every_ - 1 && m_ / every_ < (NLOADS)) {                                                 \
+        issue(IS_B, sc_, dst_);                                                                                  \
+        sc_ += sc_step_;                                                                                         \
+        dst_ += T::WAVES * 1024u;                                                                                \
+      }                                                                                                          \
       __builtin_amdgcn_sched_barrier(0);                                                                         \
     });                                                                                                          \
   } while (0)
@@ -279,15 +312,11 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
     // prologue: tiles 0 .. SB-2, the A part and half of the B part of tile SB-1, then wait for tile 0
 #pragma unroll
     for (int t = 0; t < SB - 1; ++t) {
-#pragma unroll
-      for (int q = 0; q < LA; ++q) issue_a(t, t, q);
-#pragma unroll
-      for (int q = 0; q < LB; ++q) issue_b(t, t, q);
+      issue_group(false, t, t, 0, LA);
+      issue_group(true, t, t, 0, LB);
     }
-#pragma unroll
-    for (int q = 0; q < LA; ++q) issue_a(SB - 1, SB - 1, q);
-#pragma unroll
-    for (int q = 0; q < LB / 2; ++q) issue_b(SB - 1, SB - 1, q);
+    issue_group(false, SB - 1, SB - 1, 0, LA);
+    issue_group(true, SB - 1, SB - 1, 0, LB / 2);
     wait_vmcnt<WAIT_PROLOGUE>();
     __builtin_amdgcn_s_barrier();
     MBX_READ_FRAGS(0, 0, lds_base, lds_base + B_RING);
@@ -298,13 +327,13 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
       const int sa_next = sa == SA - 1 ? 0 : sa + 1, sb_next = sb == SB - 1 ? 0 : sb + 1;
       const uint32_t a_cur = lds_base + (uint32_t)sa * T::A_BYTES, b_cur = lds_base + B_RING + (uint32_t)sb * T::B_BYTES;
       const uint32_t a_nxt = lds_base + (uint32_t)sa_next * T::A_BYTES, b_nxt = lds_base + B_RING + (uint32_t)sb_next * T::B_BYTES;
-      MBX_STEP(0, 1, a_cur, b_cur, issue_b, kt + SB - 1, sb_prev, LB / 2, LB / 2);
-      MBX_STEP(1, 2, a_cur, b_cur, issue_a, kt + SB, sa_prev, 0, LA / 2);
-      MBX_STEP(0, 3, a_cur, b_cur, issue_a, kt + SB, sa_prev, LA / 2, LA / 2);
+      MBX_STEP(0, 1, a_cur, b_cur, true, kt + SB - 1, sb_prev, LB / 2, LB / 2);
+      MBX_STEP(1, 2, a_cur, b_cur, false, kt + SB, sa_prev, 0, LA / 2);
+      MBX_STEP(0, 3, a_cur, b_cur, false, kt + SB, sa_prev, LA / 2, LA / 2);
       MBX_WAIT_FRAGS(1);
       wait_vmcnt<WAIT_LOOP>();
       __builtin_amdgcn_s_barrier();
-      MBX_STEP(1, 0, a_nxt, b_nxt, issue_b, kt + SB, sb, 0, LB / 2);   // past the last tile this reads stale LDS into dead registers
+      MBX_STEP(1, 0, a_nxt, b_nxt, true, kt + SB, sb, 0, LB / 2);   // past the last tile this reads stale LDS into dead registers
       sa = sa_next;
       sb = sb_next;
     }
