@@ -270,18 +270,17 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   // One k-step: TM x TN MFMAs on register buffer CUR_BUF.  Interleaved with them, so that neither
   // the LDS nor the texture-address unit makes the wave wait with the matrix core idle:
   //   * the operand reads of the next k-step (NEXT_KSTEP of the tiles at NEXT_A / NEXT_B) into the other buffer,
-  //   * NLOADS global->LDS loads of operand IS_B of K tile LOAD_KT into stage LOAD_STAGE, starting with
-  //     the wave's LOAD_Q0-th, one after every (TM TN / NLOADS)-th MFMA.
+  //   * NLOADS global->LDS loads of operand IS_B, one after every (TM TN / NLOADS)-th MFMA, at the running
+  //     scalar offset SC into LDS at DST (both advanced here),
+  //   * PREP(), the scalar bookkeeping for the following k-steps, behind one of the later MFMAs.
   // A wave issues at most one instruction every four cycles, eight per MFMA: every instruction placed
-  // between the MFMAs counts, also the scalar ones, hence the running offsets.
+  // between the MFMAs counts, also the scalar ones, and none should be left for the gap between k-steps.
   // The accumulator tile is c^T (operands swapped): a lane owns runs of four consecutive columns
   // of one row of c and can store them as one 8-byte word.
-#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, IS_B, LOAD_KT, LOAD_STAGE, LOAD_Q0, NLOADS)                \
+#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, IS_B, SC, DST, NLOADS, PREP)                               \
   do {                                                                                                           \
     constexpr int every_ = (T::TM * T::TN) / (NLOADS);                                                           \
-    static_assert(every_ >= 1, "not enough MFMAs per k-step to hide the loads behind");                          \
-    uint32_t sc_ = scalar_off(IS_B, LOAD_KT, LOAD_Q0), dst_ = lds_off(IS_B, LOAD_STAGE, LOAD_Q0);                \
-    const uint32_t sc_step_ = T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                           \
+    static_assert(every_ >= 2, "not enough MFMAs per k-step to hide the loads behind");                          \
     MBX_WAIT_FRAGS(CUR_BUF);                                                                                     \
     __builtin_amdgcn_sched_barrier(0);                                                                           \
     static_for<T::TM * T::TN>([&](auto mi_) {                                                                    \
@@ -290,10 +289,11 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
           mfma32<DT>(fb[CUR_BUF][m_ % T::TN], fa[CUR_BUF][m_ / T::TN], acc[m_ / T::TN][m_ % T::TN]);             \
       MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                               \
       if (m_ % every_ == every_ - 1 && m_ / every_ < (NLOADS)) {                                                 \
-        issue(IS_B, sc_, dst_);                                                                                  \
-        sc_ += sc_step_;                                                                                         \
-        dst_ += T::WAVES * 1024u;                                                                                \
+        issue(IS_B, SC, DST);                                                                                    \
+        SC += T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                                           \
+        DST += T::WAVES * 1024u;                                                                                 \
       }                                                                                                          \
+      if (m_ == (T::TM * T::TN) / 2 + 1) PREP();                                                                     \
       __builtin_amdgcn_sched_barrier(0);                                                                         \
     });                                                                                                          \
   } while (0)
@@ -321,21 +321,50 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
     __builtin_amdgcn_s_barrier();
     MBX_READ_FRAGS(0, 0, lds_base, lds_base + B_RING);
 
-    int sa = 0, sb = 0;   // kt % SA, kt % SB
+    // Running state, all scalar.  LDS addresses of the stages being multiplied (tile kt) and of the
+    // next ones; LDS offset and scalar global offset of the A loads of this iteration (tile kt + SB,
+    // stage (kt - 1) % SA) and of the B loads that start in its k-step 3 (tile kt + SB, stage kt % SB).
+    constexpr uint32_t A_RING_END = (uint32_t)SA * T::A_BYTES, B_RING_END = B_RING + (uint32_t)SB * T::B_BYTES;
+    uint32_t a_rd = lds_base, b_rd = lds_base + B_RING, a_rd_next = 0, b_rd_next = 0;
+    uint32_t a_dst0 = lds_off(false, SA - 1, 0), b_dst0 = lds_off(true, 0, 0);
+    uint32_t a_sc0 = (uint32_t)SB * a_step + (uint32_t)wave * a_jstep, b_sc0 = (uint32_t)SB * b_step + (uint32_t)wave * b_jstep;
+    const uint32_t a_dst_end = A_RING_END + (uint32_t)wave * 1024u, b_dst_end = B_RING_END + (uint32_t)wave * 1024u;
+    // the loads in flight: B continues with the second half of tile SB - 1
+    uint32_t sc_b = scalar_off(true, SB - 1, LB / 2), dst_b = lds_off(true, SB - 1, LB / 2), sc_a = 0, dst_a = 0;
+    uint32_t past = 0;
     for (int kt = 0; kt < nk; ++kt) {
-      const int sa_prev = sa == 0 ? SA - 1 : sa - 1, sb_prev = sb == 0 ? SB - 1 : sb - 1;
-      const int sa_next = sa == SA - 1 ? 0 : sa + 1, sb_next = sb == SB - 1 ? 0 : sb + 1;
-      const uint32_t a_cur = lds_base + (uint32_t)sa * T::A_BYTES, b_cur = lds_base + B_RING + (uint32_t)sb * T::B_BYTES;
-      const uint32_t a_nxt = lds_base + (uint32_t)sa_next * T::A_BYTES, b_nxt = lds_base + B_RING + (uint32_t)sb_next * T::B_BYTES;
-      MBX_STEP(0, 1, a_cur, b_cur, true, kt + SB - 1, sb_prev, LB / 2, LB / 2);
-      MBX_STEP(1, 2, a_cur, b_cur, false, kt + SB, sa_prev, 0, LA / 2);
-      MBX_STEP(0, 3, a_cur, b_cur, false, kt + SB, sa_prev, LA / 2, LA / 2);
+      auto prep0 = [&]() {   // the A loads of k-steps 1 and 2
+        past = kt + SB < nk ? 0u : 0x80000000u;
+        sc_a = a_sc0 | past;
+        dst_a = a_dst0;
+      };
+      auto prep1 = [&]() {
+        a_sc0 += a_step;
+        a_dst0 += T::A_BYTES;
+        a_dst0 = a_dst0 >= a_dst_end ? a_dst0 - A_RING_END : a_dst0;
+      };
+      auto prep2 = [&]() {   // the B loads of k-step 3 and of k-step 0 of the next iteration; the next stages to read
+        sc_b = b_sc0 | past;
+        dst_b = b_dst0;
+        a_rd_next = a_rd + T::A_BYTES;
+        a_rd_next = a_rd_next >= lds_base + A_RING_END ? lds_base : a_rd_next;
+        b_rd_next = b_rd + T::B_BYTES;
+        b_rd_next = b_rd_next >= lds_base + B_RING_END ? lds_base + B_RING : b_rd_next;
+      };
+      auto prep3 = [&]() {
+        b_sc0 += b_step;
+        b_dst0 += T::B_BYTES;
+        b_dst0 = b_dst0 >= b_dst_end ? b_dst0 - (uint32_t)SB * T::B_BYTES : b_dst0;
+      };
+      MBX_STEP(0, 1, a_rd, b_rd, true, sc_b, dst_b, LB / 2, prep0);
+      MBX_STEP(1, 2, a_rd, b_rd, false, sc_a, dst_a, LA / 2, prep1);
+      MBX_STEP(0, 3, a_rd, b_rd, false, sc_a, dst_a, LA / 2, prep2);
       MBX_WAIT_FRAGS(1);
       wait_vmcnt<WAIT_LOOP>();
       __builtin_amdgcn_s_barrier();
-      MBX_STEP(1, 0, a_nxt, b_nxt, true, kt + SB, sb, 0, LB / 2);   // past the last tile this reads stale LDS into dead registers
-      sa = sa_next;
-      sb = sb_next;
+      MBX_STEP(1, 0, a_rd_next, b_rd_next, true, sc_b, dst_b, LB / 2, prep3);   // past the last tile this reads stale LDS into dead registers
+      a_rd = a_rd_next;
+      b_rd = b_rd_next;
     }
     wait_vmcnt<0>();   // no load may still be writing LDS when the workgroup's LDS is handed on
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // nor an LDS read still be landing in a register the epilogue reuses
