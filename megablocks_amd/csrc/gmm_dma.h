@@ -252,13 +252,14 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   // m-th operand read (of TM + TN) of k-step KSTEP of the tiles at A_ADDR / B_ADDR into register buffer BUF
 #define MBX_READ_ONE(KSTEP, BUF, A_ADDR, B_ADDR, M)                                                              \
   do {                                                                                                           \
-    if ((M) < T::TM) {                                                                                           \
-      fa[BUF][(M) % T::TM] = A_MC ? read_frag<true, KSTEP>(A_ADDR, fa_off[A_MC ? (M) % T::TM : 0])               \
-                                  : read_frag<false, KSTEP, ((M) % T::TM) * KC_TILE>(A_ADDR, fa_off[0]);         \
-    } else if ((M) < T::TM + T::TN) {                                                                            \
-      fb[BUF][((M) - T::TM) % T::TN] =                                                                           \
-          B_MC ? read_frag<true, KSTEP>(B_ADDR, fb_off[B_MC ? ((M) - T::TM) % T::TN : 0])                        \
-               : read_frag<false, KSTEP, (((M) - T::TM) % T::TN) * KC_TILE>(B_ADDR, fb_off[0]);                  \
+    if constexpr ((M) < T::TM) {                                                                                 \
+      constexpr int i_ = (M);                                                                                    \
+      if constexpr (A_MC) fa[BUF][i_] = read_frag<true, KSTEP>(A_ADDR, fa_off[A_MC ? i_ : 0]);                   \
+      else fa[BUF][i_] = read_frag<false, KSTEP, i_ * KC_TILE>(A_ADDR, fa_off[0]);                               \
+    } else if constexpr ((M) < T::TM + T::TN) {                                                                  \
+      constexpr int j_ = (M) - T::TM;                                                                            \
+      if constexpr (B_MC) fb[BUF][j_] = read_frag<true, KSTEP>(B_ADDR, fb_off[B_MC ? j_ : 0]);                   \
+      else fb[BUF][j_] = read_frag<false, KSTEP, j_ * KC_TILE>(B_ADDR, fb_off[0]);                               \
     }                                                                                                            \
   } while (0)
 #define MBX_READ_FRAGS(KSTEP, BUF, A_ADDR, B_ADDR)                                                               \
