@@ -34,8 +34,8 @@ MEASURED_TRAFFIC = {
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=20)
-    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--config', default='c3', choices=['c1', 'c2', 'c3', 'c4', 'c5'])
     ap.add_argument('--tokens', type=int, default=None, help='override the token count (not the headline number)')
     ap.add_argument('--memory-optimized', action='store_true')
