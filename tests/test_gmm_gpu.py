@@ -22,6 +22,21 @@ def rel_err(a, b):
     return float((a - b).norm() / b.norm().clamp_min(1e-30))
 
 
+def max_block_err(got, ref, bm=64, bn=128):
+    """Largest relative error over bm x bn blocks of the last two dimensions: one wrong piece of one tile
+    shows here even where the error over the whole output would hide it."""
+    got, ref = got.double(), ref.double()
+    r, c = ref.shape[-2:]
+    pr, pc = (-r) % bm, (-c) % bn
+    d = torch.nn.functional.pad(got - ref, (0, pc, 0, pr))
+    b = torch.nn.functional.pad(ref, (0, pc, 0, pr))
+    shape = d.shape[:-2] + ((r + pr) // bm, bm, (c + pc) // bn, bn)
+    num = d.reshape(shape).pow(2).sum(dim=(-3, -1)).sqrt()
+    den = b.reshape(shape).pow(2).sum(dim=(-3, -1)).sqrt()
+    scale = ref.norm() / max(1, num.numel()) ** 0.5              # a typical block norm, for blocks that are almost zero
+    return float((num / torch.maximum(den, scale * 0.1)).max())
+
+
 def _sizes(groups, rows, seed, empty=()):
     g = torch.Generator().manual_seed(seed)
     cuts = torch.sort(torch.randint(0, rows + 1, (groups - 1,), generator=g))[0]
@@ -115,12 +130,14 @@ def test_gmm_benchmark_shapes_vs_fp32(gg, name, groups, rows, hidden, ffn, skew)
     x = torch.randn(rows, hidden, device='cuda').bfloat16()
     w = (torch.randn(groups, ffn, hidden, device='cuda') * 0.02).bfloat16()
     h = gg.backend.gmm(x, w, sizes, trans_b=True)                               # NT
-    assert rel_err(h, _ref_gpu(x, w, sizes, False, True)) < TOL
+    ref = _ref_gpu(x, w, sizes, False, True)
+    assert rel_err(h, ref) < TOL and max_block_err(h, ref) < 2 * TOL
     y = gg.backend.gmm(h, w, sizes)                                             # NN
-    assert rel_err(y, _ref_gpu(h, w, sizes, False, False)) < TOL
+    ref = _ref_gpu(h, w, sizes, False, False)
+    assert rel_err(y, ref) < TOL and max_block_err(y, ref) < 2 * TOL
     dw = gg.backend.gmm(h, x, sizes, trans_a=True)                              # TN
     ref = _ref_gpu(h, x, sizes, True, False)
-    assert rel_err(dw, ref) < TOL
+    assert rel_err(dw, ref) < TOL and max_block_err(dw, ref) < 2 * TOL
     for e, s in enumerate(sizes.tolist()):
         if s == 0:
             assert torch.count_nonzero(dw[e]) == 0
@@ -180,6 +197,33 @@ def test_gmm_ragged_shapes_on_the_pipelined_path(gg, groups, rows, k, n, mode):
         for e, s in enumerate(sizes.tolist()):
             if s == 0:
                 assert torch.count_nonzero(got[e]) == 0
+
+
+SCHEDULES = [  # name, groups, rows, k, n: one case per branch of the device-side tile schedulers
+    ('more than 64 experts, small tile', 80, 24000, 128, 512),
+    ('more than 64 experts, big tile', 72, 28800, 128, 768),
+    ('fewer tiles than compute units, cut in halves', 2, 1000, 256, 2048),
+    ('last round more than half full, not cut', 4, 6400, 128, 2048),
+    ('several full rounds and a cut tail', 8, 9000, 64, 2048),
+    ('TN with two tiles per workgroup', 4, 3000, 512, 768),
+    ('one row per expert', 64, 64, 64, 256),
+]
+
+
+@pytest.mark.parametrize('name,groups,rows,k,n', SCHEDULES)
+def test_gmm_tile_schedules(gg, name, groups, rows, k, n):
+    sizes = _sizes(groups, rows, seed=groups + rows, empty=(1,) if groups > 2 else ())
+    torch.manual_seed(groups)
+    a = torch.randn(rows, k, device='cuda').bfloat16()
+    b_nt = (torch.randn(groups, n, k, device='cuda') * 0.1).bfloat16()
+    b_nn = (torch.randn(groups, k, n, device='cuda') * 0.1).bfloat16()
+    b_tn = torch.randn(rows, n, device='cuda').bfloat16()
+    for b, ta, tb in ((b_nt, False, True), (b_nn, False, False), (b_tn, True, False)):
+        got = gg.backend.gmm(a, b, sizes, trans_a=ta, trans_b=tb)
+        ref = _ref_gpu(a, b, sizes, ta, tb)
+        assert rel_err(got, ref) < TOL and max_block_err(got, ref) < 2 * TOL, (name, ta, tb)
+        again = gg.backend.gmm(a, b, sizes.cuda().int(), trans_a=ta, trans_b=tb)
+        assert torch.equal(again, got)                              # same schedule, same summation order: bit-identical
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
