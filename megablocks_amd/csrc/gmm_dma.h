@@ -404,19 +404,47 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
     constexpr int ROWS_PER_INSTR = kWave / CHUNKS;    // 2 for 256-wide tiles
     const int rl = lane / CHUNKS, ch = lane % CHUNKS;
     const int n = n_base + ch * 8;
-#pragma unroll 4
-    for (int it = wave; it < T::BM / ROWS_PER_INSTR; it += T::WAVES) {
-      const int ml = it * ROWS_PER_INSTR + rl, m = m_base + ml;
-      if (m >= m_lim || n >= n_lim) continue;
-      const u32x4 v = *(const __attribute__((address_space(3))) u32x4*)(lds + ml * ROW + ch * 16);
-      uint16_t* dst = c + (int64_t)m * ldc + n;
-      if (n + 8 <= n_lim) {
-        *(u32x4*)dst = v;
+    // Eight LDS reads in flight before the first store of a batch (inline asm: the compiler would sink
+    // each read to its store, behind the row check).  Like the main loop this part is bound by
+    // instruction issue: a tile that is complete in the column direction takes a path with a 32-bit
+    // running byte offset and nothing but the row check around each store.
+    constexpr int ITERS = T::BM / ROWS_PER_INSTR / T::WAVES, BATCH = 8;
+    constexpr int ROW_STEP = T::WAVES * ROWS_PER_INSTR;   // rows between consecutive stores of a wave
+    static_assert(ITERS % BATCH == 0, "store batches");
+    const uint32_t rd_addr = lds_base + (uint32_t)((wave * ROWS_PER_INSTR + rl) * ROW + ch * 16);
+    const bool full_n = n_base + T::BN <= n_lim;          // uniform
+    int m = m_base + wave * ROWS_PER_INSTR + rl;
+    uint32_t off = ((uint32_t)m * (uint32_t)ldc + (uint32_t)n) * 2u;   // outputs are below 2 GiB
+    const uint32_t off_step = (uint32_t)ROW_STEP * (uint32_t)ldc * 2u;
+    char* const cb = (char*)c;
+#pragma unroll 1
+    for (int b = 0; b < ITERS; b += BATCH) {
+      u32x4 v[BATCH];
+      static_for<BATCH>([&](auto ui) {
+        constexpr int u = decltype(ui)::value;
+        v[u] = lds_read_b128<u * ROW_STEP * ROW>(rd_addr + (uint32_t)(b * ROW_STEP * ROW));
+      });
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+      if (full_n) {
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+          if (m + u * ROW_STEP < m_lim) *(u32x4*)(cb + (off + (uint32_t)u * off_step)) = v[u];
       } else {
 #pragma unroll
-        for (int t = 0; t < 8; ++t)
-          if (n + t < n_lim) dst[t] = (uint16_t)(v[t >> 1] >> ((t & 1) * 16));
+        for (int u = 0; u < BATCH; ++u) {
+          if (m + u * ROW_STEP >= m_lim || n >= n_lim) continue;
+          uint16_t* dst = (uint16_t*)(cb + (off + (uint32_t)u * off_step));
+          if (n + 8 <= n_lim) {
+            *(u32x4*)dst = v[u];
+          } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+              if (n + t < n_lim) dst[t] = (uint16_t)(v[u][t >> 1] >> ((t & 1) * 16));
+          }
+        }
       }
+      m += BATCH * ROW_STEP;
+      off += BATCH * off_step;
     }
   } else {
     const bool n_vec = (ldc % 4 == 0) && (((uintptr_t)c & 7u) == 0);
