@@ -32,6 +32,7 @@ enum mbx_layout { MBX_NN = 0, MBX_NT = 1, MBX_TN = 2 };
 #define MBX_EINVAL (-1)   /* bad enum / negative size / null pointer */
 #define MBX_ESCRATCH (-2) /* scratch buffer too small */
 #define MBX_ERANGE (-3)   /* size beyond what the kernels index with 32 bits */
+#define MBX_EUNSUPPORTED (-4) /* this entry point does not handle the shape / type; use the general form */
 
 /* Human-readable text for a return code (static storage). */
 const char* mbx_error_string(int code);
@@ -140,6 +141,17 @@ int mbx_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t
  * written (NN / NT). */
 int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bins,
             int num_groups, int64_t rows, int k, int n, int layout, mbx_stream_t stream);
+
+/* The input gradient of the GLU experts, megablocks/layers/glu.py:160-166
+ * (`gmm(dsdd_out, w1, c=dx); dx += gmm(dv1_out, v1)`), as one reduction over both operand pairs:
+ *   MBX_NN: c[r_e] = a[r_e] @ b[e] + a2[r_e] @ b2[e]      MBX_NT: ... @ b[e]^T + ... @ b2[e]^T
+ * with a2 / b2 shaped like a / b.  One rounding of the fp32 sum instead of the reference's three.
+ * Handles bf16 / f16 with k a multiple of 64 and at least 256, 16-byte aligned operands (n a multiple
+ * of 8 for MBX_NN) below 2 GiB each; anything else returns MBX_EUNSUPPORTED and the caller issues the
+ * two mbx_gmm calls and the addition itself. */
+int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype,
+                 const int32_t* bins, int num_groups, int64_t rows, int k, int n, int layout,
+                 mbx_stream_t stream);
 
 /* megablocks/layers/gelu.py:9-13 `_gelu_backward_inplace(g, x)`: g *= d/dx gelu_tanh(x). */
 int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel,

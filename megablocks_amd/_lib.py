@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, 'libmbx.so')
 I16, I32, I64 = 0, 1, 2
 BF16, F16, F32 = 0, 1, 2
 NN, NT, TN = 0, 1, 2
+EINVAL, ESCRATCH, ERANGE, EUNSUPPORTED = -1, -2, -3, -4
 
 ITYPE = {torch.int16: I16, torch.int32: I32, torch.int64: I64}
 DTYPE = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
@@ -37,6 +38,7 @@ _SIGNATURES = {
     'mbx_binned_scatter': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _sz, _vp]),
     'mbx_binned_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _vp]),
     'mbx_gmm': (_i, [_vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
+    'mbx_gmm_dual': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gelu_backward_inplace': (_i, [_vp, _vp, _i, _i64, _vp]),
     'mbx_glu_forward': (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp]),
     'mbx_glu_backward': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _vp]),
@@ -118,6 +120,10 @@ class record:
             self.ev0 = torch.cuda.Event(enable_timing=True)
             self.ev0.record()
         return self
+
+    def cancel(self):
+        """Drop this launch from the profile (the call turned out not to launch the kernel it names)."""
+        self.ev0 = None
 
     def __exit__(self, *exc):
         if self.ev0 is not None:

@@ -459,11 +459,15 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
 
 // Launch of the direct-to-LDS kernels (k a multiple of 64 for NN / NT, operands below 2 GiB).
 // TS is the tile the tail of an NN / NT launch is cut into (TS = T: never cut).
+// a2 / b2 non-null (NN / NT only): c = a @ b[e] + a2 @ b2[e], the second pair shaped like the first.
 template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
-            int layout, hipStream_t s) {
+            int layout, hipStream_t s, const void* a2 = nullptr, const void* b2 = nullptr) {
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
+  const uint16_t* ap2 = (const uint16_t*)a2;
+  const uint16_t* bp2 = (const uint16_t*)b2;
+  const bool dual = a2 != nullptr;
   uint16_t* cp = (uint16_t*)c;
   static_assert(T::BN == 256, "the [k][cols] LDS layout of a strided operand is written for 256-column tiles");
   if (layout == MBX_TN) {
@@ -486,17 +490,19 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
   if (tiles > 0x7fffffff) return MBX_ERANGE;
   const unsigned grid = (unsigned)persistent_grid(tiles);
+#define MBX_LAUNCH_ROWS(B_MC, DUAL)                                                                   \
+  do {                                                                                                \
+    auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL>;                                          \
+    int rc = allow_lds(kern, lds);                                                                    \
+    if (rc) return rc;                                                                                \
+    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2);  \
+  } while (0)
   if (layout == MBX_NT) {
-    auto kern = dma::gmm_rows_kernel<DT, false, T, TS>;
-    int rc = allow_lds(kern, lds);
-    if (rc) return rc;
-    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
+    if (dual) MBX_LAUNCH_ROWS(false, true); else MBX_LAUNCH_ROWS(false, false);
   } else {
-    auto kern = dma::gmm_rows_kernel<DT, true, T, TS>;
-    int rc = allow_lds(kern, lds);
-    if (rc) return rc;
-    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n);
+    if (dual) MBX_LAUNCH_ROWS(true, true); else MBX_LAUNCH_ROWS(true, false);
   }
+#undef MBX_LAUNCH_ROWS
   return launch_status();
 }
 
@@ -565,6 +571,30 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     case MBX_F16: return gmm_generic<MBX_F16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
     default: return gmm_generic<MBX_F32>(a, b, c, bins, num_groups, rows, k, n, layout, s);
   }
+}
+
+int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype, const int32_t* bins,
+                 int num_groups, int64_t rows, int k, int n, int layout, mbx_stream_t stream) {
+  if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
+  if (layout != MBX_NN && layout != MBX_NT) return MBX_EINVAL;
+  if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
+  if (num_groups == 0 || rows == 0 || n == 0) return 0;
+  if (!bins || !c || (k > 0 && (!a || !b || !a2 || !b2))) return MBX_EINVAL;
+  if (rows > 0x7fffffff) return MBX_ERANGE;
+  // only the direct-to-LDS kernels reduce over two operand pairs: whole K tiles, at least four per pair
+  const int64_t lim = (int64_t)1 << 31;
+  const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(a2) && aligned16(b2) &&
+                  k % TileDma::BK == 0 && k >= 4 * TileDma::BK && (layout == MBX_NT || n % 8 == 0) &&
+                  rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
+  if (!ok) return MBX_EUNSUPPORTED;
+  hipStream_t s = as_stream(stream);
+  const bool small_m = rows <= (int64_t)num_groups * 320;
+  if (small_m) {
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+    return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+  }
+  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+  return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
 }
 
 int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel, mbx_stream_t stream) {

@@ -172,12 +172,16 @@ struct Args {
   __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b;  // out-of-range bytes read as zero
   uint32_t a_ld_bytes, b_ld_bytes;
   int a_r0, b_r0;                         // tile origin (row of a KC operand / column of an MC operand)
-  int nk;                                 // number of 32-wide K tiles
+  int nk;                                 // number of K tiles
+  // A product of two operand pairs, a @ b + a2 @ b2 (same shapes and pitches): K tiles nk1 .. nk-1 come
+  // from the second pair.  Used only by the DUAL instantiations.
+  __amdgpu_buffer_rsrc_t rsrc_a2, rsrc_b2;
+  int nk1;
 };
 
 // acc (+)= A_tile * B_tile over all K tiles, then c[m][n] = acc for m < m_lim, n < n_lim, where
 // m = m_base + (row inside the tile) and n = n_base + (column inside the tile).
-template <int DT, bool A_MC, bool B_MC, typename T>
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
 __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
                                            int n_base, int n_lim, char* lds_generic) {
   const lds_ptr lds = (lds_ptr)lds_generic;
@@ -208,19 +212,20 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   // reads, which keeps the loop and its vmcnt bookkeeping uniform.
   constexpr uint32_t A_ROWS = A_MC ? 2u : (uint32_t)(1024 / (BK * 2)), B_ROWS = B_MC ? 2u : (uint32_t)(1024 / (BK * 2));
   const uint32_t a_jstep = A_ROWS * g.a_ld_bytes, b_jstep = B_ROWS * g.b_ld_bytes;
-  auto scalar_off = [&](bool is_b, int kt, int q) -> uint32_t {
+  auto scalar_off = [&](bool is_b, int kt, int q) -> uint32_t {   // prologue: K tiles of the first operand pair
     const uint32_t j = (uint32_t)(wave + q * T::WAVES);
     const uint32_t v = is_b ? (uint32_t)kt * b_step + j * b_jstep : (uint32_t)kt * a_step + j * a_jstep;
     return v | (kt < g.nk ? 0u : 0x80000000u);
   };
+  __amdgpu_buffer_rsrc_t ra = g.rsrc_a, rb = g.rsrc_b;   // the operand pair the loads being issued read
   auto lds_off = [&](bool is_b, int stage, int q) -> uint32_t {
     return (is_b ? B_RING + (uint32_t)stage * T::B_BYTES : (uint32_t)stage * T::A_BYTES) + (uint32_t)(wave + q * T::WAVES) * 1024u;
   };
   auto issue = [&](bool is_b, uint32_t sc, uint32_t dst) {
     if (is_b) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_b, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(b_lane + sc), 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(b_lane + sc), 0, 0, 0);
     } else {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(g.rsrc_a, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(a_lane + sc), 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(a_lane + sc), 0, 0, 0);
     }
   };
   auto issue_group = [&](bool is_b, int kt, int stage, int q0, int count) {   // prologue
@@ -338,22 +343,24 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
         past = kt + SB < nk ? 0u : 0x80000000u;
         sc_a = a_sc0 | past;
         dst_a = a_dst0;
+        if (DUAL) ra = kt + SB >= g.nk1 ? g.rsrc_a2 : g.rsrc_a;
       };
       auto prep1 = [&]() {
-        a_sc0 += a_step;
+        a_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * a_jstep : a_sc0 + a_step;   // K tile kt + SB + 1
         a_dst0 += T::A_BYTES;
         a_dst0 = a_dst0 >= a_dst_end ? a_dst0 - A_RING_END : a_dst0;
       };
       auto prep2 = [&]() {   // the B loads of k-step 3 and of k-step 0 of the next iteration; the next stages to read
         sc_b = b_sc0 | past;
         dst_b = b_dst0;
+        if (DUAL) rb = kt + SB >= g.nk1 ? g.rsrc_b2 : g.rsrc_b;
         a_rd_next = a_rd + T::A_BYTES;
         a_rd_next = a_rd_next >= lds_base + A_RING_END ? lds_base : a_rd_next;
         b_rd_next = b_rd + T::B_BYTES;
         b_rd_next = b_rd_next >= lds_base + B_RING_END ? lds_base + B_RING : b_rd_next;
       };
       auto prep3 = [&]() {
-        b_sc0 += b_step;
+        b_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * b_jstep : b_sc0 + b_step;
         b_dst0 += T::B_BYTES;
         b_dst0 = b_dst0 >= b_dst_end ? b_dst0 - (uint32_t)SB * T::B_BYTES : b_dst0;
       };
@@ -565,10 +572,13 @@ struct RowTiles {
 // T is the main tile.  When the last round would leave at least half of the compute units idle, its
 // R tiles are cut into 2 R half tiles of TS (BM / 2 rows, same columns), spread over all XCDs:
 // the tail then costs little more than half a round.  TS = T switches this off.
-template <int DT, bool B_MC, typename T, typename TS>
+// DUAL: c = a @ b[e] + a2 @ b2[e] in one pass (k is the reduction length of each pair, at least
+// (SB + 1) K tiles), as one reduction over 2 k.
+template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
-                const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n) {
+                const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
+                const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "tail tile");
   constexpr bool kSplit = T::BM != TS::BM;
@@ -585,7 +595,9 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   g.rsrc_a = make_rsrc(a, (uint32_t)(rows * k * 2));
   g.a_ld_bytes = (uint32_t)k * 2;
   g.b_ld_bytes = (uint32_t)(B_MC ? n : k) * 2;
-  g.nk = k / T::BK;
+  g.nk1 = k / T::BK;
+  g.nk = DUAL ? 2 * g.nk1 : g.nk1;
+  g.rsrc_a2 = DUAL ? make_rsrc(a2, (uint32_t)(rows * k * 2)) : g.rsrc_a;
   for (int r = 0; r < big_rounds; ++r) {
     const int id = (r * kXcds + xcd) * run + member;
     if (id >= total) break;
@@ -593,8 +605,9 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     tiles.find(id, e, start, end, tm, tn);
     g.a_r0 = start + tm * T::BM;
     g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
+    g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
     g.b_r0 = tn * T::BN;
-    block_gemm<DT, false, B_MC, T>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+    block_gemm<DT, false, B_MC, T, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
     tile_done();
   }
   if (kSplit && split) {
@@ -605,8 +618,9 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
       g.a_r0 = start + tm * T::BM + (j & 1) * TS::BM;
       if (g.a_r0 < end) {
         g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
+        g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
         g.b_r0 = tn * TS::BN;
-        block_gemm<DT, false, B_MC, TS>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+        block_gemm<DT, false, B_MC, TS, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
       }
     }
   }

@@ -89,12 +89,12 @@ int histogram_impl(const T* x, int64_t rows, int64_t n, int num_bins, int32_t* o
   const int64_t total = rows * (int64_t)num_bins;
   if (num_bins <= kHistLdsBins) {
     const size_t lds = (size_t)num_bins * sizeof(int32_t);
-    if (n <= (int64_t)kHistThreads * 256) {  // one block per row writes its counts directly
+    if (n <= (int64_t)kHistThreads * 8) {  // one block per row writes its counts directly
       histogram_kernel<T, true><<<dim3(1, (unsigned)rows), kHistThreads, lds, s>>>(x, n, num_bins, nbits, n > 0 ? n : 1, out);
       return launch_status();
     }
     fill_i32_kernel<<<(unsigned)(ceil_div(total, 256) < 1024 ? ceil_div(total, 256) : 1024), 256, 0, s>>>(out, total, 0);
-    const int64_t chunk = (int64_t)kHistThreads * 64;
+    const int64_t chunk = (int64_t)kHistThreads * 8;
     const int64_t blocks = ceil_div(n, chunk);
     if (blocks > 0x7fffffff) return MBX_ERANGE;
     histogram_kernel<T, false><<<dim3((unsigned)blocks, (unsigned)rows), kHistThreads, lds, s>>>(x, n, num_bins, nbits, chunk, out);
@@ -271,7 +271,7 @@ int sort_impl(const T* x, int64_t n, int end_bit, T* keys_out, T* perm_out, void
     T* kout = to_final ? keys_out : tmp_keys;
     T* vout = to_final ? perm_out : tmp_vals;
     radix_count_kernel<T><<<nblocks, kSortThreads, 0, s>>>(kin, n, shift, mask, pass_bits, counts, nblocks);
-    exclusive_scan_i32_kernel<<<1, 1024, 0, s>>>(counts, (int64_t)kRadix * nblocks);
+    exclusive_scan_i32_kernel<<<1, 1024, 0, s>>>(counts, ((int64_t)1 << pass_bits) * nblocks);   // digit-major: digits the pass cannot produce come last
     if (p == 0)
       radix_scatter_kernel<T, true><<<nblocks, kSortThreads, 0, s>>>(kin, nullptr, n, shift, mask, pass_bits, counts, nblocks, kout, vout);
     else
@@ -379,6 +379,7 @@ const char* mbx_error_string(int code) {
   if (code == MBX_EINVAL) return "mbx: invalid argument";
   if (code == MBX_ESCRATCH) return "mbx: scratch buffer missing or too small";
   if (code == MBX_ERANGE) return "mbx: size out of the supported range";
+  if (code == MBX_EUNSUPPORTED) return "mbx: shape or type not handled by this entry point";
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mbx: unknown error";
 }

@@ -88,6 +88,39 @@ def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None):
     return c
 
 
+def gmm_dual(a, b, a2, b2, batch_sizes, trans_b=False, c=None):
+    """out[r_e] = a[r_e] @ b[e] + a2[r_e] @ b2[e] (`trans_b`: both weights transposed), a2 / b2 shaped like a / b:
+    the input gradient of the GLU experts (glu.py:160-166) as one reduction over both pairs.  Shapes the
+    single-launch kernel does not take are computed as two `gmm` calls and an addition."""
+    _lib.require_cuda(a, b, a2, b2, c)
+    if a.shape != a2.shape or b.shape != b2.shape or a.dtype != a2.dtype or b.dtype != b2.dtype:
+        raise ValueError('gmm_dual: the two operand pairs must have the same shapes and dtypes')
+    if a.ndim != 2 or b.ndim != 3 or a.dtype != b.dtype:
+        raise ValueError('gmm_dual: a must be [rows, k] and b [num_groups, ., .] of the same dtype')
+    a, b, a2, b2 = a.contiguous(), b.contiguous(), a2.contiguous(), b2.contiguous()
+    bins = _device_bins(batch_sizes, a.device)
+    groups, rows, k = bins.shape[0], a.shape[0], a.shape[1]
+    n, layout = (b.shape[1], _lib.NT) if trans_b else (b.shape[2], _lib.NN)
+    if b.shape[0] != groups or (b.shape[2] if trans_b else b.shape[1]) != k:
+        raise ValueError('gmm_dual: b does not match a and batch_sizes')
+    if c is None:
+        c = torch.empty((rows, n), dtype=a.dtype, device=a.device)
+    elif tuple(c.shape) != (rows, n) or c.dtype != a.dtype or not c.is_contiguous():
+        raise ValueError('gmm_dual: c has the wrong shape, dtype or layout')
+    with torch.cuda.device_of(a), _lib.record('gmm_nt_dual' if trans_b else 'gmm_nn_dual', rows=rows, k=2 * k, n=n,
+                                              elem=a.element_size(), groups=groups) as rec:
+        rc = lib.mbx_gmm_dual(_lib.ptr(a), _lib.ptr(b), _lib.ptr(a2), _lib.ptr(b2), _lib.ptr(c), _lib.dtype_of(a),
+                              _lib.ptr(bins), groups, rows, k, n, layout, _lib.stream())
+        if rc == _lib.EUNSUPPORTED:
+            rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        gmm(a, b, batch_sizes, trans_b=trans_b, c=c)
+        c += gmm(a2, b2, batch_sizes, trans_b=trans_b)
+        return c
+    _lib.check(rc, 'gmm_dual')
+    return c
+
+
 class GroupedGemm(torch.autograd.Function):
     """Differentiable gmm(a, b, batch_sizes, trans_b): da = gmm(dc, b, trans_b flipped),
     db = the per-group outer product (trans_a)."""

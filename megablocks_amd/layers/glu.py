@@ -82,6 +82,31 @@ def gated_activation(activation_fn, a, b):
     return activation_fn(a) * b
 
 
+class GLUProjection(torch.autograd.Function):
+    """(x @ w1[e]^T, x @ v1[e]^T) per expert, glu.py:201-203.  Equivalent to two `gg.ops.gmm` calls, except that
+    the input gradient da @ w1 + db @ v1 is one reduction over both pairs instead of two products and a sum."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
+    def forward(ctx, x, w1, v1, batch_sizes):
+        ctx.save_for_backward(x, w1, v1, batch_sizes)
+        return (gg.backend.gmm(x, w1, batch_sizes, trans_b=True), gg.backend.gmm(x, v1, batch_sizes, trans_b=True))
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
+    def backward(ctx, d1, d2):
+        x, w1, v1, batch_sizes = ctx.saved_tensors
+        d1, d2 = d1.contiguous(), d2.contiguous()
+        dx = dw1 = dv1 = None
+        if ctx.needs_input_grad[0]:
+            dx = gg.gmm_dual(d1, w1, d2, v1, batch_sizes)
+        if ctx.needs_input_grad[1]:
+            dw1 = gg.backend.gmm(d1, x, batch_sizes, trans_a=True)
+        if ctx.needs_input_grad[2]:
+            dv1 = gg.backend.gmm(d2, x, batch_sizes, trans_a=True)
+        return dx, dw1, dv1, None
+
+
 class MemoryOptimizedGroupedGLU(torch.autograd.Function):
     """glu.py:66-167: saves (x, sdd_out, v1_out), recomputes the gated activation in backward."""
 
@@ -137,8 +162,7 @@ class MemoryOptimizedGroupedGLU(torch.autograd.Function):
 
         dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
         dv1 = gg.backend.gmm(dv1_out, x, batch_sizes, trans_a=True)
-        dx = gg.backend.gmm(dsdd_out, w1, batch_sizes, c=ddsd_out)
-        dx += gg.backend.gmm(dv1_out, v1, batch_sizes)
+        dx = gg.gmm_dual(dsdd_out, w1, dv1_out, v1, batch_sizes, c=ddsd_out)   # reuses the ddsd_out allocation
         return dx, dw1, dv1, dw2, None, None
 
 
@@ -164,8 +188,7 @@ class SparseGLU(SparseMLP):
                 raise NotImplementedError(
                     'Memory optimized implementation not yet supported with GLU with sparse kernels.')
             return memory_optimized_grouped_glu(x, w1, v1, w2, batch_sizes, self.args.activation_fn)
-        x1 = gg.ops.gmm(x, w1, batch_sizes, trans_b=True)
-        x2 = gg.ops.gmm(x, v1, batch_sizes, trans_b=True)
+        x1, x2 = GLUProjection.apply(x, w1, v1, batch_sizes)
         x1 = gated_activation(self.args.activation_fn, x1, x2)
         return gg.ops.gmm(x1, w2, batch_sizes)
 

@@ -226,6 +226,36 @@ def test_gmm_tile_schedules(gg, name, groups, rows, k, n):
         assert torch.equal(again, got)                              # same schedule, same summation order: bit-identical
 
 
+DUAL = [  # groups, rows, k, n, single launch expected
+    (8, 4000, 512, 1024, True), (3, 700, 256, 264, True), (64, 16384, 1408, 2048, True), (70, 21000, 256, 512, True),
+    (4, 1000, 192, 256, False), (2, 300, 100, 36, False), (1, 64, 256, 8, True),
+]
+
+
+@pytest.mark.parametrize('groups,rows,k,n,single', DUAL)
+@pytest.mark.parametrize('trans_b', [False, True])
+def test_gmm_dual_is_the_sum_of_two_products(gg, groups, rows, k, n, single, trans_b):
+    from megablocks_amd import _lib
+    sizes = _sizes(groups, rows, seed=rows + k, empty=(1,) if groups > 2 else ())
+    torch.manual_seed(k)
+    a, a2 = (torch.randn(rows, k, device='cuda').bfloat16() for _ in range(2))
+    shape = (groups, n, k) if trans_b else (groups, k, n)
+    b, b2 = ((torch.randn(shape, device='cuda') * 0.1).bfloat16() for _ in range(2))
+    ref = _ref_gpu(a, b, sizes, False, trans_b) + _ref_gpu(a2, b2, sizes, False, trans_b)
+    _lib.profile_hook = []
+    try:
+        got = gg.gmm_dual(a, b, a2, b2, sizes, trans_b=trans_b)
+        names = [r[0] for r in _lib.profile_hook]
+    finally:
+        _lib.profile_hook = None
+    assert (names == ['gmm_nt_dual' if trans_b else 'gmm_nn_dual']) == single   # else: two products and a sum
+    assert got.dtype == torch.bfloat16 and rel_err(got, ref) < TOL and max_block_err(got, ref) < 2 * TOL
+    c = torch.full((rows, n), 5.0, device='cuda').bfloat16()
+    assert gg.gmm_dual(a, b, a2, b2, sizes.cuda().int(), trans_b=trans_b, c=c) is c and torch.equal(c, got)
+    with pytest.raises(ValueError):
+        gg.gmm_dual(a, b, a2[:, :-8], b2, sizes, trans_b=trans_b)
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize('act_name', ['silu', 'gelu_tanh'])
 def test_fused_gated_activation_matches_the_two_step_formulation(dtype, act_name):
