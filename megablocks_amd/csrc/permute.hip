@@ -64,13 +64,19 @@ __device__ __forceinline__ void wave_copy_row(const typename Elem<DT>::type* __r
       }
       for (; c < nvec; c += kWave) d[c] = s[c];
     } else {
-      for (int c = lane; c < nvec; c += kWave) {
+      auto scaled_vec = [&](const u32x4& v) {
         float f[E];
-        Vec16<DT>::unpack(s[c], f);
+        Vec16<DT>::unpack(v, f);
 #pragma unroll
         for (int i = 0; i < E; ++i) f[i] *= scale;
-        d[c] = Vec16<DT>::pack(f);
+        return Vec16<DT>::pack(f);
+      };
+      int c = lane;
+      for (; c + 3 * kWave < nvec; c += 4 * kWave) {
+        const u32x4 v0 = s[c], v1 = s[c + kWave], v2 = s[c + 2 * kWave], v3 = s[c + 3 * kWave];
+        d[c] = scaled_vec(v0); d[c + kWave] = scaled_vec(v1); d[c + 2 * kWave] = scaled_vec(v2); d[c + 3 * kWave] = scaled_vec(v3);
       }
+      for (; c < nvec; c += kWave) d[c] = scaled_vec(s[c]);
     }
   } else {
     for (int c = lane; c < hidden; c += kWave)
@@ -101,13 +107,20 @@ __device__ __forceinline__ float wave_dot_row(const typename Elem<DT>::type* __r
     const int nvec = hidden / E;
     const u32x4* av = (const u32x4*)a;
     const u32x4* bv = (const u32x4*)b;
-    for (int c = lane; c < nvec; c += kWave) {
+    auto dot_vec = [&](const u32x4& va, const u32x4& vb) {
       float fa[E], fb[E];
-      Vec16<DT>::unpack(av[c], fa);
-      Vec16<DT>::unpack(bv[c], fb);
+      Vec16<DT>::unpack(va, fa);
+      Vec16<DT>::unpack(vb, fb);
 #pragma unroll
       for (int i = 0; i < E; ++i) acc += fa[i] * fb[i];
+    };
+    int c = lane;
+    for (; c + 3 * kWave < nvec; c += 4 * kWave) {
+      const u32x4 a0 = av[c], a1 = av[c + kWave], a2 = av[c + 2 * kWave], a3 = av[c + 3 * kWave];
+      const u32x4 b0 = bv[c], b1 = bv[c + kWave], b2 = bv[c + 2 * kWave], b3 = bv[c + 3 * kWave];
+      dot_vec(a0, b0); dot_vec(a1, b1); dot_vec(a2, b2); dot_vec(a3, b3);
     }
+    for (; c < nvec; c += kWave) dot_vec(av[c], bv[c]);
   } else {
     for (int c = lane; c < hidden; c += kWave) acc += Elem<DT>::to_f32(a[c]) * Elem<DT>::to_f32(b[c]);
   }
@@ -187,7 +200,10 @@ __global__ void fill_kernel(int32_t* __restrict__ p, int64_t n, int32_t v) {
 // out[t] = sum_j round(x[inv[t*k+j]] * w[t*k+j]); one wave per token.  Each product is
 // rounded to the storage type before the fp32 sum, as the reference's scaled copy into a
 // [tokens, top_k, hidden] buffer followed by sum(dim=1) does.
-template <int DT, bool VEC>
+// BATCH: how many of a token's expert rows are kept in flight together (2, 4 or 8: a larger batch costs
+// registers, i.e. resident waves, which the short top_k <= 2 cases need more); top_k > BATCH takes the
+// one-row-at-a-time loop.
+template <int DT, bool VEC, int BATCH>
 __global__ void __launch_bounds__(kRowThreads)
 combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ inv,
                const void* __restrict__ weights, int w_dtype, void* __restrict__ out_) {
@@ -205,7 +221,43 @@ combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_
       wave_copy_row<DT, VEC>(x + (int64_t)row * hidden, dst, hidden, weights != nullptr, scale);
       continue;
     }
-    if (VEC) {
+    if (VEC && top_k <= BATCH) {
+      // Lane j resolves expert j of the token (row in x, router weight); the wave then has the loads of all
+      // top_k rows in flight for every 16-byte column instead of one after the other.
+      constexpr int EV = Vec16<DT>::kElems;
+      const int nvec = hidden / EV;
+      const int my_row = lane < top_k ? inv[s0 + lane] : -1;
+      const float my_scale = (weights && lane < top_k) ? load_as_f32(weights, s0 + lane, w_dtype) : 1.f;
+      const u32x4* src[BATCH];
+      float scale[BATCH];
+      bool live[BATCH];
+#pragma unroll
+      for (int j = 0; j < BATCH; ++j) {
+        const int row = __shfl(my_row, j, kWave);
+        live[j] = row >= 0;
+        src[j] = (const u32x4*)(x + (int64_t)(live[j] ? row : 0) * hidden);
+        scale[j] = __shfl(my_scale, j, kWave);
+      }
+      for (int c = lane; c < nvec; c += kWave) {
+        u32x4 v[BATCH];
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j)
+          if (live[j]) v[j] = src[j][c];
+        float acc[EV];
+#pragma unroll
+        for (int i = 0; i < EV; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+          if (!live[j]) continue;
+          float f[EV];
+          Vec16<DT>::unpack(v[j], f);
+#pragma unroll
+          for (int i = 0; i < EV; ++i)
+            acc[i] += weights ? Elem<DT>::to_f32(Elem<DT>::from_f32(f[i] * scale[j])) : f[i];
+        }
+        ((u32x4*)dst)[c] = Vec16<DT>::pack(acc);
+      }
+    } else if (VEC) {
       constexpr int EV = Vec16<DT>::kElems;
       const int nvec = hidden / EV;
       for (int c = lane; c < nvec; c += kWave) {
@@ -383,7 +435,12 @@ int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
   fill_kernel<<<fb, 256, 0, s>>>(inv, n_slots, -1);
   inverse_map_kernel<<<(unsigned)ceil_div(n_slots, 256), 256, 0, s>>>(indices, bin_ids, bins, padded_bins, num_bins, (int)n_slots, inv);
   const bool vec = can_vec(dtype, hidden, x, out);
-#define CALL(DT, V) combine_kernel<DT, V><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out)
+#define CALL(DT, V)                                                                                                             \
+  do {                                                                                                                          \
+    if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
+    else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
+    else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
+  } while (0)
   MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
 #undef CALL
   return launch_status();
@@ -449,7 +506,12 @@ int mbx_binned_scatter(const void* x, int dtype, int64_t tokens, int hidden, int
   const int rc = binned_inverse(indices, bins, num_bins, capacity, n_slots, inv, s);
   if (rc) return rc;
   const bool vec = can_vec(dtype, hidden, x ? x : out, out);
-#define CALL(DT, V) combine_kernel<DT, V><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out)
+#define CALL(DT, V)                                                                                                             \
+  do {                                                                                                                          \
+    if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
+    else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
+    else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
+  } while (0)
   MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
 #undef CALL
   return launch_status();
