@@ -414,7 +414,8 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
     // Eight LDS reads in flight before the first store of a batch (inline asm: the compiler would sink
     // each read to its store, behind the row check).  Like the main loop this part is bound by
     // instruction issue: a tile that is complete in the column direction takes a path with a 32-bit
-    // running byte offset and nothing but the row check around each store.
+    // running byte offset and nothing but the row check around each store.  Those stores are
+    // non-temporal: the output is not read again by this kernel and need not displace operand panels.
     constexpr int ITERS = T::BM / ROWS_PER_INSTR / T::WAVES, BATCH = 8;
     constexpr int ROW_STEP = T::WAVES * ROWS_PER_INSTR;   // rows between consecutive stores of a wave
     static_assert(ITERS % BATCH == 0, "store batches");
@@ -435,7 +436,7 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
       if (full_n) {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u)
-          if (m + u * ROW_STEP < m_lim) *(u32x4*)(cb + (off + (uint32_t)u * off_step)) = v[u];
+          if (m + u * ROW_STEP < m_lim) __builtin_nontemporal_store(v[u], (u32x4*)(cb + (off + (uint32_t)u * off_step)));
       } else {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) {
