@@ -276,8 +276,8 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   // One k-step: TM x TN MFMAs on register buffer CUR_BUF.  Interleaved with them, so that neither
   // the LDS nor the texture-address unit makes the wave wait with the matrix core idle:
   //   * the operand reads of the next k-step (NEXT_KSTEP of the tiles at NEXT_A / NEXT_B) into the other buffer,
-  //   * NLOADS global->LDS loads of operand IS_B, one after every (TM TN / NLOADS)-th MFMA, at the running
-  //     scalar offset SC into LDS at DST (both advanced here),
+  //   * NLOADS global->LDS loads of operand IS_B at the running scalar offset SC into LDS at DST (both
+  //     advanced here),
   //   * PREP(), the scalar bookkeeping for the following k-steps, behind one of the later MFMAs.
   // A wave issues at most one instruction every four cycles, eight per MFMA: every instruction placed
   // between the MFMAs counts, also the scalar ones, and none should be left for the gap between k-steps.
@@ -285,21 +285,26 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   // of one row of c and can store them as one 8-byte word.
 #define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, IS_B, SC, DST, NLOADS, PREP)                               \
   do {                                                                                                           \
-    constexpr int every_ = (T::TM * T::TN) / (NLOADS);                                                           \
+    /* The operand reads go behind the first TM + TN MFMAs; with 16 MFMAs per k-step the loads go behind   */  \
+    /* every second MFMA of the other half and the bookkeeping between them, so that no MFMA has more than */  \
+    /* a handful of instructions queued behind it.  With 8 MFMAs per k-step the loads are spread over all. */  \
+    constexpr int n_ = T::TM * T::TN, half_ = n_ / 2;                                                            \
+    constexpr bool late_ = half_ >= T::TM + T::TN && half_ / (NLOADS) >= 2;                                      \
+    constexpr int every_ = (late_ ? half_ : n_) / (NLOADS), first_ = late_ ? half_ : 0;                          \
     static_assert(every_ >= 2, "not enough MFMAs per k-step to hide the loads behind");                          \
     MBX_WAIT_FRAGS(CUR_BUF);                                                                                     \
     __builtin_amdgcn_sched_barrier(0);                                                                           \
-    static_for<T::TM * T::TN>([&](auto mi_) {                                                                    \
+    static_for<n_>([&](auto mi_) {                                                                               \
       constexpr int m_ = decltype(mi_)::value;                                                                   \
       acc[m_ / T::TN][m_ % T::TN] =                                                                              \
           mfma32<DT>(fb[CUR_BUF][m_ % T::TN], fa[CUR_BUF][m_ / T::TN], acc[m_ / T::TN][m_ % T::TN]);             \
       MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                               \
-      if (m_ % every_ == every_ - 1 && m_ / every_ < (NLOADS)) {                                                 \
+      if (m_ >= first_ && (m_ - first_) % every_ == every_ - 1 && (m_ - first_) / every_ < (NLOADS)) {           \
         issue(IS_B, SC, DST);                                                                                    \
         SC += T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                                           \
         DST += T::WAVES * 1024u;                                                                                 \
       }                                                                                                          \
-      if (m_ == (T::TM * T::TN) / 2 + 1) PREP();                                                                     \
+      if (m_ == (late_ ? n_ - 4 : half_ + 1)) PREP();                                                            \
       __builtin_amdgcn_sched_barrier(0);                                                                         \
     });                                                                                                          \
   } while (0)
