@@ -190,12 +190,6 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
 
   f32x16 acc[T::TM][T::TN];
-#pragma unroll
-  for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-    for (int j = 0; j < T::TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   constexpr int BK = T::BK, SA = T::SA, SB = T::SB, LA = T::LA, LB = T::LB;
   static_assert(T::KS == 4, "the schedule below is written for four k-steps per K tile");
@@ -310,16 +304,24 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   } while (0)
 
   const int nk = g.nk;
+  auto clear_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  };
+  // Iteration kt multiplies K tile kt (A stage kt % SA, B stage kt % SB) and issues, spread evenly
+  // over its four k-steps:
+  //   k-step 0: the second half of B tile kt + SB - 1 -> B stage (kt - 1) % SB   (free since the barrier of kt - 1)
+  //   k-steps 1, 2: the halves of A tile kt + SB      -> A stage (kt - 1) % SA   (likewise)
+  //   barrier: every wave has tile kt in registers and tile kt + 1 has landed
+  //   k-step 3: the first half of B tile kt + SB      -> B stage kt % SB         (free since that barrier)
+  // Loads complete in order, so "tile kt + 1 has landed" is "at most WAIT_LOOP of my loads in flight".
+  constexpr int WAIT_PROLOGUE = (SB - 2) * (LA + LB) + LA + LB / 2;
+  constexpr int WAIT_LOOP = (SB - 1) * LA + (SB - 2) * LB;
   if (nk > 0) {
-    // Iteration kt multiplies K tile kt (A stage kt % SA, B stage kt % SB) and issues, spread evenly
-    // over its four k-steps:
-    //   k-step 0: the second half of B tile kt + SB - 1 -> B stage (kt - 1) % SB   (free since the barrier of kt - 1)
-    //   k-steps 1, 2: the halves of A tile kt + SB      -> A stage (kt - 1) % SA   (likewise)
-    //   barrier: every wave has tile kt in registers and tile kt + 1 has landed
-    //   k-step 3: the first half of B tile kt + SB      -> B stage kt % SB         (free since that barrier)
-    // Loads complete in order, so "tile kt + 1 has landed" is "at most WAIT_LOOP of my loads in flight".
-    constexpr int WAIT_PROLOGUE = (SB - 2) * (LA + LB) + LA + LB / 2;
-    constexpr int WAIT_LOOP = (SB - 1) * LA + (SB - 2) * LB;
     // prologue: tiles 0 .. SB-2, the A part and half of the B part of tile SB-1, then wait for tile 0
 #pragma unroll
     for (int t = 0; t < SB - 1; ++t) {
@@ -328,6 +330,10 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
     }
     issue_group(false, SB - 1, SB - 1, 0, LA);
     issue_group(true, SB - 1, SB - 1, 0, LB / 2);
+  }
+  __builtin_amdgcn_sched_barrier(0);   // the loads are on their way before the accumulators are cleared
+  clear_acc();
+  if (nk > 0) {
     wait_vmcnt<WAIT_PROLOGUE>();
     __builtin_amdgcn_s_barrier();
     MBX_READ_FRAGS(0, 0, lds_base, lds_base + B_RING);
