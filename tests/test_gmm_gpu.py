@@ -226,6 +226,40 @@ def test_gmm_tile_schedules(gg, name, groups, rows, k, n):
         assert torch.equal(again, got)                              # same schedule, same summation order: bit-identical
 
 
+def _random_shapes(count, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    shapes = []
+    for i in range(count):
+        groups, rows = r(1, 70), r(1, 5000)
+        if i % 3 == 0:      # the pipelined kernels: k a multiple of 64
+            k, n = 64 * r(1, 17), 8 * r(1, 140)
+        elif i % 3 == 1:    # the register-staged kernels: multiples of 8
+            k, n = 8 * r(1, 140), 8 * r(1, 140)
+        else:               # anything
+            k, n = r(1, 600), r(1, 600)
+        shapes.append((groups, rows, k, n))
+    return shapes
+
+
+@pytest.mark.parametrize('groups,rows,k,n', _random_shapes(36, seed=7))
+def test_gmm_random_shapes_with_canaries(gg, groups, rows, k, n):
+    sizes = _sizes(groups, rows, seed=groups * 7 + rows, empty=(0,) if groups > 3 else ())
+    torch.manual_seed(rows)
+    a = torch.randn(rows, k, device='cuda').bfloat16()
+    for mode in ('nn', 'nt', 'tn'):
+        if mode == 'tn':
+            b = torch.randn(rows, n, device='cuda').bfloat16()
+        else:
+            b = (torch.randn((groups, n, k) if mode == 'nt' else (groups, k, n), device='cuda') * 0.1).bfloat16()
+        ref = _ref_gpu(a, b, sizes, mode == 'tn', mode == 'nt')
+        guard = torch.full((ref.numel() + 4096,), 3.0, device='cuda').bfloat16()       # canary around the output
+        c = guard[2048:2048 + ref.numel()].view(ref.shape)
+        got = gg.backend.gmm(a, b, sizes, trans_a=mode == 'tn', trans_b=mode == 'nt', c=c)
+        assert rel_err(got, ref) < TOL and max_block_err(got, ref) < 2 * TOL, mode
+        assert bool((guard[:2048] == 3.0).all()) and bool((guard[2048 + ref.numel():] == 3.0).all()), mode
+
+
 DUAL = [  # groups, rows, k, n, single launch expected
     (8, 4000, 512, 1024, True), (3, 700, 256, 264, True), (64, 16384, 1408, 2048, True), (70, 21000, 256, 512, True),
     (4, 1000, 192, 256, False), (2, 300, 100, 36, False), (1, 64, 256, 8, True),
