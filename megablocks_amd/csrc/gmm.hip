@@ -316,8 +316,18 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
 
 #include "gmm_dma.h"
 
-// ---- fallback for shapes the MFMA path does not take (odd sizes, fp32) ----------------
-// c(m, n) = sum_r a(m, r) b(r, n) with arbitrary element strides; 32x32 tile, fp32 FMA.
+// ---- any shape, any alignment, fp32 included ------------------------------------------
+// c(m, n) = sum_r a(m, r) b(r, n) with element-wise addressing and bounds checks, the products and sums
+// in fp32 on the matrix cores (v_mfma_f32_32x32x2_f32 is an IEEE fp32 multiply-add; 16-bit inputs are
+// widened exactly).  128 x 128 tile per workgroup, four waves of 64 x 64, K tiles of 16 staged through a
+// double-buffered LDS tile [k][128 + 36] per operand (the MFMA wants one k per lane half, 32 consecutive
+// rows / columns across the lanes: conflict-free reads).  The next K tile is fetched into registers while
+// the current one is multiplied.
+constexpr int kGenTile = 128, kGenBK = 16;
+// row pitch of the LDS tiles in floats: 36 mod 64 banks apart, so that the 16 k-rows x 4 columns a wave stores
+// and the two k-rows x 32 columns a wave reads per instruction fall into (nearly) distinct banks
+constexpr int kGenLd = kGenTile + 36;
+
 template <int DT>
 __global__ void __launch_bounds__(256)
 gmm_generic_kernel(const void* __restrict__ a_, const void* __restrict__ b_, void* __restrict__ c_,
@@ -326,48 +336,98 @@ gmm_generic_kernel(const void* __restrict__ a_, const void* __restrict__ b_, voi
   const E* a = (const E*)a_;
   const E* b = (const E*)b_;
   E* c = (E*)c_;
-  __shared__ float as[32][33], bs[32][33];
+  __shared__ float as[2][kGenBK][kGenLd], bs[2][kGenBK][kGenLd];
   const int e = blockIdx.z;
   const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
-  const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;  // 32 x 8
   int m_dim, r_begin, r_end;
   if (layout == MBX_TN) { m_dim = k; r_begin = start; r_end = end; }
   else { m_dim = end - start; r_begin = 0; r_end = k; }
-  const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+  const int m0 = blockIdx.y * kGenTile, n0 = blockIdx.x * kGenTile;
   if (m0 >= m_dim) return;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int r0 = r_begin; r0 < r_end; r0 += 32) {
-    for (int i = ty; i < 32; i += 8) {
-      const int m = m0 + i, r = r0 + tx;   // as[i][tx] = a(m, r)
-      float va = 0.f, vb = 0.f;
-      if (m < m_dim && r < r_end)
-        va = Elem<DT>::to_f32(layout == MBX_TN ? a[(int64_t)r * k + m] : a[(int64_t)(start + m) * k + r]);
-      const int rr = r0 + i, nn = n0 + tx;  // bs[i][tx] = b(rr, nn)
-      if (rr < r_end && nn < n) {
-        if (layout == MBX_TN) vb = Elem<DT>::to_f32(b[(int64_t)rr * n + nn]);
-        else if (layout == MBX_NN) vb = Elem<DT>::to_f32(b[((int64_t)e * k + rr) * n + nn]);
-        else vb = Elem<DT>::to_f32(b[((int64_t)e * n + nn) * k + rr]);
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
+
+  // Each thread fetches 8 elements of each operand tile; consecutive threads walk the dimension that is
+  // contiguous in memory (the reduction index r for a in NN / NT and b in NT, else the row / column).
+  const bool a_r_fast = layout != MBX_TN, b_r_fast = layout == MBX_NT;
+  const int a_t0 = a_r_fast ? tid / kGenBK : tid % kGenTile, a_r = a_r_fast ? tid % kGenBK : tid / kGenTile;
+  const int b_t0 = b_r_fast ? tid / kGenBK : tid % kGenTile, b_r = b_r_fast ? tid % kGenBK : tid / kGenTile;
+  // step of the tile index / of r between a thread's 8 elements
+  const int a_ts = a_r_fast ? 256 / kGenBK : 0, a_rs = a_r_fast ? 0 : 256 / kGenTile;
+  const int b_ts = b_r_fast ? 256 / kGenBK : 0, b_rs = b_r_fast ? 0 : 256 / kGenTile;
+  auto a_at = [&](int m, int r) -> float {
+    if (m >= m_dim || r >= r_end) return 0.f;
+    return Elem<DT>::to_f32(layout == MBX_TN ? a[(int64_t)r * k + m] : a[(int64_t)(start + m) * k + r]);
+  };
+  auto b_at = [&](int r, int nn) -> float {
+    if (r >= r_end || nn >= n) return 0.f;
+    if (layout == MBX_TN) return Elem<DT>::to_f32(b[(int64_t)r * n + nn]);
+    if (layout == MBX_NN) return Elem<DT>::to_f32(b[((int64_t)e * k + r) * n + nn]);
+    return Elem<DT>::to_f32(b[((int64_t)e * n + nn) * k + r]);
+  };
+  float ra[8], rb[8];
+  auto fetch = [&](int r0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      ra[i] = a_at(m0 + a_t0 + i * a_ts, r0 + a_r + i * a_rs);
+      rb[i] = b_at(r0 + b_r + i * b_rs, n0 + b_t0 + i * b_ts);
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      as[buf][a_r + i * a_rs][a_t0 + i * a_ts] = ra[i];
+      bs[buf][b_r + i * b_rs][b_t0 + i * b_ts] = rb[i];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  fetch(r_begin);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int r0 = r_begin; r0 < r_end; r0 += kGenBK) {
+    const bool more = r0 + kGenBK < r_end;
+    if (more) fetch(r0 + kGenBK);
+#pragma unroll
+    for (int kk = 0; kk < kGenBK; kk += 2) {
+      float fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa[i] = as[buf][kk + lane / 32][wm + i * 32 + lane % 32];
+        fb[i] = bs[buf][kk + lane / 32][wn + i * 32 + lane % 32];
       }
-      as[i][tx] = va;
-      bs[i][tx] = vb;
-    }
-    __syncthreads();
-#pragma unroll 8
-    for (int r = 0; r < 32; ++r) {
-      const float bv = bs[r][tx];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) acc[q] += as[ty + 8 * q][r] * bv;
-    }
-    __syncthreads();
-  }
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int m = m0 + ty + 8 * q, nn = n0 + tx;
-    if (m < m_dim && nn < n) {
-      if (layout == MBX_TN) c[((int64_t)e * k + m) * n + nn] = Elem<DT>::from_f32(acc[q]);
-      else c[(int64_t)(start + m) * n + nn] = Elem<DT>::from_f32(acc[q]);
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
   }
+  // register r of lane l of a 32 x 32 product: row (r / 4) * 8 + (l / 32) * 4 + r % 4, column l % 32
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int nn = n0 + wn + j * 32 + lane % 32;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + i * 32 + (r / 4) * 8 + (lane / 32) * 4 + r % 4;
+        if (m < m_dim && nn < n) {
+          if (layout == MBX_TN) c[((int64_t)e * k + m) * n + nn] = Elem<DT>::from_f32(acc[i][j][r]);
+          else c[(int64_t)(start + m) * n + nn] = Elem<DT>::from_f32(acc[i][j][r]);
+        }
+      }
+    }
 }
 
 // ---- GELU backward, in place ---------------------------------------------------------
@@ -511,7 +571,7 @@ int gmm_generic(const void* a, const void* b, void* c, const int32_t* bins, int 
                 int layout, hipStream_t s) {
   // The row count of a group is only known on the device: size the grid for the worst case.
   const int64_t m_bound = layout == MBX_TN ? k : rows;
-  const int64_t gy = ceil_div(m_bound, 32), gx = ceil_div(n, 32);
+  const int64_t gy = ceil_div(m_bound, kGenTile), gx = ceil_div(n, kGenTile);
   if (gy > 65535 || num_groups > 65535) return MBX_ERANGE;
   if (gy == 0 || gx == 0) return 0;
   gmm_generic_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)num_groups), 256, 0, s>>>(a, b, c, bins, layout, k, n);
