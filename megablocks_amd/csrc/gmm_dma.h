@@ -1,4 +1,5 @@
-// Grouped-GEMM main loop with direct-to-LDS global loads and an LDS ring of K tiles.
+// Grouped-GEMM main loop with direct-to-LDS global loads and LDS rings of K tiles, and the kernels
+// that walk the tiles of a launch with it.
 //
 // Included by gmm.hip (uses its u32x4 / f32x16 types, mfma32, pack2 and the XCD tile mapping).
 //
@@ -138,18 +139,6 @@ __device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t 
     const int k3 = (2 * (wave & 1) + kl) & 3;                     // (2j + kl) & 3 with j = wave (mod 2)
     const int c = ((((pc >> 1) ^ (2 * k3)) << 1) | (pc & 1));
     return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
-  }
-}
-
-template <bool MC, int BK, int INSTRS, int WAVES>
-__device__ __forceinline__ void issue_operand(__amdgpu_buffer_rsrc_t rsrc, lds_ptr tile, int wave, uint32_t lane_off,
-                                              uint32_t tile_off, uint32_t ld_bytes) {
-  constexpr uint32_t ROWS = MC ? 2u : (uint32_t)(1024 / (BK * 2));   // global rows covered by one instruction
-#pragma unroll
-  for (int q = 0; q < INSTRS / WAVES; ++q) {
-    const int j = wave + q * WAVES;
-    const uint32_t off = lane_off + tile_off + (uint32_t)j * ROWS * ld_bytes;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(tile + j * 1024), 16, (int)off, 0, 0, 0);
   }
 }
 
