@@ -6,7 +6,10 @@ that the HIP kernels can be checked against it; nothing in ``megablocks_amd``
 imports it, and only ``tests/``, ``__graft_entry__.smoke()`` and the
 ``cpu_baseline`` leg of ``bench.py`` may call it.
 
-Every function cites the reference file:line whose behaviour it restates.
+Every function cites the reference file:line whose behaviour it restates.  The integer routing ops exist
+twice: as torch code (``oracle/routing.py``) and as plain C (``oracle/routing_c.c``, bound by
+``oracle/routing_c.py``, compiled with gcc by ``__graft_entry__.build()``); the tests hold the two
+against each other.
 The reference itself (Python + CUDA/CUB + Triton + two un-vendored packages,
 ``grouped_gemm==0.3.0`` and ``stanford-stk==0.7.1``) can neither be imported nor
 compiled in this environment, so there is no ``oracle/_ref`` build.

@@ -292,3 +292,26 @@ def test_full_size_round_trip_properties(ops):
     half = torch.full((T * k,), 0.5, device='cuda').bfloat16()
     back = ops.scatter(g, indices, bin_ids, half, bins, k)                         # 0.5 x + 0.5 x == x exactly
     assert torch.equal(back, x)
+
+
+# ------------------------------------------------------------------ the routing chain against the C oracle
+@pytest.mark.parametrize('tokens,experts,top_k', [(8192, 8, 2), (16384, 64, 1), (32768, 64, 6), (24576, 16, 4), (7, 3, 2)])
+def test_routing_chain_matches_the_c_restatement(ops, tokens, experts, top_k):
+    """sort -> histogram -> cumsum -> round_up -> cumsum as the layer runs them (moe.py:152-183,
+    dmoe.py:131-154), at the token counts of the benchmark workloads, bit for bit against oracle/routing_c.c."""
+    import os
+    import shutil
+    from oracle import routing_c
+    if not os.path.exists(routing_c.LIB_PATH) and shutil.which('gcc') is None:
+        pytest.skip('oracle/liboracle_routing.so is not built and there is no gcc')
+    g = torch.Generator().manual_seed(tokens + experts)
+    top = torch.randint(0, experts, (tokens * top_k,), dtype=torch.int32, generator=g)
+    end_bit = oracle.routing.sort_end_bit(experts)
+    want_idx, want_ids, want_bins, want_pbins, want_tpe = routing_c.route(top, experts, end_bit, 128)
+    t = top.cuda()
+    bin_ids, indices = ops.sort(t, end_bit)
+    tpe = ops.histogram(t, experts)
+    bins = ops.inclusive_cumsum(tpe, 0).view(-1)
+    pbins = ops.inclusive_cumsum(ops.round_up(tpe, 128), 0).view(-1)
+    for got, want in ((indices, want_idx), (bin_ids, want_ids), (tpe, want_tpe), (bins, want_bins), (pbins, want_pbins)):
+        assert got.dtype == torch.int32 and torch.equal(got.cpu(), want)

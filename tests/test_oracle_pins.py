@@ -7,6 +7,7 @@ oracle; invariants (permutation validity, linearity, adjointness, dense-matmul
 equivalence) cover what the loops leave open.
 """
 import itertools
+import os
 
 import numpy as np
 import pytest
@@ -399,3 +400,52 @@ def test_dmoe_single_expert_is_dense_ffn():
     out, _ = oracle.dmoe_forward(x, ew, ei, w1, w2, num_experts=1, top_k=1)
     want = torch.nn.functional.gelu(x @ w1.t(), approximate='tanh') @ w2
     assert torch.allclose(out, want, atol=1e-5)
+
+
+# ---------------------------------------------------------------------------------------------
+# The plain-C restatement of the integer routing ops (oracle/routing_c.c) against the torch one:
+# two independent restatements of the same reference lines must agree bit for bit.
+@pytest.fixture(scope='module')
+def rc():
+    import shutil
+    from oracle import routing_c
+    if not os.path.exists(routing_c.LIB_PATH) and shutil.which('gcc') is None:
+        pytest.skip('oracle/liboracle_routing.so is not built and there is no gcc')
+    routing_c.lib()
+    return routing_c
+
+
+@pytest.mark.parametrize('dtype', [torch.int16, torch.int32, torch.int64])
+def test_c_oracle_sort_histogram_cumsum(rc, dtype):
+    g = torch.Generator().manual_seed(11)
+    width = {torch.int16: 16, torch.int32: 32, torch.int64: 64}[dtype]
+    for n in (0, 1, 2, 63, 64, 1000):
+        x = torch.randint(-70, 70, (n,), dtype=dtype, generator=g)
+        for end_bit in (None, 0, 1, 3, 7, width - 1, width):
+            k1, p1 = oracle.sort(x, end_bit)
+            k2, p2 = rc.sort(x, end_bit)
+            assert torch.equal(k1, k2) and torch.equal(p1, p2), (n, end_bit)
+    h = torch.randint(-3, 12, (5, 257), dtype=dtype, generator=g)
+    for bins in (1, 9, 64):
+        assert torch.equal(oracle.histogram(h, bins), rc.histogram(h, bins))
+        assert torch.equal(oracle.histogram(h[0], bins), rc.histogram(h[0], bins))
+    c = torch.randint(0, 100, (4, 77), dtype=dtype, generator=g)
+    assert torch.equal(oracle.inclusive_cumsum(c, 1), rc.cumsum(c, False))
+    assert torch.equal(oracle.exclusive_cumsum(c, 1), rc.cumsum(c, True))
+
+
+def test_c_oracle_topology_replicate_route(rc):
+    g = torch.Generator().manual_seed(12)
+    pb = torch.tensor([256, 256, 640, 1024, 1024], dtype=torch.int32)
+    for rows in (8, 10):                       # fewer / more block-rows than the bins cover
+        assert torch.equal(oracle.topology(pb, 128, rows, 6), rc.topology(pb, 128, rows, 6))
+    x = torch.randint(0, 9, (3, 4), dtype=torch.int32, generator=g)
+    bins = torch.tensor([2, 2, 7, 9], dtype=torch.int32)
+    for cols in (9, 12):
+        assert torch.equal(oracle.replicate(x, bins, cols), rc.replicate(x, bins, cols))
+    for experts in (1, 8, 64):
+        te = torch.randint(0, experts, (777,), dtype=torch.int32, generator=g)
+        want = oracle.indices_and_padded_bins(te, experts, 128)
+        got = rc.route(te, experts, oracle.routing.sort_end_bit(experts), 128)
+        for w, t in zip(want, got):
+            assert torch.equal(w.view(-1), t.view(-1))
