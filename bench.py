@@ -118,9 +118,17 @@ def summarize(w, agg, slots_scale):
         launches = len(d['ms'])
         if name.startswith('gmm'):
             flops = 2.0 * m['rows'] * slots_scale * m['k'] * m['n']
+            # algorithmic bytes of the launch: every operand and the output once
+            pairs = 2 if name.endswith('_dual') else 1
+            kk = m['k'] / pairs
+            nbytes = (pairs * (m['rows'] * slots_scale * kk + m['groups'] * kk * m['n']) + m['rows'] * slots_scale * m['n']) \
+                * m['elem'] if not name.startswith('gmm_tn') else \
+                (m['rows'] * slots_scale * (m['k'] + m['n']) + m['groups'] * m['k'] * m['n']) * m['elem']
             gemm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, flops_per_launch=flops,
                               tflops=round(flops / (avg_ms * 1e-3) / 1e12, 1),
-                              frac_of_mfma_peak=round(flops / (avg_ms * 1e-3) / MFMA_PEAK[dn], 4))
+                              frac_of_mfma_peak=round(flops / (avg_ms * 1e-3) / MFMA_PEAK[dn], 4),
+                              bytes_per_launch=nbytes, gbps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
+                              frac_of_hbm_peak=round(nbytes / (avg_ms * 1e-3) / HBM_PEAK, 4))
         else:
             nbytes = float(w.tokens + w.slots) * m['hidden'] * m['elem']
             perm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, bytes_per_launch=nbytes,
@@ -203,9 +211,16 @@ def main():
     gemm_ms = sum(g['avg_ms'] * g['launches'] for g in gemm.values()) / args.steps
     perm_ms = sum(p['avg_ms'] * p['launches'] for p in perm.values()) / args.steps
     dom_name, dom = max(gemm.items(), key=lambda kv: kv[1]['avg_ms'] * kv[1]['launches'])
-    roofline = dict(bound='mfma', kernel=dom_name, achieved=dom['tflops'], peak=MFMA_PEAK[dn] / 1e12, unit='TFLOP/s',
-                    frac=dom['frac_of_mfma_peak'], traffic=MEASURED_TRAFFIC.get((w.name, dom_name)),
-                    flops_per_launch=dom['flops_per_launch'], avg_launch_ms=dom['avg_ms'])
+    # The kernel is bound by whichever roofline its arithmetic intensity puts lower (the ridge of the part is
+    # MFMA peak / HBM peak = 312 FLOP per byte in bf16): c2's 256-row experts stream their weights.
+    if dom['flops_per_launch'] / dom['bytes_per_launch'] >= MFMA_PEAK[dn] / HBM_PEAK:
+        roofline = dict(bound='mfma', kernel=dom_name, achieved=dom['tflops'], peak=MFMA_PEAK[dn] / 1e12, unit='TFLOP/s',
+                        frac=dom['frac_of_mfma_peak'], traffic=MEASURED_TRAFFIC.get((w.name, dom_name)),
+                        flops_per_launch=dom['flops_per_launch'], avg_launch_ms=dom['avg_ms'])
+    else:
+        roofline = dict(bound='hbm', kernel=dom_name, achieved=dom['gbps'], peak=HBM_PEAK / 1e9, unit='GB/s',
+                        frac=dom['frac_of_hbm_peak'], traffic=MEASURED_TRAFFIC.get((w.name, dom_name)),
+                        bytes_per_launch=dom['bytes_per_launch'], avg_launch_ms=dom['avg_ms'])
     all_gemm_tflops = w.gemm_flops() / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None
 
     out = {
