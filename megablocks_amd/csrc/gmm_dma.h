@@ -17,8 +17,8 @@
 //     at chunk position c ^ swz(r), swz(r) = (r >> 1) & 7 for 128-byte rows (BK 64) and
 //     (r >> 2) & 3 for 64-byte rows (BK 32), so that the 16 lanes a ds_read_b128 serves per cycle
 //     (16 consecutive rows, same chunk) touch 16 distinct 16-byte bank groups of the 64-bank LDS.
-//   MC operand (reduction dim strided): [k][256 cols] = 512-byte rows, 32-byte pair p of row k
-//     stored at pair position p ^ (2 (k & 3)), so that the 32 lanes a ds_read_b64_tr_b16 serves per
+//   MC operand (reduction dim strided): [k][R cols] = 2 R-byte rows (R = 256 or 128), 32-byte pair p of
+//     row k stored at pair position p ^ (2 (k & 3)), so that the 32 lanes a ds_read_b64_tr_b16 serves per
 //     cycle (4 k-rows x two adjacent 32-byte pairs) touch 8 distinct pairs of a 256-byte bank line.
 // A wave-wide load instruction fills 1 KiB of LDS in lane order, so the swizzle is applied by
 // choosing which global address each lane fetches.  The reads of these tiles are inline asm: the
@@ -35,9 +35,10 @@ namespace dma {
 // B load can be (the B stage to refill is still being read), so that global -> LDS loads leave the
 // compute unit at an even rate: the texture-address unit takes some 20 cycles per wave-wide load, is
 // shared by the four waves, and a wave whose load has to queue cannot issue its next MFMA either.
-template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_>
+// WGS: workgroups meant to share a compute unit (its LDS and registers are split between them).
+template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_, int WGS_ = 1>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1, WGS = WGS_;
   static constexpr int KS = BK / 16;                                           // MFMA k-steps per tile
   static constexpr int WAVES = WM * WN, THREADS = WAVES * kWave;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -48,7 +49,8 @@ struct Tile {
   static constexpr size_t RING_BYTES = (size_t)SA * A_BYTES + (size_t)SB * B_BYTES, EPILOGUE_BYTES = (size_t)BM * (BN * 2 + 16);
   static constexpr size_t LDS_BYTES = RING_BYTES > EPILOGUE_BYTES ? RING_BYTES : EPILOGUE_BYTES;
   static_assert(BK == 64, "K tile");
-  static_assert(SB >= 2 && LDS_BYTES <= 160 * 1024, "LDS rings");
+  static_assert(SB >= 2 && LDS_BYTES * WGS <= 160 * 1024, "LDS rings");
+  static_assert((BM == 256 || BM == 128) && (BN == 256 || BN == 128), "tile widths the strided-operand LDS layout knows");
   static_assert(A_INSTRS % WAVES == 0 && B_INSTRS % WAVES == 0, "loads must split evenly over the waves");
   static_assert(LA % 2 == 0 && LB % 2 == 0, "the loads of an operand tile are issued in two halves");
   static_assert(WAVES % 2 == 0, "the swizzles need the parity of a wave's load index to be fixed");
@@ -88,8 +90,9 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
 }
 
 // Per-lane byte offset (inside an operand tile) of the MFMA operand of the 32 rows/cols starting
-// at `r`, k-step 0.  KC: k-step s is the same address with bits 5.. XORed by 32 s.  MC: +8192 s.
-template <bool MC, int BK>
+// at `r`, k-step 0.  KC: k-step s is the same address with bits 5.. XORed by 32 s.  MC: 16 rows (of
+// COLS columns) further per k-step.
+template <bool MC, int BK, int COLS>
 __device__ __forceinline__ uint32_t frag_lane_offset(int r) {
   const int lane = lane_id();
   if (!MC) {
@@ -100,18 +103,18 @@ __device__ __forceinline__ uint32_t frag_lane_offset(int r) {
     const int g = lane >> 4, s = lane & 15;
     const int k = (g >> 1) * 8 + (s >> 2);
     const int pair = (r >> 4) + (g & 1);
-    return (uint32_t)(k * 512 + ((pair ^ (2 * ((s >> 2) & 3))) << 5) + ((s & 3) << 3));
+    return (uint32_t)(k * (COLS * 2) + ((pair ^ (2 * ((s >> 2) & 3))) << 5) + ((s & 3) << 3));
   }
 }
 
 // IMM: constant byte offset of the 32-row tile inside a KC operand tile (goes into the instruction).
-template <bool MC, int KS, int IMM = 0>
+template <bool MC, int KS, int IMM = 0, int COLS = 256>
 __device__ __forceinline__ u32x4 read_frag(uint32_t tile_addr, uint32_t lane_off) {
   if (!MC) {
     return lds_read_b128<IMM>(tile_addr + (lane_off ^ (KS * 32)));
   } else {
-    const u32x2 lo = lds_read_tr16_b64<KS * 8192>(tile_addr + lane_off);
-    const u32x2 hi = lds_read_tr16_b64<KS * 8192 + 2048>(tile_addr + lane_off);
+    const u32x2 lo = lds_read_tr16_b64<KS * 16 * COLS * 2>(tile_addr + lane_off);
+    const u32x2 hi = lds_read_tr16_b64<KS * 16 * COLS * 2 + 4 * COLS * 2>(tile_addr + lane_off);
     u32x4 v;
     v[0] = lo[0]; v[1] = lo[1]; v[2] = hi[0]; v[3] = hi[1];
     return v;
@@ -121,7 +124,7 @@ __device__ __forceinline__ u32x4 read_frag(uint32_t tile_addr, uint32_t lane_off
 // ---- global -> LDS ----
 // Byte offset (from the operand's buffer base) fetched by this lane in the wave's first load of
 // tile 0; `r0` is the tile origin in the non-reduction dimension, `ld_bytes` the row pitch.
-template <bool MC, int BK>
+template <bool MC, int BK, int COLS>
 __device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t ld_bytes) {
   const int lane = lane_id();
   if (!MC) {
@@ -134,10 +137,15 @@ __device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t 
       const int c = pc ^ ((row >> 2) & 3);
       return (uint32_t)(r0 + row) * ld_bytes + (uint32_t)(c << 4);
     }
-  } else {           // 2 k-rows x 32 chunks per instruction; instruction j holds k = 2j, 2j + 1
+  } else if (COLS == 256) {   // 2 k-rows x 32 chunks per instruction; instruction j holds k = 2j, 2j + 1
     const int kl = lane >> 5, pc = lane & 31;
     const int k3 = (2 * (wave & 1) + kl) & 3;                     // (2j + kl) & 3 with j = wave (mod 2)
     const int c = ((((pc >> 1) ^ (2 * k3)) << 1) | (pc & 1));
+    return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
+  } else {                    // 128 columns: 4 k-rows x 16 chunks per instruction; instruction j holds k = 4j .. 4j + 3
+    static_assert(!MC || COLS == 256 || COLS == 128, "strided operand tile width");
+    const int kl = lane >> 4, pc = lane & 15;
+    const int c = ((((pc >> 1) ^ (2 * kl)) << 1) | (pc & 1));
     return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
   }
 }
@@ -151,6 +159,8 @@ __device__ __forceinline__ void wait_frags(u32x4 (&a)[NA], u32x4 (&b)[NB]) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
   } else if constexpr (NA == 4 && NB == 2) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]));
+  } else if constexpr (NA == 2 && NB == 2) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]));
   } else {
     static_for<NA>([&](auto i) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[decltype(i)::value])); });
     static_for<NB>([&](auto i) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(b[decltype(i)::value])); });
@@ -183,8 +193,8 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   constexpr int BK = T::BK, SA = T::SA, SB = T::SB, LA = T::LA, LB = T::LB;
   static_assert(T::KS == 4, "the schedule below is written for four k-steps per K tile");
   constexpr uint32_t B_RING = (uint32_t)SA * T::A_BYTES;   // the B stages follow the A stages
-  const uint32_t a_lane = load_lane_offset<A_MC, BK>(wave, g.a_r0, g.a_ld_bytes);
-  const uint32_t b_lane = load_lane_offset<B_MC, BK>(wave, g.b_r0, g.b_ld_bytes);
+  const uint32_t a_lane = load_lane_offset<A_MC, BK, T::BM>(wave, g.a_r0, g.a_ld_bytes);
+  const uint32_t b_lane = load_lane_offset<B_MC, BK, T::BN>(wave, g.b_r0, g.b_ld_bytes);
   const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
   const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
   // The q-th wave-wide load of this wave's share of an operand tile is load number j = wave + q WAVES
@@ -193,7 +203,7 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   // kt a_step + j a_jstep.  A tile index at or past nk gets bit 31 set in the scalar part (operands are
   // below 2 GiB): the load is then out of range, fetches nothing and writes zeros into a stage nobody
   // reads, which keeps the loop and its vmcnt bookkeeping uniform.
-  constexpr uint32_t A_ROWS = A_MC ? 2u : (uint32_t)(1024 / (BK * 2)), B_ROWS = B_MC ? 2u : (uint32_t)(1024 / (BK * 2));
+  constexpr uint32_t A_ROWS = (uint32_t)(1024 / ((A_MC ? T::BM : BK) * 2)), B_ROWS = (uint32_t)(1024 / ((B_MC ? T::BN : BK) * 2));   // operand rows per load
   const uint32_t a_jstep = A_ROWS * g.a_ld_bytes, b_jstep = B_ROWS * g.b_ld_bytes;
   auto scalar_off = [&](bool is_b, int kt, int q) -> uint32_t {   // prologue: K tiles of the first operand pair
     const uint32_t j = (uint32_t)(wave + q * T::WAVES);
@@ -225,15 +235,15 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   uint32_t fa_off[A_MC ? T::TM : 1], fb_off[B_MC ? T::TN : 1];
   if (A_MC) {
 #pragma unroll
-    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true, BK>(wm + i * 32);
+    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true, BK, T::BM>(wm + i * 32);
   } else {
-    fa_off[0] = frag_lane_offset<false, BK>(wm);
+    fa_off[0] = frag_lane_offset<false, BK, T::BM>(wm);
   }
   if (B_MC) {
 #pragma unroll
-    for (int j = 0; j < T::TN; ++j) fb_off[j] = frag_lane_offset<true, BK>(wn + j * 32);
+    for (int j = 0; j < T::TN; ++j) fb_off[j] = frag_lane_offset<true, BK, T::BN>(wn + j * 32);
   } else {
-    fb_off[0] = frag_lane_offset<false, BK>(wn);
+    fb_off[0] = frag_lane_offset<false, BK, T::BN>(wn);
   }
 
   u32x4 fa[2][T::TM], fb[2][T::TN];
@@ -242,11 +252,11 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
   do {                                                                                                           \
     if constexpr ((M) < T::TM) {                                                                                 \
       constexpr int i_ = (M);                                                                                    \
-      if constexpr (A_MC) fa[BUF][i_] = read_frag<true, KSTEP>(A_ADDR, fa_off[A_MC ? i_ : 0]);                   \
+      if constexpr (A_MC) fa[BUF][i_] = read_frag<true, KSTEP, 0, T::BM>(A_ADDR, fa_off[A_MC ? i_ : 0]);                   \
       else fa[BUF][i_] = read_frag<false, KSTEP, i_ * KC_TILE>(A_ADDR, fa_off[0]);                               \
     } else if constexpr ((M) < T::TM + T::TN) {                                                                  \
       constexpr int j_ = (M) - T::TM;                                                                            \
-      if constexpr (B_MC) fb[BUF][j_] = read_frag<true, KSTEP>(B_ADDR, fb_off[B_MC ? j_ : 0]);                   \
+      if constexpr (B_MC) fb[BUF][j_] = read_frag<true, KSTEP, 0, T::BN>(B_ADDR, fb_off[B_MC ? j_ : 0]);                   \
       else fb[BUF][j_] = read_frag<false, KSTEP, j_ * KC_TILE>(B_ADDR, fb_off[0]);                               \
     }                                                                                                            \
   } while (0)
@@ -576,7 +586,7 @@ struct RowTiles {
 // DUAL: c = a @ b[e] + a2 @ b2[e] in one pass (k is the reduction length of each pair, at least
 // (SB + 1) K tiles), as one reduction over 2 k.
 template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false>
-__global__ void __launch_bounds__(T::THREADS)
+__global__ void __launch_bounds__(T::THREADS, T::WGS * T::WAVES / 4)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2) {
@@ -599,31 +609,38 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   g.nk1 = k / T::BK;
   g.nk = DUAL ? 2 * g.nk1 : g.nk1;
   g.rsrc_a2 = DUAL ? make_rsrc(a2, (uint32_t)(rows * k * 2)) : g.rsrc_a;
-  for (int r = 0; r < big_rounds; ++r) {
-    const int id = (r * kXcds + xcd) * run + member;
-    if (id >= total) break;
+  // Work items of this workgroup: one tile per round, then (if the tail is split) one half tile.
+  const int items = big_rounds + ((kSplit && split) ? 1 : 0);
+  for (int r = 0; r < items; ++r) {
+    int id, half = 0;
+    bool use_ts = false;
+    if (r < big_rounds) {
+      // Rotated by one member per round: where full and half-height tiles alternate along the list, a
+      // workgroup would otherwise be dealt the same kind in every round.
+      id = (r * kXcds + xcd) * run + (member + r) % run;
+      if (id >= total) break;
+    } else {
+      const int j = xcd * run + member;   // half tile j: tile j / 2 of the tail, rows half j % 2
+      if (j >= 2 * rest) break;
+      id = full_rounds * P + j / 2;
+      half = j & 1;
+      use_ts = true;
+    }
     int e, start, end, tm, tn;
     tiles.find(id, e, start, end, tm, tn);
-    g.a_r0 = start + tm * T::BM;
+    g.a_r0 = start + tm * T::BM + half * TS::BM;
+    if (g.a_r0 >= end) break;             // the second half of a tile whose rows end in the first (a last item)
     g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
     g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
     g.b_r0 = tn * T::BN;
-    block_gemm<DT, false, B_MC, T, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
-    tile_done();
-  }
-  if (kSplit && split) {
-    const int j = xcd * run + member;     // half tile j: tile j / 2 of the tail, rows half j % 2
-    if (j < 2 * rest) {
-      int e, start, end, tm, tn;
-      tiles.find(full_rounds * P + j / 2, e, start, end, tm, tn);
-      g.a_r0 = start + tm * T::BM + (j & 1) * TS::BM;
-      if (g.a_r0 < end) {
-        g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
-        g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
-        g.b_r0 = tn * TS::BN;
-        block_gemm<DT, false, B_MC, TS, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
-      }
+    // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
+    use_ts = kSplit && (use_ts || end - g.a_r0 <= TS::BM);
+    if (use_ts) {
+      block_gemm<DT, false, B_MC, TS, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+    } else {
+      block_gemm<DT, false, B_MC, T, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
     }
+    tile_done();
   }
 }
 
@@ -646,7 +663,7 @@ static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chun
 }
 
 template <int DT, typename T>
-__global__ void __launch_bounds__(T::THREADS)
+__global__ void __launch_bounds__(T::THREADS, T::WGS * T::WAVES / 4)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
