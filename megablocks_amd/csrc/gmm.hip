@@ -12,7 +12,6 @@
 // values of its column.  The tile -> (expert, row tile) schedule is computed on the device
 // from the inclusive row bins, so no host copy of the group sizes is needed and empty
 // experts cost nothing (NN/NT) or produce an all-zero block (TN).
-#include <cstdlib>
 #include "common.h"
 
 namespace mbx {
@@ -451,13 +450,10 @@ __global__ void gelu_backward_kernel(void* __restrict__ g_, const void* __restri
 // 256 registers per lane and needs 144 KiB of the 160 KiB LDS for two stages.
 typedef Tile<256, 256, 64, 2, 2, 8, 32> TileBig;
 typedef dma::Tile<256, 256, 2, 2, 64, 2> TileDma;
-// For small experts (NN / NT only: the row tile follows the expert's row count) a 128-row tile wastes
-// fewer rows of the last tile of every expert; its smaller stages allow a three-deep ring.
+// Half-height tile (NN / NT only: the row tile follows the expert's row count) for the last row tile of
+// an expert when it is at most half full, for the tail of a launch, and for launches of small experts;
+// its smaller stages allow a three-deep ring.
 typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;   // 4 x 16 KiB + 3 x 32 KiB
-// Two workgroups per compute unit (3 x 16 KiB + 2 x 16 KiB each): while one stores its tile or waits for
-// the first K tile of the next, the other multiplies.  For launches with short reductions or few rows per
-// expert, which are bound by HBM and by the per-tile prologue and epilogue rather than by the matrix cores.
-typedef dma::Tile<128, 128, 2, 2, 64, 2, 2> TileDmaPair;
 
 template <int DT, bool A_MC, bool B_MC, typename T>
 constexpr size_t lds_bytes() {
@@ -509,7 +505,7 @@ int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num
 
 // One persistent workgroup per compute unit (a multiple of 8, so that every XCD gets the same number),
 // fewer when there are not that many tiles.
-static inline int persistent_grid(int64_t tiles_upper_bound, int wgs_per_cu = 1) {
+static inline int persistent_grid(int64_t tiles_upper_bound) {
   static int cus[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
@@ -519,8 +515,7 @@ static inline int persistent_grid(int64_t tiles_upper_bound, int wgs_per_cu = 1)
     cus[dev] = n / kXcds * kXcds;
   }
   const int64_t need = (tiles_upper_bound + kXcds - 1) / kXcds * kXcds;
-  const int64_t cap = (int64_t)cus[dev] * wgs_per_cu;
-  return (int)(need < cap ? need : cap);
+  return (int)(need < cus[dev] ? need : cus[dev]);
 }
 
 // Launch of the direct-to-LDS kernels (k a multiple of 64 for NN / NT, operands below 2 GiB).
@@ -543,8 +538,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (rc) return rc;
     // short reductions (few rows per expert): several tiles per workgroup
     const int64_t avg_rows = rows / (num_groups > 0 ? num_groups : 1);
-    int chunk = avg_rows >= 1024 ? 1 : avg_rows >= 512 ? 2 : 4;
-    if (const char* e_ = getenv("MBX_CHUNK")) chunk = atoi(e_);   // EXPERIMENT
+    const int chunk = avg_rows >= 1024 ? 1 : avg_rows >= 512 ? 2 : 4;
     const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups, chunk);
     if (grid > 0x7fffffff) return MBX_ERANGE;
     kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n, chunk);
@@ -554,7 +548,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const int tiles_n = (int)ceil_div(n, T::BN);
   const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
   if (tiles > 0x7fffffff) return MBX_ERANGE;
-  const unsigned grid = (unsigned)persistent_grid(tiles, T::WGS);
+  const unsigned grid = (unsigned)persistent_grid(tiles);
 #define MBX_LAUNCH_ROWS(B_MC, DUAL)                                                                   \
   do {                                                                                                \
     auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL>;                                          \
@@ -584,6 +578,19 @@ int gmm_generic(const void* a, const void* b, void* c, const int32_t* bins, int 
 }
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// NN / NT: whether to tile a launch with the half-height tile only.  With about one such tile per expert
+// (up to 144 rows on average) the full tile would mostly multiply padding.  Up to 320 rows the mix of
+// full tiles and a half-height last tile moves fewer weight bytes through the compute units (the
+// weights are streamed once per row tile), but its tiles cost unequal time, and a launch of fewer than
+// three rounds of them does not balance over the statically assigned workgroups.
+static inline bool half_height_only(int64_t rows, int num_groups, int n) {
+  const int64_t avg = rows / (num_groups > 0 ? num_groups : 1);
+  if (avg <= 144) return true;
+  if (avg > 320) return false;
+  const int64_t mixed_tiles = (ceil_div(rows, TileDma::BM) + num_groups / 2) * ceil_div(n, TileDma::BN);
+  return mixed_tiles < 3 * (int64_t)persistent_grid((int64_t)1 << 30);
+}
 
 }  // namespace
 }  // namespace mbx
@@ -620,15 +627,7 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     bool dma_ok = rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
     if (layout != MBX_TN) dma_ok = dma_ok && k % TileDma::BK == 0;
     if (dma_ok) {
-      const bool small_m = layout != MBX_TN && rows <= (int64_t)num_groups * 144;   // average rows per expert
-      {   // EXPERIMENT
-        const char* e_ = getenv("MBX_TILE");
-        const int mode = e_ ? atoi(e_) : 0;
-        const bool pair = (mode & 1 && layout == MBX_NT) || (mode & 2 && layout == MBX_NN) || (mode & 4 && layout == MBX_TN);
-        if (pair && dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaPair, TileDmaPair>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-        if ((mode & 8) && dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-        if ((mode & 16) && dtype == MBX_BF16 && layout != MBX_TN) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-      }
+      const bool small_m = layout != MBX_TN && half_height_only(rows, num_groups, n);
       if (small_m) {
         if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
         return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
@@ -661,7 +660,7 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
                   rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
-  const bool small_m = rows <= (int64_t)num_groups * 144;
+  const bool small_m = half_height_only(rows, num_groups, n);
   if (small_m) {
     if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
     return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);

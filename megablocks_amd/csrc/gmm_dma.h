@@ -35,10 +35,9 @@ namespace dma {
 // B load can be (the B stage to refill is still being read), so that global -> LDS loads leave the
 // compute unit at an even rate: the texture-address unit takes some 20 cycles per wave-wide load, is
 // shared by the four waves, and a wave whose load has to queue cannot issue its next MFMA either.
-// WGS: workgroups meant to share a compute unit (its LDS and registers are split between them).
-template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_, int WGS_ = 1>
+template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1, WGS = WGS_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1;
   static constexpr int KS = BK / 16;                                           // MFMA k-steps per tile
   static constexpr int WAVES = WM * WN, THREADS = WAVES * kWave;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -49,7 +48,7 @@ struct Tile {
   static constexpr size_t RING_BYTES = (size_t)SA * A_BYTES + (size_t)SB * B_BYTES, EPILOGUE_BYTES = (size_t)BM * (BN * 2 + 16);
   static constexpr size_t LDS_BYTES = RING_BYTES > EPILOGUE_BYTES ? RING_BYTES : EPILOGUE_BYTES;
   static_assert(BK == 64, "K tile");
-  static_assert(SB >= 2 && LDS_BYTES * WGS <= 160 * 1024, "LDS rings");
+  static_assert(SB >= 2 && LDS_BYTES <= 160 * 1024, "LDS rings");
   static_assert((BM == 256 || BM == 128) && (BN == 256 || BN == 128), "tile widths the strided-operand LDS layout knows");
   static_assert(A_INSTRS % WAVES == 0 && B_INSTRS % WAVES == 0, "loads must split evenly over the waves");
   static_assert(LA % 2 == 0 && LB % 2 == 0, "the loads of an operand tile are issued in two halves");
@@ -586,7 +585,7 @@ struct RowTiles {
 // DUAL: c = a @ b[e] + a2 @ b2[e] in one pass (k is the reduction length of each pair, at least
 // (SB + 1) K tiles), as one reduction over 2 k.
 template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false>
-__global__ void __launch_bounds__(T::THREADS, T::WGS * T::WAVES / 4)
+__global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2) {
@@ -663,7 +662,7 @@ static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chun
 }
 
 template <int DT, typename T>
-__global__ void __launch_bounds__(T::THREADS, T::WGS * T::WAVES / 4)
+__global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];

@@ -226,6 +226,34 @@ def test_gmm_tile_schedules(gg, name, groups, rows, k, n):
         assert torch.equal(again, got)                              # same schedule, same summation order: bit-identical
 
 
+MIXED_ROWS = [  # per-expert row counts around the boundaries between full (256-row) and half-height (128-row) tiles
+    [256, 257, 300, 384, 385, 129, 128, 1, 0, 512, 640, 127],
+    [300] * 48,                       # full and half-height tiles alternate along the tile list, several rounds
+    [260, 250] * 40,                  # more than 64 experts
+    [130] * 64,                       # on average below the full tile: half-height tiles only
+]
+
+
+@pytest.mark.parametrize('rows_per_expert', MIXED_ROWS, ids=lambda r: f'{len(r)}experts')
+@pytest.mark.parametrize('k,n', [(256, 1024), (512, 264)])
+def test_gmm_full_and_half_height_row_tiles(gg, rows_per_expert, k, n):
+    sizes = torch.tensor(rows_per_expert, dtype=torch.int64)
+    groups, rows = len(rows_per_expert), int(sizes.sum())
+    torch.manual_seed(rows)
+    a = torch.randn(rows, k, device='cuda').bfloat16()
+    b_nt = (torch.randn(groups, n, k, device='cuda') * 0.1).bfloat16()
+    b_nn = (torch.randn(groups, k, n, device='cuda') * 0.1).bfloat16()
+    for b, tb in ((b_nt, True), (b_nn, False)):
+        got = gg.backend.gmm(a, b, sizes, trans_b=tb)
+        ref = _ref_gpu(a, b, sizes, False, tb)
+        assert rel_err(got, ref) < TOL and max_block_err(got, ref) < 2 * TOL, tb
+    a2 = torch.randn(rows, k, device='cuda').bfloat16()
+    b2 = (torch.randn(groups, k, n, device='cuda') * 0.1).bfloat16()
+    got = gg.gmm_dual(a, b_nn, a2, b2, sizes)
+    ref = _ref_gpu(a, b_nn, sizes, False, False).float() + _ref_gpu(a2, b2, sizes, False, False).float()
+    assert rel_err(got.float(), ref) < TOL
+
+
 def _random_shapes(count, seed):
     g = torch.Generator().manual_seed(seed)
     r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
