@@ -41,6 +41,8 @@ def parse():
     ap.add_argument('--memory-optimized', action='store_true')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
     ap.add_argument('--cpu-tokens', type=int, default=None)
+    ap.add_argument('--library-gemm', action='store_true',
+                    help='also time the three grouped products as per-expert torch.matmul loops (the vendor GEMM library)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also launch one plain 1 GiB device copy (a known-size reference for HBM byte counters)')
     return ap.parse_args()
@@ -135,6 +137,65 @@ def summarize(w, agg, slots_scale):
                               gbps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
                               frac_of_hbm_peak=round(nbytes / (avg_ms * 1e-3) / HBM_PEAK, 4))
     return gemm, perm
+
+
+def library_gemm_leg(w, inp):
+    """The grouped products of one layer step done the way a build without a grouped kernel does them: one
+    library GEMM (torch.matmul, i.e. hipBLASLt / rocBLAS) per expert, on this workload's shapes and its own
+    rows-per-expert.  A reference point for the grouped kernel, not part of the layer that is benchmarked."""
+    import torch
+
+    dev = torch.device('cuda', 0)
+    if w.routing == 'router':
+        logits = inp['x'].to(dev).float() @ inp['router_weight'].to(dev).float().t()
+        top = logits.topk(w.top_k, dim=-1).indices
+    else:
+        top = inp['top_experts'].to(dev)
+    counts = torch.bincount(top.flatten(), minlength=w.experts).tolist()
+    rows = sum(counts)
+    a = torch.randn(rows, w.hidden, device=dev, dtype=w.dtype)
+    mid = torch.randn(rows, w.ffn, device=dev, dtype=w.dtype)
+    w1 = torch.randn(w.experts, w.ffn, w.hidden, device=dev, dtype=w.dtype) * 0.02
+    out_f = torch.empty(rows, w.ffn, device=dev, dtype=w.dtype)
+    out_h = torch.empty(rows, w.hidden, device=dev, dtype=w.dtype)
+    dw = torch.empty(w.experts, w.ffn, w.hidden, device=dev, dtype=w.dtype)
+    bounds, start = [], 0
+    for c in counts:
+        bounds.append((start, start + c))
+        start += c
+
+    def nt():   # x @ w1[e]^T
+        for e, (lo, hi) in enumerate(bounds):
+            if hi > lo:
+                torch.matmul(a[lo:hi], w1[e].t(), out=out_f[lo:hi])
+
+    def nn():   # h @ w2[e] (w2 stored like w1: [ffn, hidden])
+        for e, (lo, hi) in enumerate(bounds):
+            if hi > lo:
+                torch.matmul(mid[lo:hi], w1[e], out=out_h[lo:hi])
+
+    def tn():   # h^T @ dy: the weight gradient
+        for e, (lo, hi) in enumerate(bounds):
+            if hi > lo:
+                torch.matmul(mid[lo:hi].t(), a[lo:hi], out=dw[e])
+            else:
+                dw[e].zero_()
+
+    flops = 2.0 * rows * w.hidden * w.ffn
+    res = {'what': 'one torch.matmul per expert (vendor GEMM library), same shapes and rows per expert', 'kernels': {}}
+    for name, fn in (('gmm_nt', nt), ('gmm_nn', nn), ('gmm_tn', tn)):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 10
+        res['kernels'][name] = dict(avg_ms=round(ms, 4), tflops=round(flops / (ms * 1e-3) / 1e12, 1))
+    return res
 
 
 def cpu_leg(args, w, inp_full):
@@ -245,6 +306,8 @@ def main():
                  'frac_of_mfma_peak': round(all_gemm_tflops * 1e12 / MFMA_PEAK[dn], 4), 'kernels': gemm},
         'permute': {'ms_per_step': round(perm_ms, 4), 'kernels': perm},
     }
+    if args.library_gemm:
+        out['library_gemm'] = library_gemm_leg(w, inp)
     if not args.no_cpu:
         del layer
         torch.cuda.empty_cache()
