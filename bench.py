@@ -131,7 +131,7 @@ def summarize(w, agg, slots_scale):
                               frac_of_mfma_peak=round(flops / (avg_ms * 1e-3) / MFMA_PEAK[dn], 4),
                               bytes_per_launch=nbytes, gbps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
                               frac_of_hbm_peak=round(nbytes / (avg_ms * 1e-3) / HBM_PEAK, 4))
-        else:
+        elif 'hidden' in m:
             nbytes = float(w.tokens + w.slots) * m['hidden'] * m['elem']
             perm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, bytes_per_launch=nbytes,
                               gbps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),

@@ -645,16 +645,21 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
 
 // ---- TN ----
 // Tiles of one expert's [k, n] product are enumerated in 8 x 4 blocks (8 row tiles x 4 column tiles:
-// 12 operand panels per 32 tiles), and that sequence is cut into 8 equal pieces, one per XCD: XCD x
-// works through piece x of the first expert, piece x of the second, and so on.  The cost of a tile
+// 12 operand panels per 32 tiles; smaller blocks for products with fewer tiles in a direction), and that
+// sequence is cut into 8 equal pieces, one per XCD: XCD x works through piece x of the first expert,
+// piece x + 1 of the second, and so on (rotated, so that products of fewer than 8 tiles per expert still
+// spread over all XCDs).  The cost of a tile
 // is proportional to its expert's row count, so with skewed routing any coarser dealing of tiles to
 // XCDs (whose queues are fixed by the workgroup id) leaves some XCDs with several times the work.
 // For the same reason the tiles of an XCD are not dealt to workgroups statically: a workgroup takes
 // `chunk` consecutive tiles of its XCD's list and the hardware hands out workgroups as compute units
 // become free (chunk > 1 when the reductions are short and the per-workgroup overhead shows).
 constexpr int kTnBlockM = 8, kTnBlockN = 4;
+__host__ __device__ static inline int tn_block_m(int tiles_m) { return tiles_m < kTnBlockM ? (tiles_m > 0 ? tiles_m : 1) : kTnBlockM; }
+__host__ __device__ static inline int tn_block_n(int tiles_n) { return tiles_n < kTnBlockN ? (tiles_n > 0 ? tiles_n : 1) : kTnBlockN; }
 static inline int64_t tn_tiles_per_group(int tiles_m, int tiles_n) {
-  return (int64_t)((tiles_m + kTnBlockM - 1) / kTnBlockM) * ((tiles_n + kTnBlockN - 1) / kTnBlockN) * (kTnBlockM * kTnBlockN);
+  const int bm = tn_block_m(tiles_m), bn = tn_block_n(tiles_n);
+  return (int64_t)((tiles_m + bm - 1) / bm) * ((tiles_n + bn - 1) / bn) * (bm * bn);
 }
 static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chunk) {
   const int64_t per_xcd = (tn_tiles_per_group(tiles_m, tiles_n) + kXcds - 1) / kXcds;
@@ -666,8 +671,9 @@ __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  const int blocks_m = (tiles_m + kTnBlockM - 1) / kTnBlockM, blocks_n = (tiles_n + kTnBlockN - 1) / kTnBlockN;
-  const int per_group = blocks_m * blocks_n * (kTnBlockM * kTnBlockN);
+  const int bm = tn_block_m(tiles_m), bn = tn_block_n(tiles_n);
+  const int blocks_m = (tiles_m + bm - 1) / bm, blocks_n = (tiles_n + bn - 1) / bn;
+  const int per_group = blocks_m * blocks_n * (bm * bn);
   const int per_xcd = (per_group + kXcds - 1) / kXcds;
   const int xcd = blockIdx.x % kXcds;
   // Experts are taken in order of decreasing row count (longest reduction first), so that the tiles
@@ -692,11 +698,17 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
   const int64_t first = (int64_t)(blockIdx.x / kXcds) * chunk;
   for (int64_t i = first; i < first + chunk && i < items; ++i) {
     const int slot = (int)(i / per_xcd);                  // position of the expert in the longest-first order
-    const int t = xcd * per_xcd + (int)(i % per_xcd);     // tile slot inside the expert
+    const int t = ((xcd + slot) % kXcds) * per_xcd + (int)(i % per_xcd);     // tile slot inside the expert
     if (t >= per_group) continue;
-    const int blk = t / (kTnBlockM * kTnBlockN), in = t % (kTnBlockM * kTnBlockN);
-    const int tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
-    if (tm >= tiles_m || tn >= tiles_n) continue;   // padding of the 8 x 4 enumeration (uniform over the workgroup)
+    int blk, in, tm, tn;
+    if (bm == kTnBlockM && bn == kTnBlockN) {   // the usual case, with constant divisors
+      blk = t / (kTnBlockM * kTnBlockN), in = t % (kTnBlockM * kTnBlockN);
+      tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
+    } else {
+      blk = t / (bm * bn), in = t % (bm * bn);
+      tm = (blk % blocks_m) * bm + in % bm, tn = (blk / blocks_m) * bn + in / bm;
+    }
+    if (tm >= tiles_m || tn >= tiles_n) continue;   // padding of the block enumeration (uniform over the workgroup)
     int e = slot;
     if (ranked) e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(__ballot(rank == slot)));
     const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];

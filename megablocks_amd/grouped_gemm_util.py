@@ -40,11 +40,12 @@ def _device_bins(batch_sizes: torch.Tensor, device) -> torch.Tensor:
     return bins
 
 
-def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None):
+def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None, _record_as=None):
     """out[r_e] = a[r_e] @ b[e] (`trans_b`: @ b[e].T); `trans_a`: out[e] = a[r_e].T @ b[r_e].
 
     a is [rows, k]; b is [E, k, n] ([E, n, k] with trans_b) or, with trans_a, [rows, n].
-    fp32 accumulation, output in a.dtype, written to `c` when given.
+    fp32 accumulation, output in a.dtype, written to `c` when given.  `_record_as` names the launch in the
+    optional per-launch timing (callers other than the expert MLPs keep out of their statistics).
     """
     _lib.require_cuda(a, b, c)
     if a.ndim != 2:
@@ -81,7 +82,7 @@ def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None):
     else:
         if tuple(c.shape) != shape or c.dtype != a.dtype or not c.is_contiguous():
             raise ValueError('gmm: c has the wrong shape, dtype or layout')
-    with torch.cuda.device_of(a), _lib.record(('gmm_nn', 'gmm_nt', 'gmm_tn')[layout], rows=rows, k=k, n=n,
+    with torch.cuda.device_of(a), _lib.record(_record_as or ('gmm_nn', 'gmm_nt', 'gmm_tn')[layout], rows=rows, k=k, n=n,
                                               elem=a.element_size(), groups=groups):
         _lib.check(lib.mbx_gmm(_lib.ptr(a), _lib.ptr(b), _lib.ptr(c), dt, _lib.ptr(bins), groups, rows, k, n, layout,
                                _lib.stream()), 'gmm')

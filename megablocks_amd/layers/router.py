@@ -1,5 +1,6 @@
 """Learned top-k router: megablocks/layers/router.py:10-114.  Plain PyTorch-ROCm (a small dense
-GEMM, softmax and top-k); its outputs feed the HIP routing kernels."""
+GEMM, softmax and top-k) except for the weight gradient of the linear layer on large 16-bit batches, which
+goes through the grouped TN kernel; its outputs feed the HIP routing kernels."""
 from typing import Any
 
 import torch
@@ -41,6 +42,47 @@ class _UniformExpertAssignment(torch.autograd.Function):
         return torch.remainder(out, num_experts).view(x.shape)
 
 
+class _RouterLinear(torch.autograd.Function):
+    """`x @ weight^T` of the router's `torch.nn.Linear` (router.py:96), with the weight gradient
+    `[E, T] @ [T, h]` (a short, wide output over a reduction as long as the batch: a handful of tiles for the
+    vendor GEMM) computed by the grouped TN kernel instead: the token range is cut into equal pieces, each
+    piece is one group, and the partial products are summed in fp32."""
+
+    PIECE_ROWS = 256   # tokens per piece (four K tiles of the TN kernel)
+    MAX_PIECES = 64
+
+    _sizes = {}
+
+    @staticmethod
+    def piece_sizes(tokens: int) -> torch.Tensor:
+        """Rows per piece (kept per batch size: the grouped GEMM caches the device-side bins on this tensor)."""
+        sizes = _RouterLinear._sizes.get(tokens)
+        if sizes is None:
+            pieces = max(1, min(_RouterLinear.MAX_PIECES, tokens // _RouterLinear.PIECE_ROWS))
+            sizes = torch.full((pieces,), tokens // pieces, dtype=torch.int64)
+            sizes[:tokens % pieces] += 1
+            _RouterLinear._sizes[tokens] = sizes
+        return sizes
+
+    @staticmethod
+    def forward(ctx: Any, x: torch.Tensor, weight: torch.Tensor):
+        ctx.save_for_backward(x, weight)
+        return torch.nn.functional.linear(x, weight)
+
+    @staticmethod
+    def backward(ctx: Any, grad: torch.Tensor):
+        x, weight = ctx.saved_tensors
+        dx = grad @ weight if ctx.needs_input_grad[0] else None
+        dw = None
+        if ctx.needs_input_grad[1]:
+            from megablocks_amd import grouped_gemm_util as gg
+            sizes = _RouterLinear.piece_sizes(x.shape[0])
+            pieces = sizes.shape[0]
+            parts = gg.gmm(grad.contiguous(), x.contiguous(), sizes, trans_a=True, _record_as='router_wgrad')   # [pieces, E, h]
+            dw = parts[0] if pieces == 1 else parts.float().sum(0).to(weight.dtype)
+        return dx, dw
+
+
 class LearnedRouter(torch.nn.Module):
 
     def __init__(self, args: Arguments):
@@ -64,7 +106,11 @@ class LearnedRouter(torch.nn.Module):
     def forward(self, x: torch.Tensor):
         if self.training and self.args.moe_jitter_eps is not None:
             x = x * self.jitter(x)
-        logits = self.layer(x.view(-1, x.shape[-1]))
+        x2d = x.view(-1, x.shape[-1])
+        if x2d.is_cuda and x2d.dtype in (torch.bfloat16, torch.float16) and x2d.shape[0] >= 4 * _RouterLinear.PIECE_ROWS:
+            logits = _RouterLinear.apply(x2d, self.layer.weight)
+        else:
+            logits = self.layer(x2d)
         _save_router_logits(logits, self.args)
         scores = logits.softmax(dim=-1)
         expert_weights, expert_indices = self._top_k(scores)

@@ -105,6 +105,32 @@ def test_dmoe_forward_backward_vs_oracle(syn, tokens, hidden, ffn, experts, top_
         assert rel_err(layer.router.layer.weight.grad, want_grads['router']) < 5 * tol
 
 
+@pytest.mark.parametrize('tokens,hidden,experts', [(4096, 1024, 64), (5003, 264, 8), (16384, 512, 16)])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_router_linear_gradients(tokens, hidden, experts, dtype):
+    """The router's linear layer on large 16-bit batches: logits are torch's own, the weight gradient comes
+    from the grouped TN kernel over equal pieces of the batch (router.py:96 and its autograd)."""
+    from megablocks_amd.layers.arguments import Arguments
+    from megablocks_amd.layers.router import LearnedRouter, _RouterLinear
+    torch.manual_seed(tokens)
+    args = Arguments(hidden_size=hidden, ffn_hidden_size=hidden, moe_num_experts=experts, moe_top_k=1, device='cuda',
+                     bf16=dtype == torch.bfloat16, fp16=dtype == torch.float16)
+    router = LearnedRouter(args)
+    x = torch.randn(tokens, hidden, device='cuda', dtype=dtype, requires_grad=True)
+    g = torch.randn(tokens, experts, device='cuda', dtype=dtype)
+    assert tokens >= 4 * _RouterLinear.PIECE_ROWS
+    logits = _RouterLinear.apply(x, router.layer.weight)
+    assert torch.equal(logits, torch.nn.functional.linear(x, router.layer.weight))
+    logits.backward(g)
+    want_dw = g.float().t() @ x.detach().float()
+    want_dx = g.float() @ router.layer.weight.detach().float()
+    assert router.layer.weight.grad.dtype == dtype and router.layer.weight.grad.shape == (experts, hidden)
+    assert rel_err(router.layer.weight.grad, want_dw) < 1e-2
+    assert rel_err(x.grad, want_dx) < 1e-2
+    sizes = _RouterLinear.piece_sizes(tokens)
+    assert int(sizes.sum()) == tokens and sizes.shape[0] == min(64, tokens // 256) and int(sizes.max() - sizes.min()) <= 1
+
+
 def test_routing_bookkeeping_is_bit_exact(syn):
     from megablocks_amd.layers.arguments import Arguments
     from megablocks_amd.layers.dmoe import ParallelDroplessMLP
