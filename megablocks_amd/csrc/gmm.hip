@@ -627,7 +627,8 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     bool dma_ok = rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
     if (layout != MBX_TN) dma_ok = dma_ok && k % TileDma::BK == 0;
     if (dma_ok) {
-      const bool small_m = layout != MBX_TN && half_height_only(rows, num_groups, n);
+      // TN: the half-height tile only when the product has at most 128 rows (it is slower otherwise)
+      const bool small_m = layout == MBX_TN ? k <= TileDmaSmallM::BM : half_height_only(rows, num_groups, n);
       if (small_m) {
         if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
         return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
