@@ -170,6 +170,24 @@ int mbx_glu_forward(const void* a, const void* b, void* out, int dtype, int act,
 int mbx_glu_backward(const void* g, const void* a, const void* b, void* da, void* db, int dtype,
                      int act, int64_t numel, mbx_stream_t stream);
 
+/* ---- router post-processing (megablocks/layers/router.py:87-106) ----
+ * What LearnedRouter.forward does after the linear layer, for `tokens` rows of `num_experts` logits:
+ *   scores  = softmax(logits, dim=-1)                                   router.py:98   [tokens, num_experts]
+ *   weights, indices = scores.max(-1) (top_k == 1) / torch.topk(scores, top_k)  router.py:87-90  [tokens, top_k]
+ *   weights = weights / norm(weights, p = norm_p, dim=-1)   if norm_p > 0        router.py:100-106
+ * computed in fp32 and rounded to `dtype` where torch's operations round (scores; the norm; the quotient).
+ * Weights come out in descending order; equal scores are taken in ascending expert index.  indices are
+ * int64 like torch.topk's.  num_experts up to 512 and top_k up to 64, else MBX_EUNSUPPORTED. */
+int mbx_router_forward(const void* logits, int dtype, int64_t tokens, int num_experts, int top_k, float norm_p,
+                       void* scores, void* weights, int64_t* indices, mbx_stream_t stream);
+
+/* Backward of the above as autograd derives it for router.py:98-106: grad_logits from grad_weights
+ * [tokens, top_k] (NULL: none) and, optionally, a gradient that reaches `scores` directly (NULL: none;
+ * e.g. from the load-balancing loss, moe.py:32-89), given the forward's scores and indices. */
+int mbx_router_backward(const void* grad_weights, const void* grad_scores, const void* scores, const int64_t* indices,
+                        int dtype, int64_t tokens, int num_experts, int top_k, float norm_p, void* grad_logits,
+                        mbx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

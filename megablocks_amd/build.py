@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
 BUILD = os.path.join(HERE, 'build')
 LIB = os.path.join(HERE, 'libmbx.so')
-SOURCES = ['routing.hip', 'permute.hip', 'gmm.hip', 'elementwise.hip']
+SOURCES = ['routing.hip', 'permute.hip', 'gmm.hip', 'elementwise.hip', 'router.hip']
 HEADERS = [os.path.join(CSRC, 'common.h'), os.path.join(CSRC, 'gmm_dma.h'),
            os.path.join(os.path.dirname(HERE), 'include', 'mbx.h')]
 ARCH = 'gfx950'

@@ -1,14 +1,19 @@
-"""Learned top-k router: megablocks/layers/router.py:10-114.  Plain PyTorch-ROCm (a small dense
-GEMM, softmax and top-k) except for the weight gradient of the linear layer on large 16-bit batches, which
-goes through the grouped TN kernel; its outputs feed the HIP routing kernels."""
+"""Learned top-k router: megablocks/layers/router.py:10-114.  The linear layer is torch's (a small dense
+GEMM), except for its weight gradient on large 16-bit batches, which goes through the grouped TN kernel;
+softmax, top-k and the renormalisation of the selected weights are one HIP kernel each way.  The outputs
+feed the HIP routing kernels."""
 from typing import Any
 
 import torch
 
+from megablocks_amd import _lib
 from megablocks_amd.layers import common
 from megablocks_amd.layers.arguments import Arguments
 
 _ROUTER_LOGITS = []
+
+# softmax / top-k / renormalisation as one HIP kernel each way (False: torch's operations, as the reference)
+FUSED_SOFTMAX_TOPK = True
 
 
 def _save_router_logits(logits: torch.Tensor, args: Arguments):
@@ -83,6 +88,45 @@ class _RouterLinear(torch.autograd.Function):
         return dx, dw
 
 
+class _SoftmaxTopK(torch.autograd.Function):
+    """softmax -> top-k -> optional p-norm renormalisation (router.py:87-106) as one kernel each way.
+    Returns (scores, expert_weights, expert_indices) with torch's shapes and dtypes (int64 indices)."""
+
+    @staticmethod
+    def supported(logits: torch.Tensor, top_k: int) -> bool:
+        return (logits.is_cuda and logits.ndim == 2 and logits.dtype in _lib.DTYPE and 0 < logits.shape[1] <= 512
+                and 0 < top_k <= min(64, logits.shape[1]))
+
+    @staticmethod
+    def forward(ctx: Any, logits: torch.Tensor, top_k: int, norm_p: float):
+        logits = logits.contiguous()
+        tokens, experts = logits.shape
+        scores = torch.empty_like(logits)
+        weights = torch.empty((tokens, top_k), dtype=logits.dtype, device=logits.device)
+        indices = torch.empty((tokens, top_k), dtype=torch.int64, device=logits.device)
+        with torch.cuda.device_of(logits):
+            _lib.check(_lib.lib.mbx_router_forward(_lib.ptr(logits), _lib.dtype_of(logits), tokens, experts, top_k,
+                                                   float(norm_p), _lib.ptr(scores), _lib.ptr(weights), _lib.ptr(indices),
+                                                   _lib.stream()), 'router_forward')
+        ctx.save_for_backward(scores, indices)
+        ctx.top_k, ctx.norm_p = top_k, float(norm_p)
+        ctx.mark_non_differentiable(indices)
+        return scores, weights, indices
+
+    @staticmethod
+    def backward(ctx: Any, grad_scores, grad_weights, _grad_indices):
+        scores, indices = ctx.saved_tensors
+        tokens, experts = scores.shape
+        grad_logits = torch.empty_like(scores)
+        gs = None if grad_scores is None else grad_scores.to(scores.dtype).contiguous()
+        gw = None if grad_weights is None else grad_weights.to(scores.dtype).contiguous()
+        with torch.cuda.device_of(scores):
+            _lib.check(_lib.lib.mbx_router_backward(_lib.ptr(gw), _lib.ptr(gs), _lib.ptr(scores), _lib.ptr(indices),
+                                                    _lib.dtype_of(scores), tokens, experts, ctx.top_k, ctx.norm_p,
+                                                    _lib.ptr(grad_logits), _lib.stream()), 'router_backward')
+        return grad_logits, None, None
+
+
 class LearnedRouter(torch.nn.Module):
 
     def __init__(self, args: Arguments):
@@ -112,11 +156,15 @@ class LearnedRouter(torch.nn.Module):
         else:
             logits = self.layer(x2d)
         _save_router_logits(logits, self.args)
-        scores = logits.softmax(dim=-1)
-        expert_weights, expert_indices = self._top_k(scores)
-        if self.args.moe_normalize_expert_weights:
-            expert_weights = expert_weights / torch.norm(
-                expert_weights, p=self.args.moe_normalize_expert_weights, dim=-1, keepdim=True)
+        if FUSED_SOFTMAX_TOPK and _SoftmaxTopK.supported(logits, self.args.moe_top_k):
+            scores, expert_weights, expert_indices = _SoftmaxTopK.apply(
+                logits, self.args.moe_top_k, self.args.moe_normalize_expert_weights or 0)
+        else:
+            scores = logits.softmax(dim=-1)
+            expert_weights, expert_indices = self._top_k(scores)
+            if self.args.moe_normalize_expert_weights:
+                expert_weights = expert_weights / torch.norm(
+                    expert_weights, p=self.args.moe_normalize_expert_weights, dim=-1, keepdim=True)
         if self.args.uniform_expert_assignment:
             expert_indices = _UniformExpertAssignment.apply(expert_indices, self.args.moe_num_experts)
         return scores, expert_weights, expert_indices

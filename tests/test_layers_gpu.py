@@ -131,6 +131,92 @@ def test_router_linear_gradients(tokens, hidden, experts, dtype):
     assert int(sizes.sum()) == tokens and sizes.shape[0] == min(64, tokens // 256) and int(sizes.max() - sizes.min()) <= 1
 
 
+def _softmax_topk_reference(logits, top_k, norm_p):
+    """router.py:87-106 with torch's own operations."""
+    scores = logits.softmax(dim=-1)
+    if top_k == 1:
+        w, i = scores.max(dim=-1, keepdim=True)
+    else:
+        w, i = torch.topk(scores, top_k, dim=-1)
+    if norm_p:
+        w = w / torch.norm(w, p=norm_p, dim=-1, keepdim=True)
+    return scores, w, i
+
+
+@pytest.mark.parametrize('tokens,experts,top_k', [(1, 1, 1), (300, 8, 2), (257, 64, 1), (200, 65, 6), (100, 128, 8),
+                                                  (50, 512, 64), (1000, 16, 4)])
+@pytest.mark.parametrize('norm_p', [0, 1, 2, 3.0])
+def test_router_softmax_topk_fp32_matches_oracle(tokens, experts, top_k, norm_p):
+    import oracle
+    from megablocks_amd.layers.router import _SoftmaxTopK
+    torch.manual_seed(tokens + experts)
+    logits = torch.randn(tokens, experts) * 3
+    want_s, want_w, want_i = oracle.router_forward(logits, torch.eye(experts), top_k, norm_p or None)
+    s, w, i = _SoftmaxTopK.apply(logits.cuda(), top_k, norm_p)
+    assert s.dtype == torch.float32 and w.shape == (tokens, top_k) and i.dtype == torch.int64
+    assert torch.allclose(s.cpu(), want_s, rtol=1e-5, atol=1e-7)
+    assert torch.equal(i.cpu(), want_i)                      # fp32 scores of random logits have no ties
+    assert torch.allclose(w.cpu(), want_w, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('tokens,experts,top_k,norm_p', [(4096, 8, 2, 1), (4096, 64, 1, 0), (2048, 64, 6, 1),
+                                                         (1024, 200, 4, 2)])
+def test_router_softmax_topk_16bit(dtype, tokens, experts, top_k, norm_p):
+    """16-bit scores tie often: the selection is checked against the kernel's own scores (descending, equal
+    scores in ascending expert index), the values against torch's operations in the same dtype."""
+    from megablocks_amd.layers.router import _SoftmaxTopK
+    torch.manual_seed(experts)
+    logits = (torch.randn(tokens, experts, device='cuda') * 2).to(dtype)
+    s, w, i = _SoftmaxTopK.apply(logits, top_k, norm_p)
+    ref_s, _, _ = _softmax_topk_reference(logits, top_k, norm_p)
+    ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    assert ((s.float() - ref_s.float()).abs() <= ulp * ref_s.float().abs() + 1e-30).all()   # at most one rounding step apart
+    order = torch.sort(s.float().cpu(), dim=-1, descending=True, stable=True).indices[:, :top_k]
+    assert torch.equal(i.cpu(), order)
+    picked = s.gather(1, i)
+    want_w = picked / torch.norm(picked, p=norm_p, dim=-1, keepdim=True) if norm_p else picked
+    assert ((w.float() - want_w.float()).abs() <= ulp * want_w.float().abs()).all()
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('experts,top_k,norm_p,with_score_grad', [(8, 2, 1, False), (64, 1, 0, True), (64, 6, 1, True),
+                                                                  (130, 4, 2, False), (16, 4, 3.0, True)])
+def test_router_softmax_topk_backward(dtype, experts, top_k, norm_p, with_score_grad):
+    from megablocks_amd.layers.router import _SoftmaxTopK
+    tokens = 777
+    torch.manual_seed(experts * top_k)
+    logits = (torch.randn(tokens, experts, device='cuda') * 2).to(dtype)
+    gw = torch.randn(tokens, top_k, device='cuda').to(dtype)
+    gs = torch.randn(tokens, experts, device='cuda').to(dtype) if with_score_grad else None
+    x = logits.clone().requires_grad_(True)
+    s, w, i = _SoftmaxTopK.apply(x, top_k, norm_p)
+    loss = (w.float() * gw.float()).sum() + ((s.float() * gs.float()).sum() if with_score_grad else 0)
+    loss.backward()
+    # reference: autograd through torch's operations in fp32, with the kernel's selection
+    xr = logits.float().clone().requires_grad_(True)
+    sr = xr.softmax(dim=-1)
+    wr = sr.gather(1, i)
+    if norm_p:
+        wr = wr / torch.norm(wr, p=norm_p, dim=-1, keepdim=True)
+    ((wr * gw.float()).sum() + ((sr * gs.float()).sum() if with_score_grad else 0)).backward()
+    assert x.grad.dtype == dtype
+    assert rel_err(x.grad, xr.grad) < (1e-5 if dtype == torch.float32 else 1e-2)
+
+
+def test_router_falls_back_to_torch_for_many_experts():
+    from megablocks_amd.layers.arguments import Arguments
+    from megablocks_amd.layers.router import LearnedRouter
+    args = Arguments(hidden_size=64, ffn_hidden_size=64, moe_num_experts=600, moe_top_k=2, device='cuda', bf16=True,
+                     fp16=False, moe_normalize_expert_weights=1)
+    router = LearnedRouter(args)
+    x = torch.randn(33, 64, device='cuda', dtype=torch.bfloat16, requires_grad=True)
+    scores, w, i = router(x)
+    assert scores.shape == (33, 600) and w.shape == (33, 2) and i.dtype == torch.int64
+    w.sum().backward()
+    assert router.layer.weight.grad is not None and x.grad is not None
+
+
 def test_routing_bookkeeping_is_bit_exact(syn):
     from megablocks_amd.layers.arguments import Arguments
     from megablocks_amd.layers.dmoe import ParallelDroplessMLP
