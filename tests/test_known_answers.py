@@ -89,6 +89,43 @@ def _check_permute(k, on_gpu):
     assert k.scatter_wgrad(g, x, indices, bin_ids, bins, p['top_k']).cpu().tolist() == p['wgrad_with_grad_equal_to_x']
 
 
+def _check_router(fn, on_gpu, ties_ascending):
+    """`fn(logits, top_k, norm_p)` -> (scores, weights, indices) as LearnedRouter computes them after its linear layer.
+    torch.topk leaves the order of equal scores open (the reference inherits that); the library takes them in
+    ascending expert index (`ties_ascending`).  Otherwise the indices only have to point at the right scores."""
+    r = KA['router']
+    logits = torch.tensor(r['logits'])
+    if on_gpu:
+        logits = logits.cuda()
+    close = lambda got, want: torch.allclose(got.cpu(), torch.tensor(want), rtol=1e-6, atol=1e-7)
+
+    def check_indices(i, s, w_unnormalised, want):
+        if ties_ascending:
+            assert i.cpu().tolist() == want
+        assert close(s.gather(1, i), w_unnormalised) and all(len(set(row)) == len(row) for row in i.cpu().tolist())
+
+    s, w, i = fn(logits, 1, 0)
+    assert close(s, r['scores']) and close(w, r['top1']['weights'])
+    check_indices(i, s, r['top1']['weights'], r['top1']['indices'])
+    s, w, i = fn(logits, 2, 0)
+    assert close(s, r['scores']) and close(w, r['top2']['weights'])
+    check_indices(i, s, r['top2']['weights'], r['top2']['indices'])
+    assert i.cpu()[0].tolist() == r['top2']['indices'][0]                 # no tie in the first row
+    assert close(fn(logits, 2, 1)[1], r['top2']['weights_p1']) and close(fn(logits, 2, 2)[1], r['top2']['weights_p2'])
+    s, w, i = fn(logits, 3, 0)
+    check_indices(i, s, [[0.5, 0.25, 0.125], [0.25, 0.25, 0.25]], r['top3_indices'])
+    x = logits[1:2].clone().requires_grad_(True)
+    _, w, i = fn(x, 1, 0)
+    w.sum().backward()
+    e = int(i[0, 0])
+    want = [r['grad_logits_row1_top1_unit_grad'][0 if j == e else 1] for j in range(4)]   # by symmetry, whichever expert was taken
+    assert close(x.grad[0], want)
+
+
+def test_torch_oracle_router():
+    _check_router(lambda logits, k, p: oracle.router_forward(logits, torch.eye(logits.shape[1]), k, p or None), False, False)
+
+
 def test_torch_oracle_permute():
     _check_permute(oracle, False)
 
@@ -103,3 +140,9 @@ def test_library_routing():
 def test_library_permute():
     from megablocks_amd.backend import kernels
     _check_permute(kernels, True)
+
+
+@pytest.mark.gpu
+def test_library_router():
+    from megablocks_amd.layers.router import _SoftmaxTopK
+    _check_router(lambda logits, k, p: _SoftmaxTopK.apply(logits, k, p), True, True)
