@@ -217,6 +217,61 @@ def test_router_falls_back_to_torch_for_many_experts():
     assert router.layer.weight.grad is not None and x.grad is not None
 
 
+@pytest.mark.parametrize('name', ['c2', 'c3', 'c4', 'c5'])
+def test_full_size_layer_properties(syn, name):
+    """The benchmark workloads at full size, through properties that do not need an oracle of that size:
+    the backward is linear in the upstream gradient (doubling it doubles every gradient exactly: a power
+    of two commutes with every rounding on the way), and sampled output rows equal the per-token definition
+    sum_j w_j MLP_{e_j}(x_t) computed in fp32."""
+    w = syn.WORKLOADS[name]
+    inp = syn.make_inputs(w, seed=0)
+    layer = syn.build_layer(w, inp)
+    x = inp['x'].to(w.dtype).cuda().requires_grad_(True)
+    grad = inp['grad'].to(w.dtype).cuda()
+    routing_t = None
+    if w.routing != 'router':
+        routing_t = (inp['scores'].to(w.dtype).cuda(), inp['expert_weights'].to(w.dtype).cuda(), inp['top_experts'].cuda())
+    params = [layer.experts.mlp.w1, layer.experts.mlp.w2] + ([layer.experts.mlp.v1] if w.mlp_type == 'glu' else [])
+    if routing_t is None:
+        params.append(layer.router.layer.weight)
+
+    def grads(g):
+        x.grad = None
+        for p in params:
+            p.grad = None
+        out = syn.layer_step(layer, w, x, g, routing_t)
+        return out.detach(), [x.grad.clone()] + [p.grad.clone() for p in params]
+
+    out, g1 = grads(grad)
+    out_again, g2 = grads(grad * 2)
+    assert torch.equal(out, out_again)                                   # same kernels, same order: deterministic
+    for a, b in zip(g1, g2):
+        assert torch.isfinite(a).all() and torch.equal(a * 2, b)
+
+    # sampled rows against the definition
+    with torch.no_grad():
+        if routing_t is None:
+            _, ew, te = layer.router(x)
+        else:
+            ew, te = routing_t[1], routing_t[2]
+        ew, te = ew.view(-1, w.top_k).float(), te.view(-1, w.top_k)
+        w1 = layer.experts.mlp.w1.view(w.experts, w.ffn, w.hidden)
+        w2 = layer.experts.mlp.w2.view(w.experts, w.ffn, w.hidden)
+        v1 = layer.experts.mlp.v1.view(w.experts, w.ffn, w.hidden) if w.mlp_type == 'glu' else None
+        act = w.activation()
+        rows = torch.randperm(w.tokens, generator=torch.Generator().manual_seed(1))[:48].tolist()
+        want = torch.zeros(len(rows), w.hidden, device='cuda')
+        for r, t in enumerate(rows):
+            xt = x[t].float()
+            for j in range(w.top_k):
+                e = int(te[t, j])
+                h = act(w1[e].float() @ xt)
+                if v1 is not None:
+                    h = h * (v1[e].float() @ xt)
+                want[r] += ew[t, j] * (w2[e].float().t() @ h)
+        assert rel_err(out[rows], want) < 2e-2
+
+
 def test_routing_bookkeeping_is_bit_exact(syn):
     from megablocks_amd.layers.arguments import Arguments
     from megablocks_amd.layers.dmoe import ParallelDroplessMLP
