@@ -431,18 +431,41 @@ gmm_generic_kernel(const void* __restrict__ a_, const void* __restrict__ b_, voi
 }
 
 // ---- GELU backward, in place ---------------------------------------------------------
+__device__ __forceinline__ float gelu_tanh_grad(float xv) {   // d/dx gelu_tanh(x), gelu.py:9-13
+  const float t = tanhf(0.79788456f * xv * (1.f + 0.044715f * xv * xv));
+  return 0.5f * xv * ((1.f - t * t) * (0.79788456f + 0.1070322243f * xv * xv)) + 0.5f * (1.f + t);
+}
+
+// elements [first, numel), one per thread and step: the tail of the vector kernel, or everything when the
+// buffers are not 16-byte aligned
 template <int DT>
-__global__ void gelu_backward_kernel(void* __restrict__ g_, const void* __restrict__ x_, int64_t numel) {
+__global__ void gelu_backward_kernel(void* __restrict__ g_, const void* __restrict__ x_, int64_t first, int64_t numel) {
   typedef typename Elem<DT>::type E;
   E* g = (E*)g_;
   const E* x = (const E*)x_;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t i = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (; i < numel; i += stride) {
-    const float xv = Elem<DT>::to_f32(x[i]);
-    const float t = tanhf(0.79788456f * xv * (1.f + 0.044715f * xv * xv));
-    const float ff = 0.5f * xv * ((1.f - t * t) * (0.79788456f + 0.1070322243f * xv * xv)) + 0.5f * (1.f + t);
-    g[i] = Elem<DT>::from_f32(Elem<DT>::to_f32(g[i]) * ff);
+  for (; i < numel; i += stride)
+    g[i] = Elem<DT>::from_f32(Elem<DT>::to_f32(g[i]) * gelu_tanh_grad(Elem<DT>::to_f32(x[i])));
+}
+
+// 16 bytes per lane and step
+template <int DT>
+__global__ void __launch_bounds__(256) gelu_backward_vec_kernel(void* __restrict__ g_, const void* __restrict__ x_, int64_t nvec) {
+  typedef typename Elem<DT>::type E;
+  constexpr int N = 16 / (int)sizeof(E);
+  u32x4* g = (u32x4*)g_;
+  const u32x4* x = (const u32x4*)x_;
+  int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; v < nvec; v += stride) {
+    u32x4 gv = g[v];
+    const u32x4 xv = x[v];
+    E* ge = (E*)&gv;
+    const E* xe = (const E*)&xv;
+#pragma unroll
+    for (int i = 0; i < N; ++i) ge[i] = Elem<DT>::from_f32(Elem<DT>::to_f32(ge[i]) * gelu_tanh_grad(Elem<DT>::to_f32(xe[i])));
+    g[v] = gv;
   }
 }
 
@@ -674,14 +697,28 @@ int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel, 
   if (numel < 0) return MBX_EINVAL;
   if (numel == 0) return 0;
   if (!g || !x) return MBX_EINVAL;
-  int64_t blocks = ceil_div(numel, 256 * 4);
-  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
   hipStream_t s = as_stream(stream);
-  switch (dtype) {
-    case MBX_BF16: gelu_backward_kernel<MBX_BF16><<<(unsigned)blocks, 256, 0, s>>>(g, x, numel); break;
-    case MBX_F16: gelu_backward_kernel<MBX_F16><<<(unsigned)blocks, 256, 0, s>>>(g, x, numel); break;
-    case MBX_F32: gelu_backward_kernel<MBX_F32><<<(unsigned)blocks, 256, 0, s>>>(g, x, numel); break;
-    default: return MBX_EINVAL;
+  const int per_vec = 16 / dtype_bytes(dtype);
+  const int64_t nvec = (aligned16(g) && aligned16(x)) ? numel / per_vec : 0;
+  if (nvec > 0) {
+    int64_t blocks = ceil_div(nvec, 256);
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    switch (dtype) {
+      case MBX_BF16: gelu_backward_vec_kernel<MBX_BF16><<<(unsigned)blocks, 256, 0, s>>>(g, x, nvec); break;
+      case MBX_F16: gelu_backward_vec_kernel<MBX_F16><<<(unsigned)blocks, 256, 0, s>>>(g, x, nvec); break;
+      default: gelu_backward_vec_kernel<MBX_F32><<<(unsigned)blocks, 256, 0, s>>>(g, x, nvec); break;
+    }
+  }
+  const int64_t first = nvec * per_vec;
+  if (first < numel) {
+    int64_t blocks = ceil_div(numel - first, 256);
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    switch (dtype) {
+      case MBX_BF16: gelu_backward_kernel<MBX_BF16><<<(unsigned)blocks, 256, 0, s>>>(g, x, first, numel); break;
+      case MBX_F16: gelu_backward_kernel<MBX_F16><<<(unsigned)blocks, 256, 0, s>>>(g, x, first, numel); break;
+      default: gelu_backward_kernel<MBX_F32><<<(unsigned)blocks, 256, 0, s>>>(g, x, first, numel); break;
+    }
   }
   return launch_status();
 }

@@ -162,12 +162,19 @@ def test_gmm_autograd(gg):
 def test_gelu_backward_inplace():
     from megablocks_amd.layers.gelu import gelu_backward_
     for dtype in (torch.bfloat16, torch.float16, torch.float32):
-        x = torch.randn(1000, 257).to(dtype)
-        g = torch.randn(1000, 257).to(dtype)
-        want = oracle.gelu_tanh_backward(g.float(), x.float())
-        gd = g.cuda()
-        out = gelu_backward_(gd, x.cuda())
-        assert out is gd and rel_err(gd.cpu().float(), want) < (1e-5 if dtype == torch.float32 else 1e-2)
+        for shape in ((1000, 257), (1003,), (5,)):            # whole 16-byte vectors; a tail; less than one vector
+            x = torch.randn(*shape).to(dtype)
+            g = torch.randn(*shape).to(dtype)
+            want = oracle.gelu_tanh_backward(g.float(), x.float())
+            gd = g.cuda()
+            out = gelu_backward_(gd, x.cuda())
+            assert out is gd and rel_err(gd.cpu().float(), want) < (1e-5 if dtype == torch.float32 else 1e-2)
+        # buffers that are not 16-byte aligned: element by element, same values
+        x, g = torch.randn(4100).to(dtype), torch.randn(4100).to(dtype)
+        aligned = gelu_backward_(g.cuda()[8:].clone(), x.cuda()[8:].clone())
+        base = g.cuda()
+        gelu_backward_(base[1:], x.cuda()[1:])
+        assert torch.equal(base[8:], aligned) and torch.equal(base[:1].cpu(), g[:1])
 
 
 DMA_EDGE = [  # groups, rows, k, n: shapes that take the direct-to-LDS kernels, off every tile boundary
