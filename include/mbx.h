@@ -147,7 +147,7 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
  *   MBX_NN: c[r_e] = a[r_e] @ b[e] + a2[r_e] @ b2[e]      MBX_NT: ... @ b[e]^T + ... @ b2[e]^T
  * with a2 / b2 shaped like a / b.  One rounding of the fp32 sum instead of the reference's three.
  * Handles bf16 / f16 with k a multiple of 64 and at least 256, 16-byte aligned operands (n a multiple
- * of 8 for MBX_NN) below 2 GiB each; anything else returns MBX_EUNSUPPORTED and the caller issues the
+ * of 8 for MBX_NN), any number of rows, one expert's weights below 2 GiB; anything else returns MBX_EUNSUPPORTED and the caller issues the
  * two mbx_gmm calls and the addition itself. */
 int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype,
                  const int32_t* bins, int num_groups, int64_t rows, int k, int n, int layout,

@@ -541,7 +541,7 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
   return (int)(need < cus[dev] ? need : cus[dev]);
 }
 
-// Launch of the direct-to-LDS kernels (k a multiple of 64 for NN / NT, operands below 2 GiB).
+// Launch of the direct-to-LDS kernels (k a multiple of 64 for NN / NT; sizes as dma_sizes_ok() allows).
 // TS is the tile the tail of an NN / NT launch is cut into (TS = T: never cut).
 // a2 / b2 non-null (NN / NT only): c = a @ b[e] + a2 @ b2[e], the second pair shaped like the first.
 template <int DT, typename T, typename TS>
@@ -556,7 +556,10 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   if (layout == MBX_TN) {
     constexpr size_t lds = T::LDS_BYTES;
     const int tiles_m = (int)ceil_div(k, T::BM), tiles_n = (int)ceil_div(n, T::BN);
-    auto kern = dma::gmm_tn_kernel<DT, T>;
+    // rows per segment of a reduction: each operand's share stays below 2 GiB (whole K tiles)
+    const int64_t seg_rows = (((int64_t)1 << 31) - 1) / ((int64_t)(k > n ? k : n) * 2) / T::BK * T::BK;
+    const bool segmented = rows > seg_rows;
+    auto kern = segmented ? dma::gmm_tn_kernel<DT, T, true> : dma::gmm_tn_kernel<DT, T, false>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
     // short reductions (few rows per expert): several tiles per workgroup
@@ -564,7 +567,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     const int chunk = avg_rows >= 1024 ? 1 : avg_rows >= 512 ? 2 : 4;
     const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups, chunk);
     if (grid > 0x7fffffff) return MBX_ERANGE;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n, chunk);
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n, chunk, (int)seg_rows);
     return launch_status();
   }
   constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
@@ -601,6 +604,15 @@ int gmm_generic(const void* a, const void* b, void* c, const int32_t* bins, int 
 }
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// The direct-to-LDS kernels address with 32-bit byte offsets from a base they set per tile (the tile's first
+// row of a and c in NN / NT), per expert (its weights; its [k, n] product in TN) or per segment of an
+// expert's rows (TN), so the row count is free; what has to stay below 2 GiB is one expert's weight matrix
+// or product and 256 rows of any operand (a 64-row K tile in TN).
+static inline bool dma_sizes_ok(int k, int n) {
+  const int64_t lim = (int64_t)1 << 31;
+  return (int64_t)k * n * 2 < lim && (int64_t)k * 2 * TileDma::BM < lim && (int64_t)n * 2 * TileDma::BM < lim;
+}
 
 // NN / NT: whether to tile a launch with the half-height tile only.  With about one such tile per expert
 // (up to 144 rows on average) the full tile would mostly multiply padding.  Up to 320 rows the mix of
@@ -645,9 +657,8 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
   if (layout == MBX_NN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (layout == MBX_TN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (fast) {
-    // direct-to-LDS kernels: whole K tiles (NN / NT) and 32-bit byte offsets inside each operand
-    const int64_t lim = (int64_t)1 << 31;
-    bool dma_ok = rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
+    // direct-to-LDS kernels: whole K tiles (NN / NT)
+    bool dma_ok = dma_sizes_ok(k, n);
     if (layout != MBX_TN) dma_ok = dma_ok && k % TileDma::BK == 0;
     if (dma_ok) {
       // TN: the half-height tile only when the product has at most 128 rows (it is slower otherwise)
@@ -678,10 +689,8 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
   if (!bins || !c || (k > 0 && (!a || !b || !a2 || !b2))) return MBX_EINVAL;
   if (rows > 0x7fffffff) return MBX_ERANGE;
   // only the direct-to-LDS kernels reduce over two operand pairs: whole K tiles, at least four per pair
-  const int64_t lim = (int64_t)1 << 31;
   const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(a2) && aligned16(b2) &&
-                  k % TileDma::BK == 0 && k >= 4 * TileDma::BK && (layout == MBX_NT || n % 8 == 0) &&
-                  rows * k * 2 < lim && (int64_t)k * n * 2 < lim && rows * n * 2 < lim;
+                  k % TileDma::BK == 0 && k >= 4 * TileDma::BK && (layout == MBX_NT || n % 8 == 0) && dma_sizes_ok(k, n);
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   const bool small_m = half_height_only(rows, num_groups, n);

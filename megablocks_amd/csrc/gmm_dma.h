@@ -177,17 +177,14 @@ struct Args {
   int nk1;
 };
 
-// acc (+)= A_tile * B_tile over all K tiles, then c[m][n] = acc for m < m_lim, n < n_lim, where
-// m = m_base + (row inside the tile) and n = n_base + (column inside the tile).
+// acc = (clear ? 0 : acc) + A_tile * B_tile over all K tiles.  On return no load is in flight and no LDS
+// read is pending, but other waves may still be reading the last stages.
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
-__device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
-                                           int n_base, int n_lim, char* lds_generic) {
+__device__ __forceinline__ void block_multiply(const Args& g, f32x16 (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
-
-  f32x16 acc[T::TM][T::TN];
 
   constexpr int BK = T::BK, SA = T::SA, SB = T::SB, LA = T::LA, LB = T::LB;
   static_assert(T::KS == 4, "the schedule below is written for four k-steps per K tile");
@@ -330,7 +327,7 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
     issue_group(true, SB - 1, SB - 1, 0, LB / 2);
   }
   __builtin_amdgcn_sched_barrier(0);   // the loads are on their way before the accumulators are cleared
-  clear_acc();
+  if (clear) clear_acc();
   if (nk > 0) {
     wait_vmcnt<WAIT_PROLOGUE>();
     __builtin_amdgcn_s_barrier();
@@ -391,7 +388,17 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
 #undef MBX_WAIT_FRAGS
 #undef MBX_READ_ONE
 #undef MBX_STEP
+}
 
+// c[m][n] = acc for m < m_lim, n < n_lim, where m = m_base + (row inside the tile) and
+// n = n_base + (column inside the tile).  Uses the LDS of the operand rings as a staging buffer.
+template <int DT, typename T>
+__device__ __forceinline__ void block_store(const f32x16 (&acc)[T::TM][T::TN], uint16_t* __restrict__ c, int64_t ldc,
+                                            int m_base, int m_lim, int n_base, int n_lim, char* lds_generic) {
+  const lds_ptr lds = (lds_ptr)lds_generic;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
+  const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
   // accumulator (i, j), register r of lane l holds c[m][n] with
   //   m = m_base + wm + 32 i + (l % 32),  n = n_base + wn + 32 j + 8 (r / 4) + 4 (l / 32) + (r % 4)
   if ((ldc % 8 == 0) && (((uintptr_t)c & 15u) == 0)) {
@@ -490,6 +497,20 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
       }
     }
   }
+}
+
+// c = A_tile * B_tile over all K tiles (the whole product of one output tile)
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
+__device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
+                                           int n_base, int n_lim, char* lds) {
+  f32x16 acc[T::TM][T::TN];
+  block_multiply<DT, A_MC, B_MC, T, DUAL>(g, acc, true, lds);
+  block_store<DT, T>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds);
+}
+
+// Buffer sizes stay below 2 GiB: bit 31 of a byte offset marks a load that must fetch nothing.
+__device__ __forceinline__ uint32_t clip_bytes(int64_t bytes) {
+  return (uint32_t)(bytes < 0x7fffffff ? bytes : 0x7fffffff);
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
@@ -602,12 +623,11 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   const int big_rounds = full_rounds + ((rest > 0 && !split) ? 1 : 0);
 
   Args g;
-  g.rsrc_a = make_rsrc(a, (uint32_t)(rows * k * 2));
   g.a_ld_bytes = (uint32_t)k * 2;
   g.b_ld_bytes = (uint32_t)(B_MC ? n : k) * 2;
   g.nk1 = k / T::BK;
   g.nk = DUAL ? 2 * g.nk1 : g.nk1;
-  g.rsrc_a2 = DUAL ? make_rsrc(a2, (uint32_t)(rows * k * 2)) : g.rsrc_a;
+  g.a_r0 = 0;   // the buffers of a and c start at the tile's first row: byte offsets stay small whatever the row count
   // Work items of this workgroup: one tile per round, then (if the tail is split) one half tile.
   const int items = big_rounds + ((kSplit && split) ? 1 : 0);
   for (int r = 0; r < items; ++r) {
@@ -627,17 +647,21 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     }
     int e, start, end, tm, tn;
     tiles.find(id, e, start, end, tm, tn);
-    g.a_r0 = start + tm * T::BM + half * TS::BM;
-    if (g.a_r0 >= end) break;             // the second half of a tile whose rows end in the first (a last item)
+    const int row0 = start + tm * T::BM + half * TS::BM;
+    if (row0 >= end) break;               // the second half of a tile whose rows end in the first (a last item)
+    const uint32_t a_bytes = clip_bytes((rows - row0) * k * 2);   // rows past the tile's are fetched, never stored
+    g.rsrc_a = make_rsrc(a + (int64_t)row0 * k, a_bytes);
+    g.rsrc_a2 = DUAL ? make_rsrc(a2 + (int64_t)row0 * k, a_bytes) : g.rsrc_a;
     g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
     g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
     g.b_r0 = tn * T::BN;
+    uint16_t* const c_tile = c + (int64_t)row0 * n;
     // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
-    use_ts = kSplit && (use_ts || end - g.a_r0 <= TS::BM);
+    use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
     if (use_ts) {
-      block_gemm<DT, false, B_MC, TS, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+      block_gemm<DT, false, B_MC, TS, DUAL>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds);
     } else {
-      block_gemm<DT, false, B_MC, T, DUAL>(g, c, n, g.a_r0, end, g.b_r0, n, lds);
+      block_gemm<DT, false, B_MC, T, DUAL>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds);
     }
     tile_done();
   }
@@ -666,10 +690,13 @@ static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chun
   return (per_xcd * num_groups + chunk - 1) / chunk * kXcds;
 }
 
-template <int DT, typename T>
+// SEGMENTED: an expert's rows of a or b may reach 2 GiB (the launch passes seg_rows, the number of rows that
+// stays below it); otherwise the whole of a and b is smaller than that.
+template <int DT, typename T, bool SEGMENTED>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
-              const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk) {
+              const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk,
+              int seg_rows) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int bm = tn_block_m(tiles_m), bn = tn_block_n(tiles_n);
   const int blocks_m = (tiles_m + bm - 1) / bm, blocks_n = (tiles_n + bn - 1) / bn;
@@ -712,14 +739,33 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
     int e = slot;
     if (ranked) e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(__ballot(rank == slot)));
     const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
-    const int64_t group_rows = end - start;
-    // the buffers cover exactly the rows of this expert: later rows read as zero
-    g.rsrc_a = make_rsrc(a + (int64_t)start * k, (uint32_t)(group_rows * k * 2));
     g.a_r0 = tm * T::BM;
-    g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
     g.b_r0 = tn * T::BN;
-    g.nk = (int)((group_rows + T::BK - 1) / T::BK);
-    block_gemm<DT, true, true, T>(g, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
+    if constexpr (!SEGMENTED) {
+      // the buffers cover exactly the rows of this expert: later rows read as zero
+      const int64_t group_rows = end - start;
+      g.rsrc_a = make_rsrc(a + (int64_t)start * k, (uint32_t)(group_rows * k * 2));
+      g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
+      g.nk = (int)((group_rows + T::BK - 1) / T::BK);
+      block_gemm<DT, true, true, T>(g, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
+    } else {
+      // The reduction runs over the expert's rows in segments of at most seg_rows rows, each with buffers
+      // of its own that cover exactly its rows.
+      f32x16 acc[T::TM][T::TN];
+      int first = start;
+      for (;;) {
+        const int64_t left = end - first;
+        const int64_t seg = left < seg_rows ? left : seg_rows;
+        g.rsrc_a = make_rsrc(a + (int64_t)first * k, (uint32_t)(seg * k * 2));
+        g.rsrc_b = make_rsrc(b + (int64_t)first * n, (uint32_t)(seg * n * 2));
+        g.nk = (int)((seg + T::BK - 1) / T::BK);
+        block_multiply<DT, true, true, T>(g, acc, first == start, lds);
+        if (left <= seg_rows) break;
+        first += seg_rows;
+        tile_done();   // the first stages are refilled next
+      }
+      block_store<DT, T>(acc, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
+    }
     tile_done();
   }
 }

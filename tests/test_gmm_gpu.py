@@ -325,6 +325,63 @@ def test_gmm_dual_is_the_sum_of_two_products(gg, groups, rows, k, n, single, tra
         gg.gmm_dual(a, b, a2[:, :-8], b2, sizes, trans_b=trans_b)
 
 
+def _ref_in_pieces(check, a, b, sizes, trans_a, trans_b, got):
+    """Compare `got` with the fp32 product expert by expert (an fp32 copy of a whole operand of several GiB
+    at once is not needed then); `check(piece_of_got, reference_piece)`."""
+    start = 0
+    for e, n in enumerate(sizes.tolist()):
+        ae = a[start:start + n].float()
+        if trans_a and n:
+            check(got[e], ae.t() @ b[start:start + n].float())
+        elif n:
+            check(got[start:start + n], ae @ (b[e].float().t() if trans_b else b[e].float()))
+        start += n
+
+
+LARGE = [  # name, rows per expert, k, n: the [rows, k] or the [rows, n] matrix (or one expert's share of it) of 2 .. 5 GiB
+    ('rows-by-k-2.3GiB', [150000, 0, 100000, 50000], 4096, 256),
+    ('rows-by-n-2.3GiB', [150000, 0, 100000, 50000], 256, 4096),
+    ('one-expert-4.3GiB-of-4.6GiB', [20000, 560000, 20], 4096, 128),
+]
+
+
+@pytest.mark.parametrize('name,rows_per_expert,k,n', LARGE, ids=[c[0] for c in LARGE])
+def test_gmm_operands_beyond_2GiB(gg, name, rows_per_expert, k, n):
+    """Byte offsets inside the big matrices pass 2^31 and 2^32: same kernels, same tolerance."""
+    from megablocks_amd import _lib
+    sizes = torch.tensor(rows_per_expert)
+    rows, groups = int(sizes.sum()), len(rows_per_expert)
+    torch.manual_seed(rows % 1000)
+    a = torch.empty(rows, k, device='cuda', dtype=torch.bfloat16).normal_()
+    a2 = a.flip(0)
+    w_nn = torch.empty(groups, k, n, device='cuda', dtype=torch.bfloat16).normal_(std=0.1)
+    w_nt = torch.empty(groups, n, k, device='cuda', dtype=torch.bfloat16).normal_(std=0.1)
+    b_tn = torch.empty(rows, n, device='cuda', dtype=torch.bfloat16).normal_()
+    assert max(a.numel(), b_tn.numel()) * 2 >= 2 ** 31
+
+    def check(got, ref):
+        assert rel_err(got, ref) < TOL and max_block_err(got, ref, bm=256, bn=256) < 2 * TOL
+
+    _lib.profile_hook = []
+    try:
+        nn = gg.backend.gmm(a, w_nn, sizes)
+        nt = gg.backend.gmm(a, w_nt, sizes, trans_b=True)
+        tn = gg.backend.gmm(a, b_tn, sizes, trans_a=True)
+        dual = gg.gmm_dual(a, w_nn, a2, w_nn, sizes) if k >= 256 else None
+        names = [r[0] for r in _lib.profile_hook]
+    finally:
+        _lib.profile_hook = None
+    _ref_in_pieces(check, a, w_nn, sizes, False, False, nn)
+    _ref_in_pieces(check, a, w_nt, sizes, False, True, nt)
+    _ref_in_pieces(check, a, b_tn, sizes, True, False, tn)
+    assert torch.count_nonzero(tn[[i for i, s in enumerate(rows_per_expert) if s == 0]]) == 0
+    if dual is not None:
+        assert names[-1] == 'gmm_nn_dual'            # one launch, not two products and a sum
+        second = gg.backend.gmm(a2, w_nn, sizes)
+        _ref_in_pieces(check, a2, w_nn, sizes, False, False, second)
+        assert rel_err(dual, nn.float() + second.float()) < TOL
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize('act_name', ['silu', 'gelu_tanh'])
 def test_fused_gated_activation_matches_the_two_step_formulation(dtype, act_name):

@@ -294,6 +294,36 @@ def test_full_size_round_trip_properties(ops):
     assert torch.equal(back, x)
 
 
+def test_permutation_of_more_than_4GiB(ops):
+    """Routed rows of 2.5e9 elements (4.9 GB in bf16): element offsets pass 2^31, byte offsets 2^32.  Same
+    size-independent properties, plus the padded forms and the weight gradient on a slice."""
+    T, h, E, k = 300000, 2048, 16, 4
+    x = torch.empty(T, h, device='cuda', dtype=torch.bfloat16).normal_()
+    top = torch.randint(0, E, (T * k,), device='cuda').int()
+    bin_ids, indices = ops.sort(top, 4)
+    tpe = ops.histogram(top, E)
+    bins = ops.inclusive_cumsum(tpe, 0)
+    pbins = ops.inclusive_cumsum(ops.round_up(tpe, 128), 0)
+    rows = indices.long() // k
+    g = ops.gather(x, indices, bin_ids, bins, k)
+    assert g.numel() > 2 ** 31
+    for lo in range(0, T * k, 200000):                                             # piecewise: no second 4.9 GB copy
+        assert torch.equal(g[lo:lo + 200000], x[rows[lo:lo + 200000]])
+    half = torch.full((T * k,), 0.25, device='cuda').bfloat16()
+    assert torch.equal(ops.scatter(g, indices, bin_ids, half, bins, k), x)         # 4 x 0.25 x == x exactly
+    del g
+    gp = ops.padded_gather(x, indices, bin_ids, bins, pbins, k)
+    assert gp.shape[0] == int(pbins[-1])
+    assert torch.equal(ops.padded_scatter(gp, indices, bin_ids, half, bins, pbins, k), x)
+    # the last expert's rows sit past the 2^32-byte mark; padding rows are zero
+    first, last, end = int(pbins[-2]), int(pbins[-2]) + int(tpe[-1]), int(pbins[-1])
+    assert torch.equal(gp[first:last], x[rows[int(bins[-2]):]]) and torch.count_nonzero(gp[last:end]) == 0
+    from megablocks_amd.backend import kernels
+    wgrad = kernels.padded_scatter_wgrad(gp, x, indices, bin_ids, bins, pbins, k)   # <x_t, x_t> for every slot
+    want = x.float().pow(2).sum(1).repeat_interleave(k)
+    assert rel_err(wgrad, want) < 1e-2 and torch.allclose(wgrad.float(), want, rtol=2e-2)
+
+
 # ------------------------------------------------------------------ the routing chain against the C oracle
 @pytest.mark.parametrize('tokens,experts,top_k', [(8192, 8, 2), (16384, 64, 1), (32768, 64, 6), (24576, 16, 4), (7, 3, 2)])
 def test_routing_chain_matches_the_c_restatement(ops, tokens, experts, top_k):
