@@ -358,6 +358,50 @@ def test_dmoe_equals_capacity_moe_without_dropping(bs, sl, hs, ne, top_k, mlp_im
     assert rel_err(dmoe_layer(x), moe_layer(x)) < 1e-2
 
 
+@pytest.mark.parametrize('bs,sl,hs', [(16, 1, 128), (1, 16, 128), (16, 16, 128), (8, 8, 256), (2, 256, 512)])
+def test_single_expert_capacity_moe_is_dense_ffn(bs, sl, hs):
+    # tests/layers/moe_test.py:155-199: forward, and the gradients of both weight matrices
+    from megablocks_amd.layers.moe import MoE
+    torch.manual_seed(42)
+    layer = MoE(_args(hidden_size=hs, ffn_hidden_size=2 * hs, moe_capacity_factor=1))
+    x = torch.randn(sl, bs, hs, device='cuda').bfloat16().requires_grad_(True)
+    out = layer(x)
+    out.sum().backward()
+    m = layer.experts.mlp
+    xf = x.detach().view(-1, hs).float().requires_grad_(True)
+    w1, w2 = m.w1.detach().float().requires_grad_(True), m.w2.detach().float().requires_grad_(True)
+    want = F.gelu(xf @ w1[0], approximate='tanh') @ w2[0]
+    want.sum().backward()
+    assert out.shape == x.shape and rel_err(out.view(-1, hs), want) < 1e-2
+    assert rel_err(m.w1.grad, w1.grad) < 1e-2 and rel_err(m.w2.grad, w2.grad) < 1e-2
+    assert rel_err(x.grad.view(-1, hs), xf.grad) < 1e-2
+
+
+@pytest.mark.parametrize('tokens,hs,ne,top_k,capacity_factor', [(256, 128, 4, 1, 1.0), (512, 128, 8, 2, 0.5),
+                                                                 (1024, 256, 16, 4, 1.0), (300, 64, 3, 2, 0.75)])
+def test_capacity_moe_with_dropped_tokens_vs_oracle(tokens, hs, ne, top_k, capacity_factor):
+    """moe.py:185-235 on the oracle's binned gather / scatter with fp32 expert products: tokens beyond an
+    expert's capacity contribute nothing, the others their weighted expert output."""
+    from megablocks_amd.layers.moe import MoE
+    torch.manual_seed(tokens)
+    layer = MoE(_args(hidden_size=hs, ffn_hidden_size=2 * hs, moe_num_experts=ne, moe_top_k=top_k,
+                      moe_capacity_factor=capacity_factor))
+    x = torch.randn(tokens, 1, hs, device='cuda').bfloat16()
+    out = layer(x)
+    with torch.no_grad():
+        _, weights, top = layer.router(x)
+    weights, top = weights.flatten().cpu(), top.flatten().cpu().int()
+    indices, _, bins, tpe = oracle.indices_and_bins(top, ne)
+    capacity = int(capacity_factor * top_k * tokens / ne)
+    assert int(tpe.max()) > capacity                               # something is dropped
+    xb = oracle.binned_gather(x.view(tokens, hs).cpu(), indices, None, bins, capacity, top_k).float()
+    m = layer.experts.mlp
+    h = F.gelu(torch.bmm(xb, m.w1.detach().float().cpu()), approximate='tanh')
+    yb = torch.bmm(h, m.w2.detach().float().cpu())
+    want = oracle.binned_scatter(yb, indices, weights.float(), bins, top_k)
+    assert rel_err(out.view(tokens, hs), want) < 1e-2
+
+
 def test_forward_shapes_bias_and_losses():
     # tests/layers/dmoe_test.py:103-188
     from megablocks_amd.layers import moe, router
