@@ -40,6 +40,8 @@ def parse():
     ap.add_argument('--tokens', type=int, default=None, help='override the token count (not the headline number)')
     ap.add_argument('--memory-optimized', action='store_true')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
+    ap.add_argument('--graph', action='store_true',
+                    help='capture the step (forward + backward) in a HIP graph after the warm-up and time replays of it')
     ap.add_argument('--cpu-tokens', type=int, default=None)
     ap.add_argument('--library-gemm', action='store_true',
                     help='also time the three grouped products as per-expert torch.matmul loops (the vendor GEMM library)')
@@ -79,11 +81,29 @@ def gpu_leg(args, w, inp):
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    timed_step = step
+    if args.graph:
+        if w.mlp_impl == 'sparse':
+            sys.exit('bench.py: --graph needs a step without host synchronisation; the block-sparse mode reads the '
+                     'padded row count on the host (as the reference does, kernels.py:123-124)')
+        step()                      # leaves the gradients unset: the captured step allocates them in the graph's pool
+        x.grad = None
+        if routing is not None:
+            routing[1].grad = None
+        for p in layer.parameters():
+            p.grad = None
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            synthetic.layer_step(layer, w, x, grad, routing)
+        timed_step = graph.replay
+        for _ in range(3):
+            timed_step()
+        torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for _ in range(args.steps):
-        step()
+        timed_step()
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -300,7 +320,7 @@ def main():
         'data': 'synthetic',
         'config': {'workload': f'{w.name}: {w.description}', 'tokens': w.tokens, 'hidden': w.hidden, 'ffn': w.ffn,
                    'experts': w.experts, 'top_k': w.top_k, 'mlp_type': w.mlp_type, 'mlp_impl': w.mlp_impl,
-                   'routing': w.routing, 'memory_optimized_mlp': args.memory_optimized},
+                   'routing': w.routing, 'memory_optimized_mlp': args.memory_optimized, 'graph_replay': args.graph},
         'roofline': roofline,
         'gemm': {'ms_per_step': round(gemm_ms, 4), 'tflops_all_launches': round(all_gemm_tflops, 1),
                  'frac_of_mfma_peak': round(all_gemm_tflops * 1e12 / MFMA_PEAK[dn], 4), 'kernels': gemm},

@@ -402,6 +402,48 @@ def test_capacity_moe_with_dropped_tokens_vs_oracle(tokens, hs, ne, top_k, capac
     assert rel_err(out.view(tokens, hs), want) < 1e-2
 
 
+@pytest.mark.parametrize('mlp_type,tokens,hs,ffn,ne,top_k,memory_optimized',
+                         [('mlp', 2048, 1024, 4096, 64, 1, False), ('glu', 1024, 512, 1408, 8, 2, False),
+                          ('glu', 1000, 256, 512, 4, 2, True)])
+def test_dmoe_step_replays_from_a_captured_graph(mlp_type, tokens, hs, ffn, ne, top_k, memory_optimized):
+    """The grouped dMoE step (forward + backward) has no host synchronisation and the library allocates
+    nothing, so it can be captured once and replayed: every replay, with new inputs in the static buffers and
+    eager work in between, gives bit for bit what the eager step gives."""
+    from megablocks_amd.layers.dmoe import dMoE
+    torch.manual_seed(tokens)
+    layer = dMoE(_args(hidden_size=hs, ffn_hidden_size=ffn, moe_num_experts=ne, moe_top_k=top_k, mlp_type=mlp_type,
+                       memory_optimized_mlp=memory_optimized, moe_normalize_expert_weights=1 if top_k > 1 else None))
+    params = list(layer.parameters())
+    xs = [torch.randn(tokens, 1, hs, device='cuda').bfloat16() for _ in range(3)]
+    gs = [torch.randn(tokens, 1, hs, device='cuda').bfloat16() for _ in range(3)]
+
+    def eager(x, g):
+        layer.zero_grad(set_to_none=True)
+        x = x.clone().requires_grad_(True)
+        out = layer(x)
+        out.backward(g)
+        return [out.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in params]
+
+    want = [eager(x, g) for x, g in zip(xs, gs)]
+    static_x, static_g = xs[0].clone().requires_grad_(True), gs[0].clone()
+    layer.zero_grad(set_to_none=True)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = layer(static_x)
+        static_out.backward(static_g)
+    static_results = [static_out.detach(), static_x.grad] + [p.grad for p in params]
+    for i in (1, 2, 0, 1, 2, 0):
+        static_x.detach().copy_(xs[i])
+        static_g.copy_(gs[i])
+        for t in static_results:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip(static_results, want[i]):
+            assert torch.equal(got, ref)
+        eager(xs[(i + 1) % 3], gs[i])                               # eager work between the replays
+
+
 def test_forward_shapes_bias_and_losses():
     # tests/layers/dmoe_test.py:103-188
     from megablocks_amd.layers import moe, router
