@@ -444,6 +444,20 @@ def test_dmoe_step_replays_from_a_captured_graph(mlp_type, tokens, hs, ffn, ne, 
         eager(xs[(i + 1) % 3], gs[i])                               # eager work between the replays
 
 
+@pytest.mark.parametrize('mlp_impl', ['grouped', 'sparse'])
+@pytest.mark.parametrize('tokens', [0, 1])
+def test_dmoe_with_no_tokens_and_with_one(mlp_impl, tokens):
+    from megablocks_amd.layers.dmoe import dMoE
+    layer = dMoE(_args(moe_num_experts=4, moe_top_k=2, mlp_impl=mlp_impl))
+    x = torch.randn(tokens, 1, 128, device='cuda').bfloat16().requires_grad_(True)
+    out = layer(x)
+    out.sum().backward()
+    assert out.shape == x.shape and x.grad.shape == x.shape
+    assert all(p.grad is not None and p.grad.shape == p.shape for p in layer.parameters())
+    if tokens == 0:
+        assert all(torch.count_nonzero(p.grad) == 0 for p in layer.parameters())
+
+
 def test_forward_shapes_bias_and_losses():
     # tests/layers/dmoe_test.py:103-188
     from megablocks_amd.layers import moe, router

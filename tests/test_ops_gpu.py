@@ -294,6 +294,37 @@ def test_full_size_round_trip_properties(ops):
     assert torch.equal(back, x)
 
 
+def test_empty_and_degenerate_inputs(ops, kernels):
+    """No tokens, no capacity, one column: shapes as the reference's wrappers give them, nothing launched wrongly."""
+    from megablocks_amd import grouped_gemm_util as gg
+    none = dev(torch.empty(0, dtype=torch.int32))
+    bins = dev(torch.zeros(4, dtype=torch.int32))
+    x = dev(torch.empty(0, 64).bfloat16())
+    assert ops.gather(x, none, none, bins, 1).shape == (0, 64)
+    assert ops.scatter(x, none, none, None, bins, 1).shape == (0, 64)
+    assert ops.padded_gather(x, none, none, bins, bins, 1).shape == (0, 64)
+    assert ops.padded_scatter(x, none, none, None, bins, bins, 1).shape == (0, 64)
+    full = ops.binned_gather(x, none, bins, 8, 1)
+    assert full.shape == (4, 8, 64) and torch.count_nonzero(full) == 0
+    assert ops.binned_scatter(dev(torch.empty(4, 0, 64).bfloat16()), none, None, bins, 1).shape == (0, 64)
+    assert kernels.scatter_wgrad(x, x, none, none, bins, 1).shape == (0,)
+    assert ops.inclusive_cumsum(dev(torch.empty(3, 0, dtype=torch.int32)), 1).shape == (3, 0)
+    assert ops.inclusive_cumsum(dev(torch.tensor([5], dtype=torch.int32)), 0).shape == ()     # the squeeze of ops/cumsum.py:24-48
+    assert ops.replicate(dev(torch.tensor([[1, 2]], dtype=torch.int32)), dev(torch.tensor([0, 0], dtype=torch.int32)), 0).shape == (1, 0)
+    assert ops.topology(dev(torch.tensor([0, 0], dtype=torch.int32)), 128, 0, 4).shape == (0,)
+    one_col = dev(torch.tensor([[1.], [2.], [3.]]).bfloat16())
+    got = ops.gather(one_col, dev(torch.tensor([2, 0, 1], dtype=torch.int32)), dev(torch.tensor([0, 0, 1], dtype=torch.int32)),
+                     dev(torch.tensor([2, 3], dtype=torch.int32)), 1)
+    assert got.view(-1).tolist() == [3.0, 1.0, 2.0]
+    sizes = torch.tensor([0, 0])
+    w = dev(torch.randn(2, 64, 32).bfloat16())
+    assert gg.backend.gmm(x, w, sizes).shape == (0, 32)
+    dw = gg.backend.gmm(x, dev(torch.empty(0, 32).bfloat16()), sizes, trans_a=True)
+    assert dw.shape == (2, 64, 32) and torch.count_nonzero(dw) == 0                       # no rows: zero gradients
+    no_k = gg.backend.gmm(dev(torch.empty(8, 0).bfloat16()), dev(torch.empty(2, 0, 32).bfloat16()), torch.tensor([4, 4]))
+    assert no_k.shape == (8, 32) and torch.count_nonzero(no_k) == 0                       # empty reduction: zeros
+
+
 def test_permutation_of_more_than_4GiB(ops):
     """Routed rows of 2.5e9 elements (4.9 GB in bf16): element offsets pass 2^31, byte offsets 2^32.  Same
     size-independent properties, plus the padded forms and the weight gradient on a slice."""
