@@ -554,12 +554,15 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const bool dual = a2 != nullptr;
   uint16_t* cp = (uint16_t*)c;
   if (layout == MBX_TN) {
-    constexpr size_t lds = T::LDS_BYTES;
+    constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
     const int tiles_m = (int)ceil_div(k, T::BM), tiles_n = (int)ceil_div(n, T::BN);
     // rows per segment of a reduction: each operand's share stays below 2 GiB (whole K tiles)
     const int64_t seg_rows = (((int64_t)1 << 31) - 1) / ((int64_t)(k > n ? k : n) * 2) / T::BK * T::BK;
     const bool segmented = rows > seg_rows;
-    auto kern = segmented ? dma::gmm_tn_kernel<DT, T, true> : dma::gmm_tn_kernel<DT, T, false>;
+    // the last row tile of the product as a TS tile when it is at most half full
+    const bool mixed = T::BM != TS::BM && k % T::BM != 0 && k % T::BM <= TS::BM;
+    auto kern = mixed ? (segmented ? dma::gmm_tn_kernel<DT, T, TS, true> : dma::gmm_tn_kernel<DT, T, TS, false>)
+                      : (segmented ? dma::gmm_tn_kernel<DT, T, T, true> : dma::gmm_tn_kernel<DT, T, T, false>);
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
     // short reductions (few rows per expert): several tiles per workgroup

@@ -690,14 +690,52 @@ static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chun
   return (per_xcd * num_groups + chunk - 1) / chunk * kXcds;
 }
 
+// One output tile of expert e's product: rows [g.a_r0, g.a_r0 + TT::BM) x columns [g.b_r0, g.b_r0 + TT::BN) of
+// c[e] = a[start:end]^T @ b[start:end].
+template <int DT, typename TT, bool SEGMENTED>
+__device__ __forceinline__ void tn_tile(Args& g, const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
+                                        uint16_t* __restrict__ c_e, int start, int end, int k, int n, int seg_rows,
+                                        char* lds) {
+  if constexpr (!SEGMENTED) {
+    // the buffers cover exactly the rows of this expert: later rows read as zero
+    const int64_t group_rows = end - start;
+    g.rsrc_a = make_rsrc(a + (int64_t)start * k, (uint32_t)(group_rows * k * 2));
+    g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
+    g.nk = (int)((group_rows + TT::BK - 1) / TT::BK);
+    block_gemm<DT, true, true, TT>(g, c_e, n, g.a_r0, k, g.b_r0, n, lds);
+  } else {
+    // The reduction runs over the expert's rows in segments of at most seg_rows rows, each with buffers
+    // of its own that cover exactly its rows.
+    f32x16 acc[TT::TM][TT::TN];
+    int first = start;
+    for (;;) {
+      const int64_t left = end - first;
+      const int64_t seg = left < seg_rows ? left : seg_rows;
+      g.rsrc_a = make_rsrc(a + (int64_t)first * k, (uint32_t)(seg * k * 2));
+      g.rsrc_b = make_rsrc(b + (int64_t)first * n, (uint32_t)(seg * n * 2));
+      g.nk = (int)((seg + TT::BK - 1) / TT::BK);
+      block_multiply<DT, true, true, TT>(g, acc, first == start, lds);
+      if (left <= seg_rows) break;
+      first += seg_rows;
+      tile_done();   // the first stages are refilled next
+    }
+    block_store<DT, TT>(acc, c_e, n, g.a_r0, k, g.b_r0, n, lds);
+  }
+}
+
+// TS: the tile for the last row tile of a product when at most TS::BM of its rows exist (k % T::BM in
+// (0, TS::BM]; half the work; tiles are handed out as compute units become free, so unequal tiles balance);
+// TS = T switches this off.
 // SEGMENTED: an expert's rows of a or b may reach 2 GiB (the launch passes seg_rows, the number of rows that
 // stays below it); otherwise the whole of a and b is smaller than that.
-template <int DT, typename T, bool SEGMENTED>
+template <int DT, typename T, typename TS, bool SEGMENTED>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk,
               int seg_rows) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
+  static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "last-row tile");
+  constexpr bool kMixed = T::BM != TS::BM;
   const int bm = tn_block_m(tiles_m), bn = tn_block_n(tiles_n);
   const int blocks_m = (tiles_m + bm - 1) / bm, blocks_n = (tiles_n + bn - 1) / bn;
   const int per_group = blocks_m * blocks_n * (bm * bn);
@@ -741,30 +779,11 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
     const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
     g.a_r0 = tm * T::BM;
     g.b_r0 = tn * T::BN;
-    if constexpr (!SEGMENTED) {
-      // the buffers cover exactly the rows of this expert: later rows read as zero
-      const int64_t group_rows = end - start;
-      g.rsrc_a = make_rsrc(a + (int64_t)start * k, (uint32_t)(group_rows * k * 2));
-      g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
-      g.nk = (int)((group_rows + T::BK - 1) / T::BK);
-      block_gemm<DT, true, true, T>(g, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
+    uint16_t* const c_e = c + (int64_t)e * k * n;
+    if (kMixed && k - g.a_r0 <= TS::BM) {
+      tn_tile<DT, TS, SEGMENTED>(g, a, b, c_e, start, end, k, n, seg_rows, lds);
     } else {
-      // The reduction runs over the expert's rows in segments of at most seg_rows rows, each with buffers
-      // of its own that cover exactly its rows.
-      f32x16 acc[T::TM][T::TN];
-      int first = start;
-      for (;;) {
-        const int64_t left = end - first;
-        const int64_t seg = left < seg_rows ? left : seg_rows;
-        g.rsrc_a = make_rsrc(a + (int64_t)first * k, (uint32_t)(seg * k * 2));
-        g.rsrc_b = make_rsrc(b + (int64_t)first * n, (uint32_t)(seg * n * 2));
-        g.nk = (int)((seg + T::BK - 1) / T::BK);
-        block_multiply<DT, true, true, T>(g, acc, first == start, lds);
-        if (left <= seg_rows) break;
-        first += seg_rows;
-        tile_done();   // the first stages are refilled next
-      }
-      block_store<DT, T>(acc, c + (int64_t)e * k * n, n, g.a_r0, k, g.b_r0, n, lds);
+      tn_tile<DT, T, SEGMENTED>(g, a, b, c_e, start, end, k, n, seg_rows, lds);
     }
     tile_done();
   }
