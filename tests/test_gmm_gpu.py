@@ -261,6 +261,23 @@ def test_gmm_full_and_half_height_row_tiles(gg, rows_per_expert, k, n):
     assert rel_err(got.float(), ref) < TOL
 
 
+@pytest.mark.parametrize('k', [264, 384, 392, 648, 1408])      # k mod 256 = 8, 128, 136, 136, 128: the last row of tiles
+@pytest.mark.parametrize('n', [256, 520])                      # is half-height up to 128 rows, full above
+def test_gmm_tn_last_row_of_tiles(gg, k, n):
+    sizes = torch.tensor([700, 0, 64, 3000, 1, 331])
+    rows = int(sizes.sum())
+    torch.manual_seed(k + n)
+    a = torch.randn(rows, k, device='cuda').bfloat16()
+    b = torch.randn(rows, n, device='cuda').bfloat16()
+    ref = _ref_gpu(a, b, sizes, True, False)
+    guard = torch.full((ref.numel() + 4096,), 3.0, device='cuda').bfloat16()
+    c = guard[2048:2048 + ref.numel()].view(ref.shape)
+    got = gg.backend.gmm(a, b, sizes, trans_a=True, c=c)
+    assert rel_err(got, ref) < TOL and max_block_err(got, ref) < 2 * TOL
+    assert torch.count_nonzero(got[1]) == 0
+    assert bool((guard[:2048] == 3.0).all()) and bool((guard[2048 + ref.numel():] == 3.0).all())
+
+
 def _random_shapes(count, seed):
     g = torch.Generator().manual_seed(seed)
     r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
