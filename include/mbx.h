@@ -82,21 +82,35 @@ int mbx_replicate_backward(const void* grad, int dtype, int64_t batch, int64_t c
  * padded_bins is NULL) receives x[indices[i] / top_k] for the i-th sorted slot of e,
  * times weights[indices[i]] (fp32 product, rounded once) when weights is not NULL.
  * out has out_rows rows; rows owned by no slot (padding) are written as zeros.
- * x is [tokens, hidden]. */
+ * x is [tokens, hidden].  slot_rows: optional, the map mbx_slot_rows() made of the same routing;
+ * with it (and rows that are 16-byte multiples at 16-byte aligned bases) every token's row is
+ * read once and written to its top_k places; without it one wave copies one output row. */
 int mbx_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
                const int32_t* indices, const int32_t* bins, const int32_t* padded_bins,
                int num_bins, const void* weights, int w_dtype, void* out, int64_t out_rows,
-               mbx_stream_t stream);
+               const int32_t* slot_rows, mbx_stream_t stream);
+
+/* The index algebra of megablocks/backend/kernels.py:60-76 turned round: slot_rows[s] = the row of
+ * the expert-major (optionally padded) buffer that holds slot s = t * top_k + j, -1 if none
+ * does.  indices[i] is the slot at sorted position i; its row is i - bins[e-1] + padded_bins[e-1]
+ * for the expert e of that position (bin_ids[i], or found in bins when bin_ids is NULL), or i
+ * when padded_bins is NULL.  One map serves every gather and scatter of a layer step (forward and
+ * backward): n_slots entries. */
+int mbx_slot_rows(const int32_t* indices, const int32_t* bin_ids, const int32_t* bins,
+                  const int32_t* padded_bins, int num_bins, int64_t n_slots, int32_t* slot_rows,
+                  mbx_stream_t stream);
 
 /* megablocks/backend/kernels.py:173-207 `scatter` / `padded_scatter` (_padded_copy,
  * !A_TO_B, then sum over top_k): out[t] = sum_j round(x[row(t*top_k+j)] * w[t*top_k+j]),
  * each product rounded to the storage type and the sum taken in fp32, like the
  * reference's two passes but without the [tokens, top_k, hidden] temporary.
- * scratch: 4 * tokens * top_k bytes (the slot -> row map). */
+ * slot_rows: the map of mbx_slot_rows(), or NULL to have it built here in scratch
+ * (4 * tokens * top_k bytes; not used otherwise). */
 int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
                 const int32_t* indices, const int32_t* bin_ids, const int32_t* bins,
                 const int32_t* padded_bins, int num_bins, const void* weights, int w_dtype,
-                void* out, void* scratch, size_t scratch_bytes, mbx_stream_t stream);
+                void* out, const int32_t* slot_rows, void* scratch, size_t scratch_bytes,
+                mbx_stream_t stream);
 
 /* megablocks/backend/kernels.py:217-307 `scatter_wgrad` / `padded_scatter_wgrad`:
  * wgrad[indices[i]] = <x[row(i)], grad[indices[i] / top_k]> (fp32 accumulate, stored

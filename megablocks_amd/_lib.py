@@ -31,8 +31,9 @@ _SIGNATURES = {
     'mbx_topology': (_i, [_vp, _i, _i, _i, _i, _vp, _vp]),
     'mbx_replicate_forward': (_i, [_vp, _i, _i64, _i, _vp, _vp, _i64, _vp]),
     'mbx_replicate_backward': (_i, [_vp, _i, _i64, _i64, _vp, _i, _vp, _vp]),
-    'mbx_gather': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _vp]),
-    'mbx_scatter': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _sz, _vp]),
+    'mbx_gather': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _vp, _vp]),
+    'mbx_slot_rows': (_i, [_vp, _vp, _vp, _vp, _i, _i64, _vp, _vp]),
+    'mbx_scatter': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _sz, _vp]),
     'mbx_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     'mbx_binned_gather': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _vp]),
     'mbx_binned_scatter': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _sz, _vp]),

@@ -41,18 +41,44 @@ def _scratch(n_slots, device):
     return torch.empty(max(n_slots, 1), dtype=torch.int32, device=device)
 
 
+def _slot_rows(indices, bin_ids, bins, padded_bins):
+    """int32 [n_slots]: the row of the expert-major (optionally padded) buffer that holds each slot.  One map
+    serves all gathers and scatters of a routing decision, forward and backward, so it is kept on the `indices`
+    tensor and reused while `indices`, `bins` and `padded_bins` are the same unmodified tensors.  Under stream
+    capture nothing is reused or kept: a captured graph has to contain the kernels that build its map."""
+    capturing = torch.cuda.is_current_stream_capturing()
+    key = (indices._version, bins.data_ptr(), bins._version,
+           None if padded_bins is None else (padded_bins.data_ptr(), padded_bins._version))
+    cached = getattr(indices, '_mbx_slot_rows', None)
+    if not capturing and cached is not None and cached[0] == key:
+        return cached[1]
+    n_slots = indices.shape[0]
+    rows = _scratch(n_slots, indices.device)
+    with torch.cuda.device_of(indices):
+        _lib.check(lib.mbx_slot_rows(_lib.ptr(indices), _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins),
+                                     bins.shape[0], n_slots, _lib.ptr(rows), _lib.stream()), 'slot_rows')
+    if not capturing:
+        try:
+            indices._mbx_slot_rows = (key, rows, bins, padded_bins)   # the references keep the data pointers of the key alive
+        except Exception:
+            pass
+    return rows
+
+
 def _gather(x, indices, bin_ids, weights, bins, padded_bins, top_k, output_rows, what):
-    _lib.require_cuda(x, indices, bins, padded_bins, weights)
+    _lib.require_cuda(x, indices, bin_ids, bins, padded_bins, weights)
     x = x.contiguous()
     indices, bins, padded_bins = _lib.as_i32(indices), _lib.as_i32(bins), _lib.as_i32(padded_bins)
     wp, wdt, weights = _w(weights)
     out = torch.empty((output_rows, x.shape[1]), dtype=x.dtype, device=x.device)
+    # top_k = 1: every row of x is read once either way, the kernel with one wave per output row needs no map
+    rows = _slot_rows(indices, _lib.as_i32(bin_ids), bins, padded_bins) if top_k > 1 and indices.shape[0] else None
     with torch.cuda.device_of(x), _lib.record('gather_weighted' if weights is not None else 'gather',
                                               rows_in=x.shape[0], rows_out=output_rows, hidden=x.shape[1],
                                               elem=x.element_size()):
         _lib.check(lib.mbx_gather(_lib.ptr(x), _lib.dtype_of(x), x.shape[0], x.shape[1], top_k, _lib.ptr(indices),
                                   _lib.ptr(bins), _lib.ptr(padded_bins), bins.shape[0], wp, wdt, _lib.ptr(out),
-                                  output_rows, _lib.stream()), what)
+                                  output_rows, _lib.ptr(rows), _lib.stream()), what)
     return out
 
 
@@ -124,13 +150,13 @@ def _scatter(x, indices, bin_ids, weights, bins, padded_bins, top_k):
     bins, padded_bins = _lib.as_i32(bins), _lib.as_i32(padded_bins)
     wp, wdt, weights = _w(weights)
     out = torch.empty((tokens, x.shape[1]), dtype=x.dtype, device=x.device)
-    scratch = _scratch(n_slots, x.device)
+    rows = _slot_rows(indices, bin_ids, bins, padded_bins) if n_slots else None
     with torch.cuda.device_of(x), _lib.record('scatter_weighted' if weights is not None else 'scatter',
                                               rows_in=n_slots, rows_out=tokens, hidden=x.shape[1],
                                               elem=x.element_size()):
         _lib.check(lib.mbx_scatter(_lib.ptr(x), _lib.dtype_of(x), tokens, x.shape[1], top_k, _lib.ptr(indices),
                                    _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins), bins.shape[0], wp, wdt,
-                                   _lib.ptr(out), _lib.ptr(scratch), scratch.numel() * 4, _lib.stream()), 'scatter')
+                                   _lib.ptr(out), _lib.ptr(rows), None, 0, _lib.stream()), 'scatter')
     return out
 
 

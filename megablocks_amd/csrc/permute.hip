@@ -115,12 +115,13 @@ __device__ __forceinline__ float wave_dot_row(const typename Elem<DT>::type* __r
       for (int i = 0; i < E; ++i) acc += fa[i] * fb[i];
     };
     int c = lane;
-    for (; c + 3 * kWave < nvec; c += 4 * kWave) {
-      const u32x4 a0 = av[c], a1 = av[c + kWave], a2 = av[c + 2 * kWave], a3 = av[c + 3 * kWave];
+    for (; c + 3 * kWave < nvec; c += 4 * kWave) {   // a: rows read once (non-temporal); b: rows other slots read again
+      const u32x4 a0 = __builtin_nontemporal_load(av + c), a1 = __builtin_nontemporal_load(av + c + kWave);
+      const u32x4 a2 = __builtin_nontemporal_load(av + c + 2 * kWave), a3 = __builtin_nontemporal_load(av + c + 3 * kWave);
       const u32x4 b0 = bv[c], b1 = bv[c + kWave], b2 = bv[c + 2 * kWave], b3 = bv[c + 3 * kWave];
       dot_vec(a0, b0); dot_vec(a1, b1); dot_vec(a2, b2); dot_vec(a3, b3);
     }
-    for (; c < nvec; c += kWave) dot_vec(av[c], bv[c]);
+    for (; c < nvec; c += kWave) dot_vec(__builtin_nontemporal_load(av + c), bv[c]);
   } else {
     for (int c = lane; c < hidden; c += kWave) acc += Elem<DT>::to_f32(a[c]) * Elem<DT>::to_f32(b[c]);
   }
@@ -170,7 +171,7 @@ __global__ void inverse_map_kernel(const int32_t* __restrict__ indices, const in
   if (s < 0 || s >= n_slots) return;
   int row = i;
   if (padded_bins != nullptr) {
-    const int e = bin_ids[i];
+    const int e = bin_ids ? bin_ids[i] : upper_bound_i32(bins, num_bins, i);   // sorted position i lies in bins[e-1] .. bins[e]
     if (e < 0 || e >= num_bins) return;
     if (e > 0) row = i - bins[e - 1] + padded_bins[e - 1];
   }
@@ -194,6 +195,81 @@ __global__ void fill_kernel(int32_t* __restrict__ p, int64_t n, int32_t v) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (; i < n; i += stride) p[i] = v;
+}
+
+// ------------------------------------------------------------------ gather, one wave per token
+// The token's row is read once (the row-major kernel reads it once per slot, from wherever in the expert-major
+// order that slot landed) and written to the rows of its top_k slots, inv[t * top_k + j] (-1: none).  Then
+// the rows that no slot owns (padding, slots with an invalid index) are zero-filled: lane l of a wave looks at
+// row base + l, and the wave clears the rows its ballot names.  Loads and stores are non-temporal: every byte
+// is touched once, and keeping it out of the caches is worth a fifth of the kernel's time.
+template <int DT>
+__global__ void __launch_bounds__(kRowThreads)
+gather_tokens_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ indices,
+                     const int32_t* __restrict__ inv, const int32_t* __restrict__ bins,
+                     const int32_t* __restrict__ padded_bins, int num_bins, const void* __restrict__ weights, int w_dtype,
+                     void* __restrict__ out_, int64_t out_rows) {
+  typedef typename Elem<DT>::type E;
+  constexpr int EV = Vec16<DT>::kElems;
+  const E* x = (const E*)x_;
+  E* out = (E*)out_;
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int nvec = hidden / EV;
+  const int64_t wave_id = (int64_t)blockIdx.x * kRowWaves + wave, waves = (int64_t)gridDim.x * kRowWaves;
+  // a work item: 4 x 64 16-byte columns of one token's row (long rows are shared out over several waves)
+  const int chunks = (nvec + 4 * kWave - 1) / (4 * kWave);
+  for (int64_t item = wave_id; item < tokens * chunks; item += waves) {
+    const int64_t t = item / chunks;
+    const int c0 = (int)(item % chunks) * 4 * kWave;
+    const u32x4* src = (const u32x4*)(x + t * hidden);
+    const int64_t s0 = t * top_k;
+    const int my_row = lane < top_k ? inv[s0 + lane] : -1;
+    const float my_scale = (weights && lane < top_k) ? load_as_f32(weights, s0 + lane, w_dtype) : 1.f;
+    {
+      u32x4 v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = c0 + i * kWave + lane;
+        if (c < nvec) v[i] = __builtin_nontemporal_load(src + c);
+      }
+      for (int j = 0; j < top_k; ++j) {
+        const int row = __shfl(my_row, j, kWave);
+        if (row < 0) continue;
+        const float scale = __shfl(my_scale, j, kWave);
+        u32x4* dst = (u32x4*)(out + (int64_t)row * hidden);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c = c0 + i * kWave + lane;
+          if (c >= nvec) continue;
+          u32x4 w = v[i];
+          if (weights) {
+            float f[EV];
+            Vec16<DT>::unpack(w, f);
+#pragma unroll
+            for (int q = 0; q < EV; ++q) f[q] *= scale;
+            w = Vec16<DT>::pack(f);
+          }
+          __builtin_nontemporal_store(w, dst + c);
+        }
+      }
+    }
+  }
+  const int n_slots = (int)(tokens * top_k);
+  for (int64_t base = wave_id * kWave; base < out_rows; base += waves * kWave) {
+    const int64_t row = base + lane;
+    bool empty = false;
+    if (row < out_rows) {
+      const int pos = slot_of_row((int)row, bins, padded_bins, num_bins, n_slots);
+      const int sl = pos >= 0 ? indices[pos] : -1;
+      empty = sl < 0 || sl >= n_slots;
+    }
+    uint64_t todo = __ballot(empty);
+    while (todo) {
+      const int l = (int)__builtin_ctzll(todo);
+      todo &= todo - 1;
+      wave_zero_row<DT, true>(out + (base + l) * hidden, hidden);
+    }
+  }
 }
 
 // ------------------------------------------------------------------ combine (scatter)
@@ -242,7 +318,7 @@ combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_
         u32x4 v[BATCH];
 #pragma unroll
         for (int j = 0; j < BATCH; ++j)
-          if (live[j]) v[j] = src[j][c];
+          if (live[j]) v[j] = __builtin_nontemporal_load(src[j] + c);   // expert-major rows are read once
         float acc[EV];
 #pragma unroll
         for (int i = 0; i < EV; ++i) acc[i] = 0.f;
@@ -269,7 +345,7 @@ combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_
           if (row < 0) continue;
           const float scale = weights ? load_as_f32(weights, s0 + j, w_dtype) : 1.f;
           float f[EV];
-          Vec16<DT>::unpack(((const u32x4*)(x + (int64_t)row * hidden))[c], f);
+          Vec16<DT>::unpack(__builtin_nontemporal_load((const u32x4*)(x + (int64_t)row * hidden) + c), f);
 #pragma unroll
           for (int i = 0; i < EV; ++i)
             acc[i] += weights ? Elem<DT>::to_f32(Elem<DT>::from_f32(f[i] * scale)) : f[i];
@@ -405,7 +481,7 @@ extern "C" {
 
 int mbx_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
                const int32_t* bins, const int32_t* padded_bins, int num_bins, const void* weights, int w_dtype,
-               void* out, int64_t out_rows, mbx_stream_t stream) {
+               void* out, int64_t out_rows, const int32_t* slot_rows, mbx_stream_t stream) {
   if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || out_rows < 0 || bad_dtype(dtype)) return MBX_EINVAL;
   if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
   if (out_rows == 0 || hidden == 0) return 0;
@@ -413,27 +489,58 @@ int mbx_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k, 
   if (tokens * top_k > 0x7fffffff || out_rows > 0x7fffffff) return MBX_ERANGE;
   const bool vec = can_vec(dtype, hidden, x ? x : out, out);
   hipStream_t s = as_stream(stream);
+  if (vec && tokens > 0 && top_k <= kWave && slot_rows) {
+    // one wave per token, through the slot -> row map
+    const int32_t* inv = slot_rows;
+    const int64_t items = tokens * ceil_div((int64_t)hidden * dtype_bytes(dtype) / 16, 4 * kWave);
+    const unsigned grid = row_grid(items > out_rows / kWave ? items : out_rows / kWave);
+    switch (dtype) {
+      case MBX_BF16: gather_tokens_kernel<MBX_BF16><<<grid, kRowThreads, 0, s>>>(x, tokens, hidden, top_k, indices, inv, bins, padded_bins, num_bins, weights, w_dtype, out, out_rows); break;
+      case MBX_F16: gather_tokens_kernel<MBX_F16><<<grid, kRowThreads, 0, s>>>(x, tokens, hidden, top_k, indices, inv, bins, padded_bins, num_bins, weights, w_dtype, out, out_rows); break;
+      default: gather_tokens_kernel<MBX_F32><<<grid, kRowThreads, 0, s>>>(x, tokens, hidden, top_k, indices, inv, bins, padded_bins, num_bins, weights, w_dtype, out, out_rows); break;
+    }
+    return launch_status();
+  }
 #define CALL(DT, V) gather_kernel<DT, V><<<row_grid(out_rows), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, indices, bins, padded_bins, num_bins, weights, w_dtype, out, out_rows)
   MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
 #undef CALL
   return launch_status();
 }
 
-int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
-                const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins, int num_bins,
-                const void* weights, int w_dtype, void* out, void* scratch, size_t scratch_bytes, mbx_stream_t stream) {
-  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || bad_dtype(dtype)) return MBX_EINVAL;
-  if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
-  if (tokens == 0 || hidden == 0) return 0;
-  if (!x || !out || !indices || (padded_bins && (!bins || !bin_ids))) return MBX_EINVAL;
-  const int64_t n_slots = tokens * top_k;
-  if (n_slots > 0x7fffffff) return MBX_ERANGE;
-  if (!scratch || scratch_bytes < (size_t)n_slots * sizeof(int32_t)) return MBX_ESCRATCH;
-  int32_t* inv = (int32_t*)scratch;
-  hipStream_t s = as_stream(stream);
+static void build_slot_rows(const int32_t* indices, const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins,
+                            int num_bins, int64_t n_slots, int32_t* inv, hipStream_t s) {
   const unsigned fb = (unsigned)(ceil_div(n_slots, 256) < 2048 ? ceil_div(n_slots, 256) : 2048);
   fill_kernel<<<fb, 256, 0, s>>>(inv, n_slots, -1);
   inverse_map_kernel<<<(unsigned)ceil_div(n_slots, 256), 256, 0, s>>>(indices, bin_ids, bins, padded_bins, num_bins, (int)n_slots, inv);
+}
+
+int mbx_slot_rows(const int32_t* indices, const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins,
+                  int num_bins, int64_t n_slots, int32_t* slot_rows, mbx_stream_t stream) {
+  if (n_slots < 0 || num_bins < 0) return MBX_EINVAL;
+  if (n_slots == 0) return 0;
+  if (!indices || !slot_rows || (padded_bins && !bins)) return MBX_EINVAL;
+  if (n_slots > 0x7fffffff) return MBX_ERANGE;
+  build_slot_rows(indices, bin_ids, bins, padded_bins, num_bins, n_slots, slot_rows, as_stream(stream));
+  return launch_status();
+}
+
+int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
+                const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins, int num_bins,
+                const void* weights, int w_dtype, void* out, const int32_t* slot_rows, void* scratch, size_t scratch_bytes,
+                mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
+  if (tokens == 0 || hidden == 0) return 0;
+  if (!x || !out || (!slot_rows && (!indices || (padded_bins && !bins)))) return MBX_EINVAL;
+  const int64_t n_slots = tokens * top_k;
+  if (n_slots > 0x7fffffff) return MBX_ERANGE;
+  hipStream_t s = as_stream(stream);
+  const int32_t* inv = slot_rows;
+  if (!inv) {
+    if (!scratch || scratch_bytes < (size_t)n_slots * sizeof(int32_t)) return MBX_ESCRATCH;
+    build_slot_rows(indices, bin_ids, bins, padded_bins, num_bins, n_slots, (int32_t*)scratch, s);
+    inv = (const int32_t*)scratch;
+  }
   const bool vec = can_vec(dtype, hidden, x, out);
 #define CALL(DT, V)                                                                                                             \
   do {                                                                                                                          \

@@ -22,9 +22,11 @@ def assert_grouped_gemm_is_available():
 
 
 def _device_bins(batch_sizes: torch.Tensor, device) -> torch.Tensor:
-    """Inclusive int32 row bins on the device for a vector of group sizes (cached on the tensor)."""
+    """Inclusive int32 row bins on the device for a vector of group sizes (cached on the tensor; not under stream
+    capture, where a graph must contain the kernel that computes the bins it uses)."""
+    capturing = batch_sizes.is_cuda and torch.cuda.is_current_stream_capturing()
     cached = getattr(batch_sizes, '_mbx_bins', None)
-    if cached is not None and cached[1] == batch_sizes._version and cached[0].device == device:
+    if not capturing and cached is not None and cached[1] == batch_sizes._version and cached[0].device == device:
         return cached[0]
     if batch_sizes.ndim != 1:
         raise ValueError('batch_sizes must be a vector')
@@ -33,10 +35,11 @@ def _device_bins(batch_sizes: torch.Tensor, device) -> torch.Tensor:
         bins = inclusive_cumsum(batch_sizes.to(torch.int32), 0).view(-1)
     else:
         bins = torch.cumsum(batch_sizes, 0).to(torch.int32).to(device)
-    try:
-        batch_sizes._mbx_bins = (bins, batch_sizes._version)
-    except Exception:
-        pass
+    if not capturing:
+        try:
+            batch_sizes._mbx_bins = (bins, batch_sizes._version)
+        except Exception:
+            pass
     return bins
 
 

@@ -325,6 +325,35 @@ def test_empty_and_degenerate_inputs(ops, kernels):
     assert no_k.shape == (8, 32) and torch.count_nonzero(no_k) == 0                       # empty reduction: zeros
 
 
+@pytest.mark.parametrize('padded', [False, True])
+def test_c_abi_gather_and_scatter_without_a_prebuilt_map(kernels, padded):
+    """mbx_gather with slot_rows = NULL copies by output row, mbx_scatter with slot_rows = NULL builds the map in
+    the caller's scratch: same results as the calls the Python wrappers make (with the shared map)."""
+    from megablocks_amd import _lib
+    lib = _lib.lib
+    sl, hs, ne, top_k = 1000, 256, 16, 4
+    indices, bin_ids, bins, pbins = (dev(t) for t in _routing(sl, ne, top_k, seed=5))
+    x = dev(torch.randn(sl, hs).bfloat16())
+    w = dev(torch.rand(sl * top_k).bfloat16())
+    pb = pbins if padded else None
+    rows = int(pbins[-1]) if padded else sl * top_k
+    want = kernels.padded_gather(x, indices, bin_ids, w, bins, pbins, top_k) if padded else \
+        kernels.gather(x, indices, bin_ids, w, bins, top_k)
+    got = torch.full((rows, hs), 7.0, device='cuda').bfloat16()
+    _lib.check(lib.mbx_gather(_lib.ptr(x), _lib.dtype_of(x), sl, hs, top_k, _lib.ptr(indices), _lib.ptr(bins), _lib.ptr(pb),
+                              ne, _lib.ptr(w), _lib.dtype_of(w), _lib.ptr(got), rows, None, _lib.stream()), 'gather')
+    assert torch.equal(got, want)
+    want_back = kernels.padded_scatter(want, indices, bin_ids, w, bins, pbins, top_k) if padded else \
+        kernels.scatter(want, indices, bin_ids, w, bins, top_k)
+    back = torch.full((sl, hs), 7.0, device='cuda').bfloat16()
+    scratch = torch.empty(sl * top_k, dtype=torch.int32, device='cuda')
+    args = (_lib.ptr(want), _lib.dtype_of(x), sl, hs, top_k, _lib.ptr(indices), _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(pb),
+            ne, _lib.ptr(w), _lib.dtype_of(w), _lib.ptr(back), None)
+    _lib.check(lib.mbx_scatter(*args, _lib.ptr(scratch), scratch.numel() * 4, _lib.stream()), 'scatter')
+    assert torch.equal(back, want_back)
+    assert lib.mbx_scatter(*args, None, 0, _lib.stream()) == -2                      # neither a map nor scratch
+
+
 def test_permutation_of_more_than_4GiB(ops):
     """Routed rows of 2.5e9 elements (4.9 GB in bf16): element offsets pass 2^31, byte offsets 2^32.  Same
     size-independent properties, plus the padded forms and the weight gradient on a slice."""
