@@ -152,7 +152,9 @@ def summarize(w, agg, slots_scale):
                               bytes_per_launch=nbytes, gbps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
                               frac_of_hbm_peak=round(nbytes / (avg_ms * 1e-3) / HBM_PEAK, 4))
         elif 'hidden' in m:
-            nbytes = float(w.tokens + w.slots) * m['hidden'] * m['elem']
+            # scatter_backward (weighted gather and router-weight gradient in one pass) also reads the routed rows
+            rows_moved = w.tokens + (2 if name == 'scatter_backward' else 1) * w.slots
+            nbytes = float(rows_moved) * m['hidden'] * m['elem']
             perm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, bytes_per_launch=nbytes,
                               gbps=round(nbytes / (avg_ms * 1e-3) / 1e9, 1),
                               frac_of_hbm_peak=round(nbytes / (avg_ms * 1e-3) / HBM_PEAK, 4))

@@ -120,6 +120,21 @@ int mbx_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens
                       const int32_t* bins, const int32_t* padded_bins, int num_bins,
                       void* wgrad, mbx_stream_t stream);
 
+/* The backward of `scatter` / `padded_scatter` with weights, megablocks/ops/scatter.py:34-62 and
+ * megablocks/ops/padded_scatter.py:49-80 (a weighted gather of the output gradient, then
+ * `scatter_wgrad`), in one pass over grad[tokens, hidden]:
+ *   grad_x[row(s)] = round(grad[s / top_k] * weights[s]),   wgrad[s] = <x[row(s)], grad[s / top_k]>
+ * for every slot s with a row in slot_rows (the map of mbx_slot_rows(), required); the other
+ * rows of grad_x[out_rows, hidden] are written as zeros, the other entries of wgrad are left
+ * alone.  Same values as mbx_gather + mbx_scatter_wgrad.  MBX_EUNSUPPORTED (the caller makes the
+ * two calls): no map, top_k above 4 (where the two kernels are faster), rows that are not
+ * 16-byte multiples at aligned bases. */
+int mbx_scatter_backward(const void* grad, const void* x, int dtype, int64_t tokens, int hidden,
+                         int top_k, const int32_t* indices, const int32_t* bins,
+                         const int32_t* padded_bins, int num_bins, const void* weights,
+                         int w_dtype, const int32_t* slot_rows, void* grad_x, int64_t out_rows,
+                         void* wgrad, mbx_stream_t stream);
+
 /* megablocks/backend/kernels.py:392-418 `binned_gather`: out [num_bins, capacity, hidden];
  * entry j of expert e = x[indices[bins[e-1]+j] / top_k] (* weight) for j < min(count_e,
  * capacity), zeros otherwise. */

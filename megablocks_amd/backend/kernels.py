@@ -160,6 +160,40 @@ def _scatter(x, indices, bin_ids, weights, bins, padded_bins, top_k):
     return out
 
 
+def scatter_backward(x, grad, indices, bin_ids, weights, bins, padded_bins, top_k):
+    """Both gradients of the weighted `scatter` / `padded_scatter` (padded_bins None: unpadded) of `x`:
+    (gather of `grad` weighted, scatter_wgrad), as megablocks/ops/scatter.py:34-62 and
+    megablocks/ops/padded_scatter.py:49-80 compute them with two kernels, in one pass over `grad` where the
+    library has a kernel for the shape, else by those two calls."""
+    _lib.require_cuda(x, grad, indices, bin_ids, weights, bins, padded_bins)
+    xc = x.contiguous()
+    gc = grad.contiguous().to(xc.dtype)
+    n_slots = indices.shape[0]
+    tokens = n_slots // top_k
+    if n_slots and tuple(gc.shape) == (tokens, xc.shape[1]) and indices.dtype == torch.int32:
+        idx, bi = indices.contiguous(), _lib.as_i32(bin_ids)
+        b, pb = _lib.as_i32(bins), _lib.as_i32(padded_bins)
+        wp, wdt, wc = _w(weights)
+        rows = _slot_rows(idx, bi, b, pb)
+        dgrad = torch.empty_like(xc)
+        wgrad = torch.empty((n_slots,), dtype=xc.dtype, device=xc.device)
+        with torch.cuda.device_of(xc), _lib.record('scatter_backward', rows_in=tokens, rows_out=xc.shape[0],
+                                                   hidden=xc.shape[1], elem=xc.element_size()) as rec:
+            rc = lib.mbx_scatter_backward(_lib.ptr(gc), _lib.ptr(xc), _lib.dtype_of(xc), tokens, xc.shape[1], top_k,
+                                          _lib.ptr(idx), _lib.ptr(b), _lib.ptr(pb), b.shape[0], wp, wdt, _lib.ptr(rows),
+                                          _lib.ptr(dgrad), xc.shape[0], _lib.ptr(wgrad), _lib.stream())
+            if rc == _lib.EUNSUPPORTED:
+                rec.cancel()
+        if rc != _lib.EUNSUPPORTED:
+            _lib.check(rc, 'scatter_backward')
+            return dgrad, wgrad
+    if padded_bins is None:
+        return (gather(grad, indices, bin_ids, weights, bins, top_k),
+                scatter_wgrad(x, grad, indices, bin_ids, bins, top_k))
+    return (padded_gather(grad, indices, bin_ids, weights, bins, padded_bins, top_k),
+            padded_scatter_wgrad(x, grad, indices, bin_ids, bins, padded_bins, top_k))
+
+
 def padded_scatter_wgrad(x, grad, indices, bin_ids, bins, padded_bins, top_k):
     """megablocks/backend/kernels.py:279-303."""
     assert_is_matrix(x)

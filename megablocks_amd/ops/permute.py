@@ -56,6 +56,9 @@ class ScatterOp(torch.autograd.Function):
         grad = grad.contiguous()
         saved = ctx.saved_tensors
         indices, bin_ids, weights, bins = saved[:4]
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and weights is not None:   # both read grad's rows: one pass
+            dgrad, wgrad = kernels.scatter_backward(saved[-1], grad, indices, bin_ids, weights, bins, None, ctx.top_k)
+            return dgrad, None, None, wgrad, None, None, None
         dgrad = None
         if ctx.needs_input_grad[0]:
             dgrad = kernels.gather(grad, indices, bin_ids, weights, bins, ctx.top_k)
@@ -108,6 +111,10 @@ class PaddedScatterOp(torch.autograd.Function):
         grad = grad.contiguous()
         saved = ctx.saved_tensors
         indices, bin_ids, weights, bins, padded_bins = saved[:5]
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and weights is not None:   # both read grad's rows: one pass
+            dgrad, wgrad = kernels.scatter_backward(saved[-1], grad, indices, bin_ids, weights, bins, padded_bins,
+                                                    ctx.top_k)
+            return dgrad, None, None, wgrad, None, None, None, None
         dgrad = None
         if ctx.needs_input_grad[0]:
             dgrad = kernels.padded_gather(grad, indices, bin_ids, weights, bins, padded_bins, ctx.top_k)

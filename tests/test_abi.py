@@ -22,7 +22,7 @@ def test_header_declares_the_expected_surface():
     names = declared_symbols()
     for required in ['mbx_histogram', 'mbx_sort', 'mbx_sort_scratch_bytes', 'mbx_cumsum', 'mbx_topology',
                      'mbx_replicate_forward', 'mbx_replicate_backward', 'mbx_gather', 'mbx_slot_rows', 'mbx_scatter',
-                     'mbx_scatter_wgrad', 'mbx_binned_gather', 'mbx_binned_scatter', 'mbx_binned_scatter_wgrad',
+                     'mbx_scatter_wgrad', 'mbx_scatter_backward', 'mbx_binned_gather', 'mbx_binned_scatter', 'mbx_binned_scatter_wgrad',
                      'mbx_gmm', 'mbx_gelu_backward_inplace', 'mbx_error_string', 'mbx_version']:
         assert required in names
 

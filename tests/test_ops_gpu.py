@@ -354,6 +354,35 @@ def test_c_abi_gather_and_scatter_without_a_prebuilt_map(kernels, padded):
     assert lib.mbx_scatter(*args, None, 0, _lib.stream()) == -2                      # neither a map nor scratch
 
 
+@pytest.mark.parametrize('sl,hs,ne,top_k', [(1024, 256, 8, 1), (1000, 4096, 8, 2), (777, 264, 5, 3), (2048, 2048, 64, 6),
+                                            (512, 1024, 16, 8), (300, 100, 4, 2), (256, 128, 32, 9)])
+@pytest.mark.parametrize('padded', [False, True])
+def test_scatter_backward_in_one_pass_equals_the_two_kernels(kernels, sl, hs, ne, top_k, padded):
+    """mbx_scatter_backward against mbx_gather (weighted) + mbx_scatter_wgrad: the same values bit for bit, padding
+    rows zero; shapes it does not take (rows that are not 16-byte multiples, top_k above 4) fall back to the two."""
+    from megablocks_amd import _lib
+    indices, bin_ids, bins, pbins = (dev(t) for t in _routing(sl, ne, top_k, seed=9))
+    grad = dev(torch.randn(sl, hs).bfloat16())
+    w = dev(torch.rand(sl * top_k).bfloat16())
+    if padded:
+        x = kernels.padded_gather(dev(torch.randn(sl, hs).bfloat16()), indices, bin_ids, None, bins, pbins, top_k)
+        want = (kernels.padded_gather(grad, indices, bin_ids, w, bins, pbins, top_k),
+                kernels.padded_scatter_wgrad(x, grad, indices, bin_ids, bins, pbins, top_k))
+    else:
+        x = kernels.gather(dev(torch.randn(sl, hs).bfloat16()), indices, bin_ids, None, bins, top_k)
+        want = (kernels.gather(grad, indices, bin_ids, w, bins, top_k),
+                kernels.scatter_wgrad(x, grad, indices, bin_ids, bins, top_k))
+    _lib.profile_hook = []
+    try:
+        got = kernels.scatter_backward(x, grad, indices, bin_ids, w, bins, pbins if padded else None, top_k)
+        names = [r[0] for r in _lib.profile_hook]
+    finally:
+        _lib.profile_hook = None
+    one_pass = hs % 8 == 0 and top_k <= 4
+    assert names == (['scatter_backward'] if one_pass else ['gather_weighted', 'scatter_wgrad'])
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
 def test_permutation_of_more_than_4GiB(ops):
     """Routed rows of 2.5e9 elements (4.9 GB in bf16): element offsets pass 2^31, byte offsets 2^32.  Same
     size-independent properties, plus the padded forms and the weight gradient on a slice."""
