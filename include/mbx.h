@@ -127,8 +127,7 @@ int mbx_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens
  * for every slot s with a row in slot_rows (the map of mbx_slot_rows(), required); the other
  * rows of grad_x[out_rows, hidden] are written as zeros, the other entries of wgrad are left
  * alone.  Same values as mbx_gather + mbx_scatter_wgrad.  MBX_EUNSUPPORTED (the caller makes the
- * two calls): no map, top_k above 4 (where the two kernels are faster), rows that are not
- * 16-byte multiples at aligned bases. */
+ * two calls): no map, top_k above 8, rows that are not 16-byte multiples at aligned bases. */
 int mbx_scatter_backward(const void* grad, const void* x, int dtype, int64_t tokens, int hidden,
                          int top_k, const int32_t* indices, const int32_t* bins,
                          const int32_t* padded_bins, int num_bins, const void* weights,

@@ -400,7 +400,8 @@ wgrad_kernel(const void* __restrict__ x_, const void* __restrict__ grad_, int64_
 // One wave per token reads grad[t] once, and for each of its slots reads x[row], accumulates the dot product
 // in the order wgrad_kernel does and writes the dx row: N h e bytes of reads through L2 and one launch less
 // than the two kernels.  Then the rows of dx that no slot owns are zero-filled, as in gather_tokens_kernel.
-template <int DT, int BATCH>
+// WRITE = false: only dw (a read-only pass; dx is left to gather_tokens_kernel).
+template <int DT, int BATCH, bool WRITE>
 __global__ void __launch_bounds__(kRowThreads)
 scatter_backward_kernel(const void* __restrict__ grad_, const void* __restrict__ x_, int64_t tokens, int hidden, int top_k,
                         const int32_t* __restrict__ indices, const int32_t* __restrict__ inv,
@@ -465,7 +466,7 @@ scatter_backward_kernel(const void* __restrict__ grad_, const void* __restrict__
             acc[j] += fx[q] * fg[q];
             fg[q] *= scale[j];
           }
-          __builtin_nontemporal_store(Vec16<DT>::pack(fg), dr + c);
+          if (WRITE) __builtin_nontemporal_store(Vec16<DT>::pack(fg), dr + c);
         }
       }
     }
@@ -475,6 +476,7 @@ scatter_backward_kernel(const void* __restrict__ grad_, const void* __restrict__
       if (lane == 0 && row[j] >= 0) wgrad[s0 + j] = Elem<DT>::from_f32(d);
     }
   }
+  if (!WRITE) return;
   const int n_slots = (int)(tokens * top_k);
   for (int64_t base = wave_id * kWave; base < out_rows; base += waves * kWave) {
     const int64_t r = base + lane;
@@ -675,20 +677,27 @@ int mbx_scatter_backward(const void* grad, const void* x, int dtype, int64_t tok
                          void* wgrad, mbx_stream_t stream) {
   if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || out_rows < 0 || bad_dtype(dtype) || bad_dtype(w_dtype)) return MBX_EINVAL;
   if (tokens * top_k > 0x7fffffff || out_rows > 0x7fffffff) return MBX_ERANGE;
-  // The one-pass kernel needs the slot -> row map and whole 16-byte columns.  It is kept to at most 4 experts per
-  // token: with more, a token's wave alternates between reading and writing so many scattered rows that the pass
-  // takes longer than the read-only and the write-mostly kernel it replaces (6 experts: 480 against 430 us).
-  if (!slot_rows || top_k > 4 || hidden == 0 || !can_vec(dtype, hidden, grad, x, grad_x)) return MBX_EUNSUPPORTED;
+  // Needs the slot -> row map and whole 16-byte columns.  One pass for up to 4 experts per token.  With 5 to 8 a
+  // token's wave would alternate between reading and writing so many scattered rows that the pass takes longer
+  // than a write-mostly and a read-only kernel (6 experts: 480 against 375 us): then the gather by token writes
+  // grad_x and the same kernel, without its stores, computes wgrad.
+  if (!slot_rows || top_k > 8 || hidden == 0 || !can_vec(dtype, hidden, grad, x, grad_x)) return MBX_EUNSUPPORTED;
   if (tokens == 0) return 0;
   if (!grad || !x || !indices || !weights || !grad_x || !wgrad || (padded_bins && !bins)) return MBX_EINVAL;
   hipStream_t s = as_stream(stream);
   const unsigned grid = row_grid(tokens > out_rows / kWave ? tokens : out_rows / kWave);
-#define CALL(DT, B) scatter_backward_kernel<DT, B><<<grid, kRowThreads, 0, s>>>(grad, x, tokens, hidden, top_k, indices, slot_rows, bins, padded_bins, num_bins, weights, w_dtype, grad_x, out_rows, wgrad)
+#define CALL(DT, B, W) scatter_backward_kernel<DT, B, W><<<grid, kRowThreads, 0, s>>>(grad, x, tokens, hidden, top_k, indices, slot_rows, bins, padded_bins, num_bins, weights, w_dtype, grad_x, out_rows, wgrad)
 #define CALL_DT(DT)                        \
   do {                                     \
-    if (top_k == 1) CALL(DT, 1);           \
-    else if (top_k == 2) CALL(DT, 2);      \
-    else CALL(DT, 4);                      \
+    if (top_k == 1) CALL(DT, 1, true);     \
+    else if (top_k == 2) CALL(DT, 2, true);\
+    else if (top_k <= 4) CALL(DT, 4, true);\
+    else {                                 \
+      const int64_t items = tokens * ceil_div((int64_t)hidden * dtype_bytes(dtype) / 16, 4 * kWave);                       \
+      const unsigned ggrid = row_grid(items > out_rows / kWave ? items : out_rows / kWave);                               \
+      gather_tokens_kernel<DT><<<ggrid, kRowThreads, 0, s>>>(grad, tokens, hidden, top_k, indices, slot_rows, bins, padded_bins, num_bins, weights, w_dtype, grad_x, out_rows); \
+      CALL(DT, 8, false);                  \
+    }                                      \
   } while (0)
   switch (dtype) {
     case MBX_BF16: CALL_DT(MBX_BF16); break;
