@@ -383,6 +383,30 @@ def test_scatter_backward_in_one_pass_equals_the_two_kernels(kernels, sl, hs, ne
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
 
 
+def test_slot_row_map_is_rebuilt_when_the_routing_changes(kernels):
+    """The map the wrappers keep on `indices` is reused only for the same, unmodified indices / bins / padded_bins."""
+    sl, hs, ne, top_k = 512, 128, 8, 2
+    x = torch.randn(sl, hs).bfloat16()
+    ia, ba, bina, pba = _routing(sl, ne, top_k, seed=11)
+    ib, bb, binb, pbb = _routing(sl, ne, top_k, seed=12)
+    indices, bin_ids, bins, pbins = dev(ia), dev(ba), dev(bina), dev(pba)
+    got = kernels.gather(dev(x), indices, bin_ids, None, bins, top_k)
+    assert torch.equal(got.cpu(), oracle.gather(x, ia, ba, None, bina, top_k))
+    first = indices._mbx_slot_rows[1]
+    kernels.scatter(got, indices, bin_ids, None, bins, top_k)
+    assert indices._mbx_slot_rows[1] is first                                    # same routing: the map is reused
+    got = kernels.padded_gather(dev(x), indices, bin_ids, None, bins, pbins, top_k)     # other layout, same indices
+    assert torch.equal(got.cpu(), oracle.padded_gather(x, ia, ba, None, bina, pba, top_k))
+    indices.copy_(dev(ib)); bin_ids.copy_(dev(bb)); bins.copy_(dev(binb)); pbins.copy_(dev(pbb))   # new routing in place
+    got = kernels.padded_gather(dev(x), indices, bin_ids, None, bins, pbins, top_k)
+    assert torch.equal(got.cpu(), oracle.padded_gather(x, ib, bb, None, binb, pbb, top_k))
+    got = kernels.gather(dev(x), indices, bin_ids, None, bins, top_k)
+    assert torch.equal(got.cpu(), oracle.gather(x, ib, bb, None, binb, top_k))
+    w = torch.rand(sl * top_k).bfloat16()
+    back = kernels.scatter(got, indices, bin_ids, dev(w), bins, top_k)
+    assert torch.equal(back.cpu(), oracle.scatter(got.cpu(), ib, bb, w, binb, top_k))
+
+
 def test_permutation_of_more_than_4GiB(ops):
     """Routed rows of 2.5e9 elements (4.9 GB in bf16): element offsets pass 2^31, byte offsets 2^32.  Same
     size-independent properties, plus the padded forms and the weight gradient on a slice."""
