@@ -677,10 +677,10 @@ int mbx_scatter_backward(const void* grad, const void* x, int dtype, int64_t tok
                          void* wgrad, mbx_stream_t stream) {
   if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || out_rows < 0 || bad_dtype(dtype) || bad_dtype(w_dtype)) return MBX_EINVAL;
   if (tokens * top_k > 0x7fffffff || out_rows > 0x7fffffff) return MBX_ERANGE;
-  // Needs the slot -> row map and whole 16-byte columns.  One pass for up to 4 experts per token.  With 5 to 8 a
-  // token's wave would alternate between reading and writing so many scattered rows that the pass takes longer
-  // than a write-mostly and a read-only kernel (6 experts: 480 against 375 us): then the gather by token writes
-  // grad_x and the same kernel, without its stores, computes wgrad.
+  // Needs the slot -> row map and whole 16-byte columns.  One pass for one expert per token.  With more, a
+  // token's wave would alternate between reading and writing several scattered rows, and the pass takes longer
+  // than a write-mostly and a read-only kernel (4 experts: 247 against 212 us, 6 experts: 480 against 375): then
+  // the gather by token writes grad_x and the same kernel, without its stores, computes wgrad.
   if (!slot_rows || top_k > 8 || hidden == 0 || !can_vec(dtype, hidden, grad, x, grad_x)) return MBX_EUNSUPPORTED;
   if (tokens == 0) return 0;
   if (!grad || !x || !indices || !weights || !grad_x || !wgrad || (padded_bins && !bins)) return MBX_EINVAL;
@@ -690,13 +690,13 @@ int mbx_scatter_backward(const void* grad, const void* x, int dtype, int64_t tok
 #define CALL_DT(DT)                        \
   do {                                     \
     if (top_k == 1) CALL(DT, 1, true);     \
-    else if (top_k == 2) CALL(DT, 2, true);\
-    else if (top_k <= 4) CALL(DT, 4, true);\
     else {                                 \
       const int64_t items = tokens * ceil_div((int64_t)hidden * dtype_bytes(dtype) / 16, 4 * kWave);                       \
       const unsigned ggrid = row_grid(items > out_rows / kWave ? items : out_rows / kWave);                               \
       gather_tokens_kernel<DT><<<ggrid, kRowThreads, 0, s>>>(grad, tokens, hidden, top_k, indices, slot_rows, bins, padded_bins, num_bins, weights, w_dtype, grad_x, out_rows); \
-      CALL(DT, 8, false);                  \
+      if (top_k == 2) CALL(DT, 2, false);  \
+      else if (top_k <= 4) CALL(DT, 4, false); \
+      else CALL(DT, 8, false);             \
     }                                      \
   } while (0)
   switch (dtype) {
