@@ -75,8 +75,36 @@ def ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def stream():
+    """The current stream of the current device as the ABI takes it.  Called once per launch: the raw handle
+    straight from the binding where torch has one (several times cheaper than building a Stream object)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class device_of:
+    """`with device_of(tensor):` makes the tensor's device current for the launch (and restores the previous one);
+    nothing to do, and nearly free, when it already is."""
+    __slots__ = ('idx', 'prev')
+
+    def __init__(self, t):
+        self.idx, self.prev = t.device.index, -1
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if self.idx is not None and cur != self.idx:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 def require_cuda(*tensors):

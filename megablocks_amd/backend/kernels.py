@@ -54,7 +54,7 @@ def _slot_rows(indices, bin_ids, bins, padded_bins):
         return cached[1]
     n_slots = indices.shape[0]
     rows = _scratch(n_slots, indices.device)
-    with torch.cuda.device_of(indices):
+    with _lib.device_of(indices):
         _lib.check(lib.mbx_slot_rows(_lib.ptr(indices), _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins),
                                      bins.shape[0], n_slots, _lib.ptr(rows), _lib.stream()), 'slot_rows')
     if not capturing:
@@ -73,7 +73,7 @@ def _gather(x, indices, bin_ids, weights, bins, padded_bins, top_k, output_rows,
     out = torch.empty((output_rows, x.shape[1]), dtype=x.dtype, device=x.device)
     # top_k = 1: every row of x is read once either way, the kernel with one wave per output row needs no map
     rows = _slot_rows(indices, _lib.as_i32(bin_ids), bins, padded_bins) if top_k > 1 and indices.shape[0] else None
-    with torch.cuda.device_of(x), _lib.record('gather_weighted' if weights is not None else 'gather',
+    with _lib.device_of(x), _lib.record('gather_weighted' if weights is not None else 'gather',
                                               rows_in=x.shape[0], rows_out=output_rows, hidden=x.shape[1],
                                               elem=x.element_size()):
         _lib.check(lib.mbx_gather(_lib.ptr(x), _lib.dtype_of(x), x.shape[0], x.shape[1], top_k, _lib.ptr(indices),
@@ -151,7 +151,7 @@ def _scatter(x, indices, bin_ids, weights, bins, padded_bins, top_k):
     wp, wdt, weights = _w(weights)
     out = torch.empty((tokens, x.shape[1]), dtype=x.dtype, device=x.device)
     rows = _slot_rows(indices, bin_ids, bins, padded_bins) if n_slots else None
-    with torch.cuda.device_of(x), _lib.record('scatter_weighted' if weights is not None else 'scatter',
+    with _lib.device_of(x), _lib.record('scatter_weighted' if weights is not None else 'scatter',
                                               rows_in=n_slots, rows_out=tokens, hidden=x.shape[1],
                                               elem=x.element_size()):
         _lib.check(lib.mbx_scatter(_lib.ptr(x), _lib.dtype_of(x), tokens, x.shape[1], top_k, _lib.ptr(indices),
@@ -177,7 +177,7 @@ def scatter_backward(x, grad, indices, bin_ids, weights, bins, padded_bins, top_
         rows = _slot_rows(idx, bi, b, pb)
         dgrad = torch.empty_like(xc)
         wgrad = torch.empty((n_slots,), dtype=xc.dtype, device=xc.device)
-        with torch.cuda.device_of(xc), _lib.record('scatter_backward', rows_in=tokens, rows_out=xc.shape[0],
+        with _lib.device_of(xc), _lib.record('scatter_backward', rows_in=tokens, rows_out=xc.shape[0],
                                                    hidden=xc.shape[1], elem=xc.element_size()) as rec:
             rc = lib.mbx_scatter_backward(_lib.ptr(gc), _lib.ptr(xc), _lib.dtype_of(xc), tokens, xc.shape[1], top_k,
                                           _lib.ptr(idx), _lib.ptr(b), _lib.ptr(pb), b.shape[0], wp, wdt, _lib.ptr(rows),
@@ -229,7 +229,7 @@ def _scatter_wgrad(x, grad, indices, bin_ids, bins, padded_bins, top_k):
     indices, bin_ids = _lib.as_i32(indices), _lib.as_i32(bin_ids)
     bins, padded_bins = _lib.as_i32(bins), _lib.as_i32(padded_bins)
     out = torch.empty((n_slots,), dtype=x.dtype, device=x.device)
-    with torch.cuda.device_of(x), _lib.record('scatter_wgrad', rows_in=n_slots, rows_out=tokens, hidden=x.shape[1],
+    with _lib.device_of(x), _lib.record('scatter_wgrad', rows_in=n_slots, rows_out=tokens, hidden=x.shape[1],
                                               elem=x.element_size()):
         _lib.check(lib.mbx_scatter_wgrad(_lib.ptr(x), _lib.ptr(grad), _lib.dtype_of(x), tokens, x.shape[1], top_k,
                                          _lib.ptr(indices), _lib.ptr(bin_ids), _lib.ptr(bins), _lib.ptr(padded_bins),
@@ -251,7 +251,7 @@ def binned_gather(x, indices, weights, bins, expert_capacity, top_k):
     wp, wdt, weights = _w(weights)
     num_experts = bins.shape[0]
     out = torch.empty((num_experts, expert_capacity, x.shape[1]), dtype=x.dtype, device=x.device)
-    with torch.cuda.device_of(x):
+    with _lib.device_of(x):
         _lib.check(lib.mbx_binned_gather(_lib.ptr(x), _lib.dtype_of(x), x.shape[0], x.shape[1], top_k, _lib.ptr(indices),
                                          _lib.ptr(bins), num_experts, expert_capacity, wp, wdt, _lib.ptr(out),
                                          _lib.stream()), 'binned_gather')
@@ -275,7 +275,7 @@ def binned_scatter(x, indices, weights, bins, top_k):
     wp, wdt, weights = _w(weights)
     out = torch.empty((tokens, hidden_size), dtype=x.dtype, device=x.device)
     scratch = _scratch(n_slots, x.device)
-    with torch.cuda.device_of(x):
+    with _lib.device_of(x):
         _lib.check(lib.mbx_binned_scatter(_lib.ptr(x), _lib.dtype_of(x), tokens, hidden_size, top_k, _lib.ptr(indices),
                                           _lib.ptr(bins), num_experts, expert_capacity, wp, wdt, _lib.ptr(out),
                                           _lib.ptr(scratch), scratch.numel() * 4, _lib.stream()), 'binned_scatter')
@@ -299,7 +299,7 @@ def binned_scatter_wgrad(x, grad, indices, bins, top_k):
     assert_equal(grad.shape[0], tokens)
     indices, bins = _lib.as_i32(indices), _lib.as_i32(bins)
     out = torch.empty((n_slots,), dtype=x.dtype, device=x.device)
-    with torch.cuda.device_of(x):
+    with _lib.device_of(x):
         _lib.check(lib.mbx_binned_scatter_wgrad(_lib.ptr(x), _lib.ptr(grad), _lib.dtype_of(x), tokens, hidden_size, top_k,
                                                 _lib.ptr(indices), _lib.ptr(bins), num_experts, expert_capacity,
                                                 _lib.ptr(out), _lib.stream()), 'binned_scatter_wgrad')

@@ -85,7 +85,7 @@ def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None, _record_as=None
     else:
         if tuple(c.shape) != shape or c.dtype != a.dtype or not c.is_contiguous():
             raise ValueError('gmm: c has the wrong shape, dtype or layout')
-    with torch.cuda.device_of(a), _lib.record(_record_as or ('gmm_nn', 'gmm_nt', 'gmm_tn')[layout], rows=rows, k=k, n=n,
+    with _lib.device_of(a), _lib.record(_record_as or ('gmm_nn', 'gmm_nt', 'gmm_tn')[layout], rows=rows, k=k, n=n,
                                               elem=a.element_size(), groups=groups):
         _lib.check(lib.mbx_gmm(_lib.ptr(a), _lib.ptr(b), _lib.ptr(c), dt, _lib.ptr(bins), groups, rows, k, n, layout,
                                _lib.stream()), 'gmm')
@@ -111,7 +111,7 @@ def gmm_dual(a, b, a2, b2, batch_sizes, trans_b=False, c=None):
         c = torch.empty((rows, n), dtype=a.dtype, device=a.device)
     elif tuple(c.shape) != (rows, n) or c.dtype != a.dtype or not c.is_contiguous():
         raise ValueError('gmm_dual: c has the wrong shape, dtype or layout')
-    with torch.cuda.device_of(a), _lib.record('gmm_nt_dual' if trans_b else 'gmm_nn_dual', rows=rows, k=2 * k, n=n,
+    with _lib.device_of(a), _lib.record('gmm_nt_dual' if trans_b else 'gmm_nn_dual', rows=rows, k=2 * k, n=n,
                                               elem=a.element_size(), groups=groups) as rec:
         rc = lib.mbx_gmm_dual(_lib.ptr(a), _lib.ptr(b), _lib.ptr(a2), _lib.ptr(b2), _lib.ptr(c), _lib.dtype_of(a),
                               _lib.ptr(bins), groups, rows, k, n, layout, _lib.stream())

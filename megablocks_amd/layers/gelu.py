@@ -12,7 +12,7 @@ def gelu_backward_(grad: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
         raise ValueError('gelu_backward_: grad and x must match in shape and dtype')
     if not grad.is_contiguous() or not x.is_contiguous():
         raise ValueError('gelu_backward_: expected contiguous tensors')
-    with torch.cuda.device_of(grad):
+    with _lib.device_of(grad):
         _lib.check(lib.mbx_gelu_backward_inplace(_lib.ptr(grad), _lib.ptr(x), _lib.dtype_of(grad), grad.numel(),
                                                  _lib.stream()), 'gelu_backward_')
     return grad

@@ -36,7 +36,7 @@ def _fusable(*tensors):
 
 def _glu_forward(a, b, act):
     out = torch.empty_like(a)
-    with torch.cuda.device_of(a):
+    with _lib.device_of(a):
         _lib.check(lib.mbx_glu_forward(_lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.dtype_of(a), act, a.numel(),
                                        _lib.stream()), 'glu_forward')
     return out
@@ -44,7 +44,7 @@ def _glu_forward(a, b, act):
 
 def _glu_backward(g, a, b, act):
     da, db = torch.empty_like(a), torch.empty_like(a)
-    with torch.cuda.device_of(a):
+    with _lib.device_of(a):
         _lib.check(lib.mbx_glu_backward(_lib.ptr(g), _lib.ptr(a), _lib.ptr(b), _lib.ptr(da), _lib.ptr(db),
                                         _lib.dtype_of(a), act, a.numel(), _lib.stream()), 'glu_backward')
     return da, db

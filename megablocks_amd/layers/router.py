@@ -104,7 +104,7 @@ class _SoftmaxTopK(torch.autograd.Function):
         scores = torch.empty_like(logits)
         weights = torch.empty((tokens, top_k), dtype=logits.dtype, device=logits.device)
         indices = torch.empty((tokens, top_k), dtype=torch.int64, device=logits.device)
-        with torch.cuda.device_of(logits):
+        with _lib.device_of(logits):
             _lib.check(_lib.lib.mbx_router_forward(_lib.ptr(logits), _lib.dtype_of(logits), tokens, experts, top_k,
                                                    float(norm_p), _lib.ptr(scores), _lib.ptr(weights), _lib.ptr(indices),
                                                    _lib.stream()), 'router_forward')
@@ -120,7 +120,7 @@ class _SoftmaxTopK(torch.autograd.Function):
         grad_logits = torch.empty_like(scores)
         gs = None if grad_scores is None else grad_scores.to(scores.dtype).contiguous()
         gw = None if grad_weights is None else grad_weights.to(scores.dtype).contiguous()
-        with torch.cuda.device_of(scores):
+        with _lib.device_of(scores):
             _lib.check(_lib.lib.mbx_router_backward(_lib.ptr(gw), _lib.ptr(gs), _lib.ptr(scores), _lib.ptr(indices),
                                                     _lib.dtype_of(scores), tokens, experts, ctx.top_k, ctx.norm_p,
                                                     _lib.ptr(grad_logits), _lib.stream()), 'router_backward')

@@ -23,7 +23,7 @@ def _histogram(x: torch.Tensor, num_bins: int) -> torch.Tensor:
     x = x.contiguous()
     rows, n = (1, x.numel()) if x.ndim == 1 else x.shape
     out = torch.empty((rows, num_bins), dtype=torch.int32, device=x.device)
-    with torch.cuda.device_of(x):
+    with _lib.device_of(x):
         _lib.check(lib.mbx_histogram(_lib.ptr(x), it, rows, n, num_bins, _lib.ptr(out), _lib.stream()), 'histogram')
     return out.flatten() if x.ndim == 1 else out
 
@@ -53,7 +53,7 @@ def _sort(x, end_bit, x_out, iota_out):
     n = x.numel()
     nbytes = lib.mbx_sort_scratch_bytes(n, it, end_bit)
     scratch = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device_of(x):
+    with _lib.device_of(x):
         _lib.check(lib.mbx_sort(_lib.ptr(x), it, n, end_bit, _lib.ptr(x_out), _lib.ptr(iota_out), _lib.ptr(scratch),
                                 nbytes, _lib.stream()), 'sort')
 
@@ -85,7 +85,7 @@ def _cumsum(x, dim, exclusive):
         raise RuntimeError('cumsum expects a 2-D tensor scanned along dim 1')  # csrc/cumsum.h:115-117
     x = x.contiguous()
     out = torch.empty_like(x)
-    with torch.cuda.device_of(x):
+    with _lib.device_of(x):
         _lib.check(lib.mbx_cumsum(_lib.ptr(x), it, x.shape[0], x.shape[1], int(exclusive), _lib.ptr(out),
                                   _lib.stream()), 'cumsum')
     return out.squeeze() if squeeze else out  # a one-element 1-D input comes back 0-dim, as in the reference
@@ -122,7 +122,7 @@ class TopologyOp(torch.autograd.Function):
             raise RuntimeError('topology expects a 1-D int32 padded_bins')
         padded_bins = padded_bins.contiguous()
         out = torch.empty(output_block_rows * output_block_columns, dtype=torch.int16, device=padded_bins.device)
-        with torch.cuda.device_of(padded_bins):
+        with _lib.device_of(padded_bins):
             _lib.check(lib.mbx_topology(_lib.ptr(padded_bins), padded_bins.numel(), int(block_size),
                                         int(output_block_rows), int(output_block_columns), _lib.ptr(out),
                                         _lib.stream()), 'topology')
@@ -147,7 +147,7 @@ def replicate_forward(x, bins, out):
         return
     x, bins = x.contiguous(), bins.contiguous()
     assert out.is_contiguous()
-    with torch.cuda.device_of(x):
+    with _lib.device_of(x):
         _lib.check(lib.mbx_replicate_forward(_lib.ptr(x), x.element_size(), x.shape[0], bins.shape[0], _lib.ptr(bins),
                                              _lib.ptr(out), out.shape[1], _lib.stream()), 'replicate_forward')
 
@@ -166,7 +166,7 @@ def replicate_backward(grad, bins, out):
         return
     grad, bins = grad.contiguous(), bins.contiguous()
     assert out.is_contiguous()
-    with torch.cuda.device_of(grad):
+    with _lib.device_of(grad):
         _lib.check(lib.mbx_replicate_backward(_lib.ptr(grad), dt, grad.shape[0], grad.shape[1], _lib.ptr(bins),
                                               bins.shape[0], _lib.ptr(out), _lib.stream()), 'replicate_backward')
 
