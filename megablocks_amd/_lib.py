@@ -107,6 +107,11 @@ class device_of:
         return False
 
 
+def autocast_gpu_dtype():
+    get = getattr(torch, 'get_autocast_dtype', None)
+    return get('cuda') if get is not None else torch.get_autocast_gpu_dtype()
+
+
 def require_cuda(*tensors):
     for t in tensors:
         if t is not None and not t.is_cuda:

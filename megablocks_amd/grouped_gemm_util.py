@@ -149,7 +149,19 @@ class GroupedGemm(torch.autograd.Function):
         return agrad, bgrad, None, None
 
 
+def autocast_operands(*tensors):
+    """Under autocast the operands of a product are taken in the autocast type, as torch's own matmul does: with
+    fp32 master weights the grouped experts then work like the block-sparse ones, whose stk products are
+    autocast-aware in the reference.  The casts are ordinary autograd nodes (a weight's gradient comes back in the
+    weight's type)."""
+    if tensors[0].is_cuda and torch.is_autocast_enabled():
+        dt = _lib.autocast_gpu_dtype()
+        return tuple(t.to(dt) for t in tensors)
+    return tensors
+
+
 def _ops_gmm(a, b, batch_sizes, trans_b=False):
+    a, b = autocast_operands(a, b)
     return GroupedGemm.apply(a, b, batch_sizes, trans_b)
 
 

@@ -1,6 +1,7 @@
 """megablocks/layers/common.py:9-26."""
 import torch
 
+from megablocks_amd import _lib
 from megablocks_amd.layers.arguments import Arguments
 
 
@@ -15,7 +16,7 @@ def dtype(args: Arguments):
 def cast_if_autocast_enabled(tensor):
     if torch.is_autocast_enabled():
         if tensor.device.type == 'cuda':
-            target = torch.get_autocast_gpu_dtype()
+            target = _lib.autocast_gpu_dtype()
         elif tensor.device.type == 'cpu':
             target = torch.get_autocast_cpu_dtype()
         else:

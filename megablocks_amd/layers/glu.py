@@ -188,7 +188,7 @@ class SparseGLU(SparseMLP):
                 raise NotImplementedError(
                     'Memory optimized implementation not yet supported with GLU with sparse kernels.')
             return memory_optimized_grouped_glu(x, w1, v1, w2, batch_sizes, self.args.activation_fn)
-        x1, x2 = GLUProjection.apply(x, w1, v1, batch_sizes)
+        x1, x2 = GLUProjection.apply(*gg.autocast_operands(x, w1, v1), batch_sizes)
         x1 = gated_activation(self.args.activation_fn, x1, x2)
         return gg.ops.gmm(x1, w2, batch_sizes)
 

@@ -458,6 +458,37 @@ def test_dmoe_with_no_tokens_and_with_one(mlp_impl, tokens):
         assert all(torch.count_nonzero(p.grad) == 0 for p in layer.parameters())
 
 
+@pytest.mark.parametrize('mlp_type,mlp_impl,memopt', [('mlp', 'grouped', False), ('mlp', 'grouped', True), ('mlp', 'sparse', False),
+                                                      ('mlp', 'sparse', True), ('glu', 'grouped', False),
+                                                      ('glu', 'grouped', True), ('glu', 'sparse', False)])
+def test_autocast_with_fp32_parameters_equals_the_bf16_layer(mlp_type, mlp_impl, memopt):
+    """fp32 master weights under torch.autocast(bf16): the products run on the bf16 casts, so the layer gives what
+    the same layer with bf16 parameters gives, and its gradients arrive in fp32."""
+    from megablocks_amd.layers.dmoe import dMoE
+    torch.manual_seed(7)
+    kw = dict(hidden_size=256, ffn_hidden_size=512, moe_num_experts=4, moe_top_k=2, mlp_type=mlp_type, mlp_impl=mlp_impl,
+              memory_optimized_mlp=memopt)
+    master = dMoE(_args(bf16=False, **kw))
+    half = dMoE(_args(**kw))
+    with torch.no_grad():
+        for p16, p32 in zip(half.parameters(), master.parameters()):
+            assert p32.dtype == torch.float32 and p16.dtype == torch.bfloat16
+            p16.copy_(p32)
+    x = torch.randn(64, 4, 256, device='cuda')
+    x32 = x.clone().requires_grad_(True)
+    x16 = x.bfloat16().requires_grad_(True)
+    grad = torch.randn(64, 4, 256, device='cuda').bfloat16()
+    with torch.autocast('cuda', dtype=torch.bfloat16):
+        out = master(x32)
+    out.backward(grad)
+    want = half(x16)
+    want.backward(grad)
+    assert out.dtype == torch.bfloat16 and torch.equal(out, want)
+    assert x32.grad.dtype == torch.float32 and rel_err(x32.grad, x16.grad) < 1e-6
+    for p32, p16 in zip(master.parameters(), half.parameters()):
+        assert p32.grad.dtype == torch.float32 and rel_err(p32.grad, p16.grad) < 1e-6
+
+
 def test_forward_shapes_bias_and_losses():
     # tests/layers/dmoe_test.py:103-188
     from megablocks_amd.layers import moe, router
