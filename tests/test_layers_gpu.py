@@ -489,6 +489,25 @@ def test_autocast_with_fp32_parameters_equals_the_bf16_layer(mlp_type, mlp_impl,
         assert p32.grad.dtype == torch.float32 and rel_err(p32.grad, p16.grad) < 1e-6
 
 
+def test_parameter_names_and_shapes_are_the_reference_checkpoint_layout():
+    """A state dict written by the reference's dMoE / MoE loads unchanged: `router.layer.weight [E, h]`,
+    `experts.mlp.{w1, v1, w2} [E * ffn, h]` (mlp.py:315-330, glu.py:23-43), `experts.bias [h]` (moe.py:116-128); the
+    capacity-factor MoE keeps `w1 [E, h, ffn]`, `w2 [E, ffn, h]` (mlp.py:99-116)."""
+    from megablocks_amd.layers.dmoe import dMoE
+    from megablocks_amd.layers.moe import MoE
+    kw = dict(hidden_size=128, ffn_hidden_size=384, moe_num_experts=4, moe_top_k=2, bias=True)
+    for mlp_impl in ('grouped', 'sparse'):
+        shapes = {k: tuple(v.shape) for k, v in dMoE(_args(mlp_type='glu', mlp_impl=mlp_impl, **kw)).state_dict().items()}
+        assert shapes == {'router.layer.weight': (4, 128), 'experts.bias': (128,), 'experts.mlp.w1': (4 * 384, 128),
+                          'experts.mlp.w2': (4 * 384, 128), 'experts.mlp.v1': (4 * 384, 128)}
+        shapes = {k: tuple(v.shape) for k, v in dMoE(_args(mlp_type='mlp', mlp_impl=mlp_impl, **kw)).state_dict().items()}
+        assert shapes == {'router.layer.weight': (4, 128), 'experts.bias': (128,), 'experts.mlp.w1': (4 * 384, 128),
+                          'experts.mlp.w2': (4 * 384, 128)}
+    shapes = {k: tuple(v.shape) for k, v in MoE(_args(**kw)).state_dict().items()}
+    assert shapes == {'router.layer.weight': (4, 128), 'experts.bias': (128,), 'experts.mlp.w1': (4, 128, 384),
+                      'experts.mlp.w2': (4, 384, 128)}
+
+
 def test_forward_shapes_bias_and_losses():
     # tests/layers/dmoe_test.py:103-188
     from megablocks_amd.layers import moe, router
