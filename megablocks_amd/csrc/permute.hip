@@ -197,12 +197,37 @@ __global__ void fill_kernel(int32_t* __restrict__ p, int64_t n, int32_t v) {
   for (; i < n; i += stride) p[i] = v;
 }
 
+// Zero-fill the rows of an expert-major buffer that no slot owns (padding; a sorted position whose index is not a
+// slot), for the kernels that write such a buffer slot by slot.  Lane l of a wave looks at row base + l, and the
+// wave clears the rows its ballot names; wave `wave_id` of `waves` takes every waves-th group of 64 rows.
+template <int DT>
+__device__ __forceinline__ void zero_unowned_rows(typename Elem<DT>::type* __restrict__ out, int64_t out_rows, int hidden,
+                                                  const int32_t* __restrict__ indices, const int32_t* __restrict__ bins,
+                                                  const int32_t* __restrict__ padded_bins, int num_bins, int n_slots,
+                                                  int64_t wave_id, int64_t waves) {
+  const int lane = lane_id();
+  for (int64_t base = wave_id * kWave; base < out_rows; base += waves * kWave) {
+    const int64_t row = base + lane;
+    bool empty = false;
+    if (row < out_rows) {
+      const int pos = slot_of_row((int)row, bins, padded_bins, num_bins, n_slots);
+      const int sl = pos >= 0 ? indices[pos] : -1;
+      empty = sl < 0 || sl >= n_slots;
+    }
+    uint64_t todo = __ballot(empty);
+    while (todo) {
+      const int l = (int)__builtin_ctzll(todo);
+      todo &= todo - 1;
+      wave_zero_row<DT, true>(out + (base + l) * hidden, hidden);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ gather, one wave per token
 // The token's row is read once (the row-major kernel reads it once per slot, from wherever in the expert-major
 // order that slot landed) and written to the rows of its top_k slots, inv[t * top_k + j] (-1: none).  Then
-// the rows that no slot owns (padding, slots with an invalid index) are zero-filled: lane l of a wave looks at
-// row base + l, and the wave clears the rows its ballot names.  Loads and stores are non-temporal: every byte
-// is touched once, and keeping it out of the caches is worth a fifth of the kernel's time.
+// the rows that no slot owns are zero-filled.  Loads and stores are non-temporal: every byte is touched once,
+// and keeping it out of the caches is worth a fifth of the kernel's time.
 template <int DT>
 __global__ void __launch_bounds__(kRowThreads)
 gather_tokens_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ indices,
@@ -254,22 +279,7 @@ gather_tokens_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, in
       }
     }
   }
-  const int n_slots = (int)(tokens * top_k);
-  for (int64_t base = wave_id * kWave; base < out_rows; base += waves * kWave) {
-    const int64_t row = base + lane;
-    bool empty = false;
-    if (row < out_rows) {
-      const int pos = slot_of_row((int)row, bins, padded_bins, num_bins, n_slots);
-      const int sl = pos >= 0 ? indices[pos] : -1;
-      empty = sl < 0 || sl >= n_slots;
-    }
-    uint64_t todo = __ballot(empty);
-    while (todo) {
-      const int l = (int)__builtin_ctzll(todo);
-      todo &= todo - 1;
-      wave_zero_row<DT, true>(out + (base + l) * hidden, hidden);
-    }
-  }
+  zero_unowned_rows<DT>(out, out_rows, hidden, indices, bins, padded_bins, num_bins, (int)(tokens * top_k), wave_id, waves);
 }
 
 // ------------------------------------------------------------------ combine (scatter)
@@ -476,23 +486,7 @@ scatter_backward_kernel(const void* __restrict__ grad_, const void* __restrict__
       if (lane == 0 && row[j] >= 0) wgrad[s0 + j] = Elem<DT>::from_f32(d);
     }
   }
-  if (!WRITE) return;
-  const int n_slots = (int)(tokens * top_k);
-  for (int64_t base = wave_id * kWave; base < out_rows; base += waves * kWave) {
-    const int64_t r = base + lane;
-    bool empty = false;
-    if (r < out_rows) {
-      const int pos = slot_of_row((int)r, bins, padded_bins, num_bins, n_slots);
-      const int sl = pos >= 0 ? indices[pos] : -1;
-      empty = sl < 0 || sl >= n_slots;
-    }
-    uint64_t todo = __ballot(empty);
-    while (todo) {
-      const int l = (int)__builtin_ctzll(todo);
-      todo &= todo - 1;
-      wave_zero_row<DT, true>(dx + (base + l) * hidden, hidden);
-    }
-  }
+  if (WRITE) zero_unowned_rows<DT>(dx, out_rows, hidden, indices, bins, padded_bins, num_bins, (int)(tokens * top_k), wave_id, waves);
 }
 
 // ------------------------------------------------------------------ binned variants
