@@ -27,7 +27,7 @@ HBM_PEAK = 8e12
 MEASURED_TRAFFIC = {
     # workload c3, rocprofv3 FETCH_SIZE (x2.00, the factor a plain 1 GiB copy shows) + WRITE_SIZE, bytes per launch;
     # see profiles/gmm_dmoe_c3_mixtral_hbm_traffic.txt
-    ('c3', 'gmm_nn'): 3.50e9, ('c3', 'gmm_nt'): 4.00e9, ('c3', 'gmm_tn'): 4.93e9, ('c3', 'gmm_nn_dual'): 6.84e9,
+    ('c3', 'gmm_nn'): 4.94e9, ('c3', 'gmm_nt'): 6.41e9, ('c3', 'gmm_tn'): 4.90e9, ('c3', 'gmm_nn_dual'): 9.90e9,
 }
 
 
