@@ -54,16 +54,22 @@ class ParallelDroplessMLP(moe.ParallelMLP):
                              f'the block size {self.blocking}. Please update your configuration.')
         block_rows = padded_tokens // self.blocking
         blocks_per_row = self.ffn_hidden_size // self.blocking
-        offsets = torch.arange(0, block_rows * blocks_per_row + 1, blocks_per_row, dtype=torch.int32, device=x.device)
-        column_indices = ops.topology(padded_bins, self.blocking, block_rows, blocks_per_row)
         shape = (padded_tokens, self.ffn_hidden_size * mpu.experts_per_rank(self.args))
-        # every block-row holds blocks_per_row blocks, so block b lies in block-row b // blocks_per_row
-        row_indices = torch.arange(block_rows, dtype=torch.int32, device=x.device).repeat_interleave(
-            blocks_per_row).to(torch.int16)
-        column_indices_t, offsets_t, block_offsets_t = self.sparse_transpose(shape, row_indices, column_indices, offsets)
+        device = x.device
+
+        def index_arrays():
+            offsets = torch.arange(0, block_rows * blocks_per_row + 1, blocks_per_row, dtype=torch.int32, device=device)
+            column_indices = ops.topology(padded_bins, self.blocking, block_rows, blocks_per_row)
+            # every block-row holds blocks_per_row blocks, so block b lies in block-row b // blocks_per_row
+            row_indices = torch.arange(block_rows, dtype=torch.int32, device=device).repeat_interleave(
+                blocks_per_row).to(torch.int16)
+            column_indices_t, offsets_t, block_offsets_t = self.sparse_transpose(shape, row_indices, column_indices,
+                                                                                 offsets)
+            return dict(row_indices=row_indices, column_indices=column_indices, offsets=offsets,
+                        column_indices_t=column_indices_t, offsets_t=offsets_t, block_offsets_t=block_offsets_t)
+
         padded_tokens_per_expert = torch.diff(padded_bins, prepend=padded_bins.new_zeros(1))
-        return Topology(shape, self.blocking, row_indices, column_indices, offsets, column_indices_t, offsets_t,
-                        block_offsets_t, padded_tokens_per_expert)
+        return Topology(shape, self.blocking, padded_tokens_per_expert, index_arrays)
 
     def indices_and_padded_bins(self, top_experts):
         """dmoe.py:131-154."""

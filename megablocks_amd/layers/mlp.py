@@ -6,7 +6,6 @@ w1 and w2 (mlp.py:315-330), so the first product is `x @ w1[e].T` (NT) and the s
 sdd/dsd on a block-diagonal topology) is the same pair of grouped products taken over
 128-padded row groups, and is computed that way here.
 """
-import dataclasses
 from typing import Any, Optional
 
 import torch
@@ -107,20 +106,30 @@ class MLP(torch.nn.Module):
         return gg.ops.gmm(x, w2, sizes, False).view(experts, capacity, -1)
 
 
-@dataclasses.dataclass
 class Topology:
     """Metadata of the block-diagonal sparse matrix the reference hands to stk (what
     `stk.Matrix(shape, data, row_indices, column_indices, offsets, column_indices_t, offsets_t,
-    block_offsets_t)` carries at dmoe.py:120-129), plus the padded row groups it was built from."""
-    shape: tuple
-    blocking: int
-    row_indices: torch.Tensor
-    column_indices: torch.Tensor
-    offsets: torch.Tensor
-    column_indices_t: torch.Tensor
-    offsets_t: torch.Tensor
-    block_offsets_t: torch.Tensor
-    padded_tokens_per_expert: torch.Tensor   # int32 [E], multiples of `blocking`
+    block_offsets_t)` carries at dmoe.py:120-129), plus the padded row groups it was built from.
+
+    The products here are grouped GEMMs over `padded_tokens_per_expert` and read none of the index arrays, so
+    those are built (by `build`, a callable returning them by name) the first time one of them is asked for:
+    a layer step that never looks at them spares the dozen small launches of dmoe.py:35-129."""
+    _INDEX_ARRAYS = ('row_indices', 'column_indices', 'offsets', 'column_indices_t', 'offsets_t', 'block_offsets_t')
+
+    def __init__(self, shape, blocking: int, padded_tokens_per_expert: torch.Tensor, build):
+        self.shape = shape
+        self.blocking = blocking
+        self.padded_tokens_per_expert = padded_tokens_per_expert   # int32 [E], multiples of `blocking`
+        self._build = build
+
+    def __getattr__(self, name):
+        # reached only for attributes that are not set yet
+        if name in Topology._INDEX_ARRAYS and self.__dict__.get('_build') is not None:
+            build, self._build = self._build, None
+            for key, value in build().items():
+                setattr(self, key, value)
+            return self.__dict__[name]
+        raise AttributeError(name)
 
     def size(self):
         return self.shape
