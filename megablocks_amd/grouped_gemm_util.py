@@ -43,6 +43,17 @@ def _device_bins(batch_sizes: torch.Tensor, device) -> torch.Tensor:
     return bins
 
 
+def note_bins(batch_sizes: torch.Tensor, bins: torch.Tensor):
+    """A caller that has already computed the inclusive cumsum of `batch_sizes` (int32, on the same device) hands
+    it over, and the products of this step do not compute it again."""
+    if batch_sizes.is_cuda and bins.dtype == torch.int32 and bins.device == batch_sizes.device \
+            and bins.numel() == batch_sizes.numel() and not torch.cuda.is_current_stream_capturing():
+        try:
+            batch_sizes._mbx_bins = (bins.view(-1), batch_sizes._version)
+        except Exception:
+            pass
+
+
 def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None, _record_as=None):
     """out[r_e] = a[r_e] @ b[e] (`trans_b`: @ b[e].T); `trans_a`: out[e] = a[r_e].T @ b[r_e].
 

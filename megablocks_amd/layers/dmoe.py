@@ -8,6 +8,7 @@ import numpy as np
 import torch
 
 import megablocks_amd.ops as ops
+from megablocks_amd import grouped_gemm_util as gg
 from megablocks_amd.layers import common, dmlp_registry, moe, mpu
 from megablocks_amd.layers.arguments import Arguments
 from megablocks_amd.layers.mlp import Topology
@@ -69,6 +70,7 @@ class ParallelDroplessMLP(moe.ParallelMLP):
                         column_indices_t=column_indices_t, offsets_t=offsets_t, block_offsets_t=block_offsets_t)
 
         padded_tokens_per_expert = torch.diff(padded_bins, prepend=padded_bins.new_zeros(1))
+        gg.note_bins(padded_tokens_per_expert, padded_bins)    # the row bins of this step's grouped products
         return Topology(shape, self.blocking, padded_tokens_per_expert, index_arrays)
 
     def indices_and_padded_bins(self, top_experts):

@@ -6,6 +6,7 @@ import numpy as np
 import torch
 
 import megablocks_amd.ops as ops
+from megablocks_amd import grouped_gemm_util as gg
 from megablocks_amd.layers import common, mlp, router
 from megablocks_amd.layers.arguments import Arguments
 
@@ -95,6 +96,7 @@ class ParallelMLP(torch.nn.Module):
         tokens_per_expert = ops.histogram(top_expert, self.num_experts)
         bins = ops.inclusive_cumsum(tokens_per_expert, 0)
         bins = bins.view(1) if not len(bins.size()) else bins
+        gg.note_bins(tokens_per_expert, bins)     # the grouped products of this step take these row bins
         return indices, bin_ids, bins, tokens_per_expert
 
     def permute_and_compute(self, x, tokens_per_expert, indices, bin_ids, expert_weights, bins, expert_capacity,
