@@ -532,9 +532,9 @@ __device__ __forceinline__ void tile_done() {
 }
 
 // ---- NN / NT ----
-// Logical tile id -> (expert, column tile, row tile inside the expert), row tiles fastest.  With at
-// most 64 experts lane e of every wave keeps expert e's row range and the inclusive count of tiles
-// up to it, and a tile id is resolved with one ballot; with more, by a scan over the bins.
+// Logical tile id -> (expert, column tile, row tile inside the expert).  With at most 64 experts lane e of
+// every wave keeps expert e's row range and the inclusive count of tiles up to it, and a tile id is
+// resolved with one ballot; with more, by a scan over the bins.
 template <int BM>
 struct RowTiles {
   int lane_start = 0, lane_end = 0, lane_mt = 0, lane_incl = 0;
@@ -595,8 +595,24 @@ struct RowTiles {
         start = end;
       }
     }
-    tn = id / mt;
-    tm = id % mt;
+    // Inside an expert the tiles are counted in bands of kBand row tiles: rows fastest, then columns, then the
+    // next band.  Any 32 consecutive ids of a band are an 8 x 4 block with 12 operand panels, however many row
+    // tiles the expert has; counting all its row tiles fastest would make them a 32 x 1 strip with 33.  The
+    // last band has the rows that are left, 5 to 12 of them (up to 4 left-over rows join the band before:
+    // a band of one row would be a 1 x 32 strip).
+    constexpr int kBand = 8;
+    const int per_band = kBand * tiles_n;
+    const int bands = mt + kBand / 2 - 1 < kBand ? 1 : (mt + kBand / 2 - 1) / kBand;
+    const int full = (bands - 1) * per_band;
+    if (id < full) {
+      const int band = id / per_band, q = id - band * per_band;
+      tn = q / kBand;
+      tm = band * kBand + q % kBand;
+    } else {
+      const int left = mt - (bands - 1) * kBand, q = id - full;
+      tn = q / left;
+      tm = (bands - 1) * kBand + q % left;
+    }
   }
 };
 
