@@ -532,63 +532,73 @@ __device__ __forceinline__ void tile_done() {
 }
 
 // ---- NN / NT ----
-// Logical tile id -> (expert, column tile, row tile inside the expert).  With at most 64 experts lane e of
-// every wave keeps expert e's row range and the inclusive count of tiles up to it, and a tile id is
-// resolved with one ballot; with more, by a scan over the bins.
+// Logical tile id -> (expert, column tile, row tile inside the expert).  Lane l of every wave keeps the
+// inclusive count of tiles up to its experts (one expert per lane up to 64 experts, else a group of
+// consecutive ones), and a tile id is resolved with one ballot, then, with several experts per lane, a short
+// search through the bins of that lane's group.
 template <int BM>
 struct RowTiles {
   int lane_start = 0, lane_end = 0, lane_mt = 0, lane_incl = 0;
   int total = 0;
-  bool table;
+  int per_lane;            // experts per lane: 1 up to 64 experts (the lane then keeps its expert's row range too)
   const int32_t* bins;
   int num_groups, tiles_n;
 
+  static __device__ __forceinline__ int row_tiles(int rows) { return rows > 0 ? (rows + BM - 1) / BM : 0; }
+
   __device__ __forceinline__ RowTiles(const int32_t* bins_, int num_groups_, int tiles_n_)
       : bins(bins_), num_groups(num_groups_), tiles_n(tiles_n_) {
-    table = num_groups <= kWave;
-    if (table) {
-      const int lane = lane_id();
+    per_lane = (num_groups + kWave - 1) / kWave;
+    const int lane = lane_id();
+    const int first = lane * per_lane;
+    int span = 0;
+    if (per_lane == 1) {
       if (lane < num_groups) {
         lane_end = bins[lane];
         lane_start = lane > 0 ? bins[lane - 1] : 0;
-        const int mt = (lane_end - lane_start + BM - 1) / BM;
-        lane_mt = mt > 0 ? mt : 0;
+        lane_mt = row_tiles(lane_end - lane_start);
       }
-      int incl = lane_mt * tiles_n;
-#pragma unroll
-      for (int o = 1; o < kWave; o <<= 1) {
-        const int v = __shfl_up(incl, o, kWave);
-        if (lane >= o) incl += v;
-      }
-      lane_incl = incl;
-      total = __builtin_amdgcn_readlane(incl, kWave - 1);
-    } else {
-      int start = 0;
-      for (int e = 0; e < num_groups; ++e) {
+      span = lane_mt * tiles_n;
+    } else if (first < num_groups) {
+      // lane l keeps the tile count of experts l per_lane .. (l + 1) per_lane - 1 and the first row of that group
+      lane_start = first > 0 ? bins[first - 1] : 0;
+      int start = lane_start;
+      for (int e = first; e < first + per_lane && e < num_groups; ++e) {
         const int end = bins[e];
-        const int mt = (end - start + BM - 1) / BM;
-        total += (mt > 0 ? mt : 0) * tiles_n;
+        span += row_tiles(end - start) * tiles_n;
         start = end;
       }
+      lane_mt = span;
     }
+    int incl = span;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const int v = __shfl_up(incl, o, kWave);
+      if (lane >= o) incl += v;
+    }
+    lane_incl = incl;
+    total = __builtin_amdgcn_readlane(incl, kWave - 1);
   }
 
   // id in [0, total) -> expert, its row range, the row tile and the column tile
   __device__ __forceinline__ void find(int id, int& e, int& start, int& end, int& tm, int& tn) const {
     int mt;
-    if (table) {
-      const uint64_t hit = __ballot(id < lane_incl);
-      e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
-      start = __builtin_amdgcn_readlane(lane_start, e);
-      end = __builtin_amdgcn_readlane(lane_end, e);
-      mt = __builtin_amdgcn_readlane(lane_mt, e);
-      id -= __builtin_amdgcn_readlane(lane_incl, e) - mt * tiles_n;
+    const uint64_t hit = __ballot(id < lane_incl);
+    const int l = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
+    if (per_lane == 1) {
+      e = l;
+      start = __builtin_amdgcn_readlane(lane_start, l);
+      end = __builtin_amdgcn_readlane(lane_end, l);
+      mt = __builtin_amdgcn_readlane(lane_mt, l);
+      id -= __builtin_amdgcn_readlane(lane_incl, l) - mt * tiles_n;
     } else {
-      start = 0; end = 0; mt = 0;
-      for (e = 0; e < num_groups; ++e) {
+      // the lane's group of experts is searched in the bins (per_lane - 1 steps at most)
+      id -= __builtin_amdgcn_readlane(lane_incl, l) - __builtin_amdgcn_readlane(lane_mt, l);
+      start = __builtin_amdgcn_readlane(lane_start, l);
+      end = start; mt = 0;
+      for (e = l * per_lane; e < num_groups; ++e) {
         end = bins[e];
-        mt = (end - start + BM - 1) / BM;
-        mt = mt > 0 ? mt : 0;
+        mt = row_tiles(end - start);
         const int span = mt * tiles_n;
         if (id < span) break;
         id -= span;
