@@ -214,6 +214,9 @@ SCHEDULES = [  # name, groups, rows, k, n: one case per branch of the device-sid
     ('several full rounds and a cut tail', 8, 9000, 64, 2048),
     ('TN with two tiles per workgroup', 4, 3000, 512, 768),
     ('one row per expert', 64, 64, 64, 256),
+    ('256 experts: four per lane of the tile table', 256, 40000, 128, 512),
+    ('300 experts: five per lane, the last lanes empty', 300, 30000, 64, 264),
+    ('65 experts: two per lane', 65, 9000, 192, 512),
 ]
 
 
