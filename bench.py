@@ -45,6 +45,9 @@ def parse():
     ap.add_argument('--cpu-tokens', type=int, default=None)
     ap.add_argument('--library-gemm', action='store_true',
                     help='also time the three grouped products as per-expert torch.matmul loops (the vendor GEMM library)')
+    ap.add_argument('--operand-patterns', action='store_true',
+                    help='also time the grouped GEMM launches on all-zero and all-one operands (same shapes): what the '
+                         'same instruction stream gives when the operands cost no switching power')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also launch one plain 1 GiB device copy (a known-size reference for HBM byte counters)')
     return ap.parse_args()
@@ -220,6 +223,87 @@ def library_gemm_leg(w, inp):
     return res
 
 
+def _shader_clock_mhz():
+    """The GPU's current shader clock as the driver's sysfs table marks it (MHz), None when unreadable."""
+    import glob
+    for path in sorted(glob.glob('/sys/class/drm/card*/device/pp_dpm_sclk')):
+        try:
+            for line in open(path):
+                if line.rstrip().endswith('*'):
+                    return int(line.split(':')[1].strip().lower().split('mhz')[0])
+        except (OSError, ValueError, IndexError):
+            continue
+    return None
+
+
+def operand_pattern_leg(w, inp):
+    """The three grouped products of this workload's shapes through the shipped kernel, one second of
+    back-to-back launches each, with operands drawn as the workload draws them (N(0,1) activations, N(0,0.02)
+    weights), all zero, and all one.  The instruction stream, the addresses and the memory traffic are the same
+    in the three cases; only the switching activity of the operands differs, so the spread is what the power
+    limit takes.  The shader clock is sampled from sysfs while the launches run."""
+    import threading
+
+    import torch
+
+    from megablocks_amd import grouped_gemm_util as gg
+
+    dev = torch.device('cuda', 0)
+    if w.routing == 'router':
+        logits = inp['x'].to(dev).float() @ inp['router_weight'].to(dev).float().t()
+        top = logits.topk(w.top_k, dim=-1).indices
+    else:
+        top = inp['top_experts'].to(dev)
+    sizes = torch.bincount(top.flatten(), minlength=w.experts).to(torch.int64)
+    rows = int(sizes.sum())
+    flops = 2.0 * rows * w.hidden * w.ffn
+    res = {'what': 'mbx_gmm on this workload\'s shapes, >= 1 s of back-to-back launches per case', 'cases': {}}
+    for pattern in ('workload', 'zeros', 'ones'):
+        def draw(*shape, scale=1.0):
+            if pattern == 'zeros':
+                return torch.zeros(*shape, device=dev, dtype=w.dtype)
+            if pattern == 'ones':
+                return torch.ones(*shape, device=dev, dtype=w.dtype)
+            return (torch.randn(*shape, device=dev) * scale).to(w.dtype)
+        a, mid = draw(rows, w.hidden), draw(rows, w.ffn)
+        w1 = draw(w.experts, w.ffn, w.hidden, scale=0.02)
+        case = {}
+        for name, fn in (('gmm_nt', lambda: gg.backend.gmm(a, w1, sizes, trans_b=True)),
+                         ('gmm_nn', lambda: gg.backend.gmm(mid, w1, sizes)),
+                         ('gmm_tn', lambda: gg.backend.gmm(mid, a, sizes, trans_a=True))):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            clocks, stop = [], threading.Event()
+
+            def sample():
+                while not stop.is_set():
+                    mhz = _shader_clock_mhz()
+                    if mhz:
+                        clocks.append(mhz)
+                    stop.wait(0.05)
+            th = threading.Thread(target=sample)
+            th.start()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            n, t0 = 0, time.perf_counter()
+            e0.record()
+            while time.perf_counter() - t0 < 1.0:
+                for _ in range(20):
+                    fn()
+                n += 20
+                torch.cuda.synchronize()
+            e1.record()
+            torch.cuda.synchronize()
+            stop.set()
+            th.join()
+            ms = e0.elapsed_time(e1) / n
+            case[name] = dict(avg_ms=round(ms, 4), tflops=round(flops / (ms * 1e-3) / 1e12, 1),
+                              shader_clock_mhz=round(sum(clocks) / len(clocks)) if clocks else None)
+        res['cases'][pattern] = case
+        del a, mid, w1
+    return res
+
+
 def cpu_leg(args, w, inp_full):
     """The CPU formulation (oracle) of the same layer, fp32, forward+backward, on a bounded sample."""
     import torch
@@ -330,6 +414,8 @@ def main():
     }
     if args.library_gemm:
         out['library_gemm'] = library_gemm_leg(w, inp)
+    if args.operand_patterns:
+        out['operand_patterns'] = operand_pattern_leg(w, inp)
     if not args.no_cpu:
         del layer
         torch.cuda.empty_cache()

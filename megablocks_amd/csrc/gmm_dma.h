@@ -285,8 +285,9 @@ __device__ __forceinline__ void block_multiply(const Args& g, f32x16 (&acc)[T::T
     __builtin_amdgcn_sched_barrier(0);                                                                           \
     static_for<n_>([&](auto mi_) {                                                                               \
       constexpr int m_ = decltype(mi_)::value;                                                                   \
-      acc[m_ / T::TN][m_ % T::TN] =                                                                              \
-          mfma32<DT>(fb[CUR_BUF][m_ % T::TN], fa[CUR_BUF][m_ / T::TN], acc[m_ / T::TN][m_ % T::TN]);             \
+      /* boustrophedon order over the TM x TN products: consecutive MFMAs differ in one operand only */         \
+      constexpr int i_ = m_ / T::TN, j_ = (i_ & 1) ? T::TN - 1 - m_ % T::TN : m_ % T::TN;                        \
+      acc[i_][j_] = mfma32<DT>(fb[CUR_BUF][j_], fa[CUR_BUF][i_], acc[i_][j_]);                                   \
       MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                               \
       if (m_ >= first_ && (m_ - first_) % every_ == every_ - 1 && (m_ - first_) / every_ < (NLOADS)) {           \
         issue(IS_B, SC, DST);                                                                                    \
