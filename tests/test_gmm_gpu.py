@@ -67,6 +67,23 @@ SMALL = [  # groups, rows, k, n
 ]
 
 
+@pytest.mark.parametrize('groups,k,n', [(1, 64, 256), (59, 1440, 704), (56, 960, 1104), (174, 1344, 256), (5, 33, 17)])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('sizes_on_device', [False, True])
+def test_gmm_with_no_rows_at_all(gg, groups, k, n, dtype, sizes_on_device):
+    """Every expert empty: the weight gradients (trans_a) are exact zeros written over whatever the output
+    buffer held, and the row products are empty."""
+    sizes = torch.zeros(groups, dtype=torch.int64)
+    bs = sizes.cuda() if sizes_on_device else sizes
+    a = torch.empty(0, k, device='cuda', dtype=dtype)
+    c = torch.full((groups, k, n), float('nan'), device='cuda', dtype=dtype)
+    out = gg.backend.gmm(a, torch.empty(0, n, device='cuda', dtype=dtype), bs, trans_a=True, c=c)
+    assert out.shape == (groups, k, n) and int(torch.count_nonzero(out)) == 0
+    w = torch.randn(groups, k, n, device='cuda').to(dtype)
+    assert gg.backend.gmm(a, w, bs).shape == (0, n)
+    assert gg.backend.gmm(torch.empty(0, n, device='cuda', dtype=dtype), w, bs, trans_b=True).shape == (0, k)
+
+
 @pytest.mark.parametrize('groups,rows,k,n', SMALL)
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize('mode', ['nn', 'nt', 'tn'])
