@@ -108,3 +108,14 @@ def test_synthetic_workloads_match_the_stated_sizes():
     counts = torch.bincount(te.flatten(), minlength=64)
     assert int((counts == 0).sum()) == 4                                           # four empty experts
     assert torch.allclose(inp['expert_weights'].sum(-1), torch.ones(2048), atol=1e-5)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU holding all experts; asking for more ends with a message, not a number."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    run = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True,
+                         timeout=120)
+    assert run.returncode != 0
+    assert 'one GPU' in run.stderr and run.stdout.strip() == ''
