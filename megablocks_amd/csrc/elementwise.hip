@@ -10,7 +10,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <int DT> struct Pack {  // 16 bytes of storage <-> fp32 values
   static constexpr int N = 16 / (int)sizeof(typename Elem<DT>::type);
   static __device__ __forceinline__ void load(const void* p, int64_t vec, float* f) {
-    const u32x4 v = ((const u32x4*)p)[vec];
+    // every byte of these tensors is touched once per pass and they are far larger than the caches
+    const u32x4 v = __builtin_nontemporal_load((const u32x4*)p + vec);
     const typename Elem<DT>::type* e = (const typename Elem<DT>::type*)&v;
 #pragma unroll
     for (int i = 0; i < N; ++i) f[i] = Elem<DT>::to_f32(e[i]);
@@ -20,7 +21,7 @@ template <int DT> struct Pack {  // 16 bytes of storage <-> fp32 values
     typename Elem<DT>::type* e = (typename Elem<DT>::type*)&v;
 #pragma unroll
     for (int i = 0; i < N; ++i) e[i] = Elem<DT>::from_f32(f[i]);
-    ((u32x4*)p)[vec] = v;
+    __builtin_nontemporal_store(v, (u32x4*)p + vec);
   }
 };
 
