@@ -224,16 +224,19 @@ def library_gemm_leg(w, inp):
 
 
 def _shader_clock_mhz():
-    """The GPU's current shader clock as the driver's sysfs table marks it (MHz), None when unreadable."""
+    """The current shader clock as the driver's sysfs table marks it (MHz), None when unreadable.  Where the host
+    shows several cards, the busy one is the one with the highest clock (idle cards sit at their lowest level)."""
     import glob
+    best = None
     for path in sorted(glob.glob('/sys/class/drm/card*/device/pp_dpm_sclk')):
         try:
             for line in open(path):
                 if line.rstrip().endswith('*'):
-                    return int(line.split(':')[1].strip().lower().split('mhz')[0])
+                    mhz = int(line.split(':')[1].strip().lower().split('mhz')[0])
+                    best = mhz if best is None or mhz > best else best
         except (OSError, ValueError, IndexError):
             continue
-    return None
+    return best
 
 
 def operand_pattern_leg(w, inp):
