@@ -44,8 +44,11 @@ def _scratch(n_slots, device):
 def _slot_rows(indices, bin_ids, bins, padded_bins):
     """int32 [n_slots]: the row of the expert-major (optionally padded) buffer that holds each slot.  One map
     serves all gathers and scatters of a routing decision, forward and backward, so it is kept on the `indices`
-    tensor and reused while `indices`, `bins` and `padded_bins` are the same unmodified tensors.  Under stream
-    capture nothing is reused or kept: a captured graph has to contain the kernels that build its map."""
+    tensor and reused while `indices`, `bins` and `padded_bins` are the same unmodified tensors ("unmodified" as
+    torch sees it, by `_version`: a caller that rewrites them through raw pointers or by replaying a captured graph
+    into them must pass new tensors, or delete the `_mbx_slot_rows` attribute).  A caller that builds a new `indices` tensor for every
+    call gets a new map for every call.  Under stream capture nothing is reused or kept: a captured graph has to
+    contain the kernels that build its map."""
     capturing = torch.cuda.is_current_stream_capturing()
     key = (indices._version, bins.data_ptr(), bins._version,
            None if padded_bins is None else (padded_bins.data_ptr(), padded_bins._version))
@@ -60,7 +63,7 @@ def _slot_rows(indices, bin_ids, bins, padded_bins):
     if not capturing:
         try:
             indices._mbx_slot_rows = (key, rows, bins, padded_bins)   # the references keep the data pointers of the key alive
-        except Exception:
+        except AttributeError:   # a tensor type without instance attributes: the map is built on every call
             pass
     return rows
 

@@ -267,17 +267,21 @@ static inline int64_t xcd_grid(int64_t tiles, int run = kXcdRun) {
   return (tiles + q - 1) / q * q;
 }
 
+// A row bound read from the bins, kept inside [lo, rows]: a table that does not belong to the operands can make
+// the result wrong but never an access out of range.
+__device__ __forceinline__ int clamp_bound(int v, int lo, int rows) { return v < lo ? lo : (v > rows ? rows : v); }
+
 // ---- NN / NT: row tiles follow the expert bins --------------------------------------
 // Logical tile id -> (expert, column tile, row tile inside the expert), row tiles fastest.
 template <int DT, bool B_MC, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
-                const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_n) {
+                const int32_t* __restrict__ bins, int num_groups, int rows, int k, int n, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   int id = xcd_tile_id(blockIdx.x);
   int e = 0, start = 0, end = 0, mt = 0;
   for (; e < num_groups; ++e) {
-    end = bins[e];
+    end = clamp_bound(bins[e], start, rows);
     mt = (end - start + T::BM - 1) / T::BM;
     const int span = mt * tiles_n;
     if (id < span) break;
@@ -299,7 +303,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
 template <int DT, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
-              const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n) {
+              const int32_t* __restrict__ bins, int num_groups, int rows, int k, int n, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   const int id = xcd_tile_id(blockIdx.x);
   const int per_group = tiles_m * tiles_n;
@@ -307,7 +311,7 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
   if (e >= num_groups) return;
   const int t = id % per_group;
   const int tm = t % tiles_m, tn = t / tiles_m;
-  const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
+  const int start = e > 0 ? clamp_bound(bins[e - 1], 0, rows) : 0, end = clamp_bound(bins[e], start, rows);
   Operand opa, opb;
   opa.base = a; opa.ld = k; opa.r0 = tm * T::BM; opa.r_lim = k;
   opb.base = b; opb.ld = n; opb.r0 = tn * T::BN; opb.r_lim = n;
@@ -331,14 +335,14 @@ constexpr int kGenLd = kGenTile + 36;
 template <int DT>
 __global__ void __launch_bounds__(256)
 gmm_generic_kernel(const void* __restrict__ a_, const void* __restrict__ b_, void* __restrict__ c_,
-                   const int32_t* __restrict__ bins, int layout, int k, int n) {
+                   const int32_t* __restrict__ bins, int layout, int rows, int k, int n) {
   typedef typename Elem<DT>::type E;
   const E* a = (const E*)a_;
   const E* b = (const E*)b_;
   E* c = (E*)c_;
   __shared__ float as[2][kGenBK][kGenLd], bs[2][kGenBK][kGenLd];
   const int e = blockIdx.z;
-  const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
+  const int start = e > 0 ? clamp_bound(bins[e - 1], 0, rows) : 0, end = clamp_bound(bins[e], start, rows);
   int m_dim, r_begin, r_end;
   if (layout == MBX_TN) { m_dim = k; r_begin = start; r_end = end; }
   else { m_dim = end - start; r_begin = 0; r_end = k; }
@@ -503,7 +507,7 @@ int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num
     if (rc) return rc;
     const int64_t grid = xcd_grid((int64_t)tiles_m * tiles_n * num_groups);
     if (grid > 0x7fffffff) return MBX_ERANGE;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n);
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n);
     return launch_status();
   }
   const int tiles_n = (int)ceil_div(n, T::BN);
@@ -515,13 +519,13 @@ int gmm_mfma(const void* a, const void* b, void* c, const int32_t* bins, int num
     auto kern = gmm_rows_kernel<DT, false, T>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_n);
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_n);
   } else {
     constexpr size_t lds = lds_bytes<DT, false, true, T>();
     auto kern = gmm_rows_kernel<DT, true, T>;
     int rc = allow_lds(kern, lds);
     if (rc) return rc;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_n);
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_n);
   }
   return launch_status();
 }
@@ -570,7 +574,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     const int chunk = avg_rows >= 1024 ? 1 : avg_rows >= 512 ? 2 : 4;
     const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups, chunk);
     if (grid > 0x7fffffff) return MBX_ERANGE;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, k, n, tiles_m, tiles_n, chunk, (int)seg_rows);
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, chunk, (int)seg_rows);
     return launch_status();
   }
   constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
@@ -602,7 +606,7 @@ int gmm_generic(const void* a, const void* b, void* c, const int32_t* bins, int 
   const int64_t gy = ceil_div(m_bound, kGenTile), gx = ceil_div(n, kGenTile);
   if (gy > 65535 || num_groups > 65535) return MBX_ERANGE;
   if (gy == 0 || gx == 0) return 0;
-  gmm_generic_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)num_groups), 256, 0, s>>>(a, b, c, bins, layout, k, n);
+  gmm_generic_kernel<DT><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)num_groups), 256, 0, s>>>(a, b, c, bins, layout, (int)rows, k, n);
   return launch_status();
 }
 

@@ -532,6 +532,8 @@ __device__ __forceinline__ void tile_done() {
   __builtin_amdgcn_s_barrier();
 }
 
+__device__ __forceinline__ int clamp_row(int v, int rows) { return v < 0 ? 0 : (v > rows ? rows : v); }
+
 // ---- NN / NT ----
 // Logical tile id -> (expert, column tile, row tile inside the expert).  Lane l of every wave keeps the
 // inclusive count of tiles up to its experts (one expert per lane up to 64 experts, else a group of
@@ -543,29 +545,32 @@ struct RowTiles {
   int total = 0;
   int per_lane;            // experts per lane: 1 up to 64 experts (the lane then keeps its expert's row range too)
   const int32_t* bins;
-  int num_groups, tiles_n;
+  int num_groups, tiles_n, rows;
 
   static __device__ __forceinline__ int row_tiles(int rows) { return rows > 0 ? (rows + BM - 1) / BM : 0; }
+  // A bin bound as the kernels use it: inside [0, rows] whatever the table holds, so that a table that does not
+  // belong to this operand (stale, or of another batch) can make the result wrong but never an access out of range.
+  __device__ __forceinline__ int bound(int e) const { return clamp_row(bins[e], rows); }
 
-  __device__ __forceinline__ RowTiles(const int32_t* bins_, int num_groups_, int tiles_n_)
-      : bins(bins_), num_groups(num_groups_), tiles_n(tiles_n_) {
+  __device__ __forceinline__ RowTiles(const int32_t* bins_, int num_groups_, int tiles_n_, int rows_)
+      : bins(bins_), num_groups(num_groups_), tiles_n(tiles_n_), rows(rows_) {
     per_lane = (num_groups + kWave - 1) / kWave;
     const int lane = lane_id();
     const int first = lane * per_lane;
     int span = 0;
     if (per_lane == 1) {
       if (lane < num_groups) {
-        lane_end = bins[lane];
-        lane_start = lane > 0 ? bins[lane - 1] : 0;
+        lane_end = bound(lane);
+        lane_start = lane > 0 ? bound(lane - 1) : 0;
         lane_mt = row_tiles(lane_end - lane_start);
       }
       span = lane_mt * tiles_n;
     } else if (first < num_groups) {
       // lane l keeps the tile count of experts l per_lane .. (l + 1) per_lane - 1 and the first row of that group
-      lane_start = first > 0 ? bins[first - 1] : 0;
+      lane_start = first > 0 ? bound(first - 1) : 0;
       int start = lane_start;
       for (int e = first; e < first + per_lane && e < num_groups; ++e) {
-        const int end = bins[e];
+        const int end = bound(e);
         span += row_tiles(end - start) * tiles_n;
         start = end;
       }
@@ -598,7 +603,7 @@ struct RowTiles {
       start = __builtin_amdgcn_readlane(lane_start, l);
       end = start; mt = 0;
       for (e = l * per_lane; e < num_groups; ++e) {
-        end = bins[e];
+        end = bound(e);
         mt = row_tiles(end - start);
         const int span = mt * tiles_n;
         if (id < span) break;
@@ -643,7 +648,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   static_assert(!kSplit || T::BM == 2 * TS::BM, "tail tile");
   const int P = gridDim.x, run = P / kXcds;
   const int xcd = blockIdx.x % kXcds, member = blockIdx.x / kXcds;
-  const RowTiles<T::BM> tiles(bins, num_groups, tiles_n);
+  const RowTiles<T::BM> tiles(bins, num_groups, tiles_n, (int)rows);
   const int total = tiles.total;
   const int full_rounds = total / P, rest = total - full_rounds * P;
   const bool split = kSplit && rest > 0 && 2 * rest <= P;
@@ -758,8 +763,8 @@ __device__ __forceinline__ void tn_tile(Args& g, const uint16_t* __restrict__ a,
 template <int DT, typename T, typename TS, bool SEGMENTED>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
-              const int32_t* __restrict__ bins, int num_groups, int k, int n, int tiles_m, int tiles_n, int chunk,
-              int seg_rows) {
+              const int32_t* __restrict__ bins, int num_groups, int rows, int k, int n, int tiles_m, int tiles_n,
+              int chunk, int seg_rows) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "last-row tile");
   constexpr bool kMixed = T::BM != TS::BM;
@@ -803,7 +808,10 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
     if (tm >= tiles_m || tn >= tiles_n) continue;   // padding of the block enumeration (uniform over the workgroup)
     int e = slot;
     if (ranked) e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(__ballot(rank == slot)));
-    const int start = e > 0 ? bins[e - 1] : 0, end = bins[e];
+    // bounds inside [0, rows] and in order whatever the table holds: a wrong table cannot take a load out of range
+    const int start = e > 0 ? clamp_row(bins[e - 1], rows) : 0;
+    int end = clamp_row(bins[e], rows);
+    end = end < start ? start : end;
     g.a_r0 = tm * T::BM;
     g.b_r0 = tn * T::BN;
     uint16_t* const c_e = c + (int64_t)e * k * n;

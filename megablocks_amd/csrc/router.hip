@@ -26,8 +26,8 @@ __device__ __forceinline__ float wave_pnorm(float w, bool live, float p) {
 
 // scores = softmax(logits) rounded to the storage type (computed in fp32: exp(x - max) / sum, as
 // torch's softmax does for 16-bit inputs); the k largest rounded scores in descending order, ties to the
-// lower expert index; weights = those scores, divided by their rounded p-norm if p > 0 (each of torch's
-// two operations rounds to the storage type).
+// lower expert index (NaN scores first); weights = those scores, divided by their rounded p-norm if p > 0
+// (each of torch's two operations rounds to the storage type).
 template <int DT, int R>
 __global__ void __launch_bounds__(kTokenThreads)
 router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_experts, int top_k, float p,
@@ -60,7 +60,11 @@ router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_
       const int e = lane + r * kWave;
       const E s = Elem<DT>::from_f32(x[r] / sum);
       if (e < num_experts) scores[t * num_experts + e] = s;
-      x[r] = e < num_experts ? Elem<DT>::to_f32(s) : -1.f;   // scores are >= 0: -1 marks "not a candidate"
+      // The selection key: the rounded score; -1 marks "not a candidate" (scores are >= 0).  A NaN score (a NaN
+      // or +inf logit makes the whole row NaN) ranks above every number, as torch.topk ranks it, so that the
+      // indices written are always experts: +inf, which no score can be, stands for it.
+      const float v = Elem<DT>::to_f32(s);
+      x[r] = e < num_experts ? (v != v ? INFINITY : v) : -1.f;
     }
     float my_w = 0.f;
     int my_i = 0;
@@ -76,7 +80,7 @@ router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_
         const int oe = __shfl_xor(best_e, off, 64);
         if (ov > best || (ov == best && oe < best_e)) { best = ov; best_e = oe; }
       }
-      if (lane == j) { my_w = best; my_i = best_e; }
+      if (lane == j) { my_w = best == INFINITY ? NAN : best; my_i = best_e; }
 #pragma unroll
       for (int r = 0; r < R; ++r)
         if (lane + r * kWave == best_e) x[r] = -1.f;

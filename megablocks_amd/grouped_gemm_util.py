@@ -21,26 +21,54 @@ def assert_grouped_gemm_is_available():
     assert grouped_gemm_is_available()
 
 
-def _device_bins(batch_sizes: torch.Tensor, device) -> torch.Tensor:
-    """Inclusive int32 row bins on the device for a vector of group sizes (cached on the tensor; not under stream
-    capture, where a graph must contain the kernel that computes the bins it uses)."""
+def _device_bins(batch_sizes: torch.Tensor, device, rows: int) -> torch.Tensor:
+    """Inclusive int32 row bins on the device for a vector of group sizes that must add up to `rows`.
+
+    Sizes on the host (what the reference passes, mlp.py:502) are checked here, as grouped_gemm checks them: negative
+    sizes or a sum other than `rows` raise ValueError.  Sizes on the device cannot be checked without a
+    synchronisation; the kernels keep every bin bound inside [0, rows], so a table that does not match the operands
+    gives wrong values, never an access out of range.
+
+    The bins are kept on the `batch_sizes` tensor and reused while its `_version` is unchanged, i.e. while no torch
+    operation has written to it.  A write torch does not see (a kernel launched on its raw pointer, the replay of
+    a captured graph into it) does not invalidate them: hand such a tensor to `forget_bins` first, or pass a new
+    one.  Nothing is kept or reused under stream capture, where a graph must contain the kernel that computes
+    the bins it uses."""
+    if batch_sizes.ndim != 1:
+        raise ValueError('batch_sizes must be a vector')
     capturing = batch_sizes.is_cuda and torch.cuda.is_current_stream_capturing()
     cached = getattr(batch_sizes, '_mbx_bins', None)
     if not capturing and cached is not None and cached[1] == batch_sizes._version and cached[0].device == device:
+        if cached[2] is not None and cached[2] != rows:
+            raise ValueError(f'gmm: batch_sizes add up to {cached[2]} rows but the operand has {rows}')
         return cached[0]
-    if batch_sizes.ndim != 1:
-        raise ValueError('batch_sizes must be a vector')
+    total = None
     if batch_sizes.is_cuda:
         from megablocks_amd.ops.routing import inclusive_cumsum
         bins = inclusive_cumsum(batch_sizes.to(torch.int32), 0).view(-1)
     else:
+        total = int(batch_sizes.sum()) if batch_sizes.numel() else 0
+        if batch_sizes.numel() and int(batch_sizes.min()) < 0:
+            raise ValueError('gmm: batch_sizes must not be negative')
+        if total != rows:
+            raise ValueError(f'gmm: batch_sizes add up to {total} rows but the operand has {rows}')
         bins = torch.cumsum(batch_sizes, 0).to(torch.int32).to(device)
     if not capturing:
-        try:
-            batch_sizes._mbx_bins = (bins, batch_sizes._version)
-        except Exception:
-            pass
+        _remember(batch_sizes, (bins, batch_sizes._version, total))
     return bins
+
+
+def _remember(batch_sizes: torch.Tensor, entry):
+    try:
+        batch_sizes._mbx_bins = entry
+    except AttributeError:   # a tensor type without instance attributes: the bins are computed on every call
+        pass
+
+
+def forget_bins(batch_sizes: torch.Tensor):
+    """Drops the bins kept for `batch_sizes` (for a tensor whose contents were changed behind torch's back)."""
+    if getattr(batch_sizes, '_mbx_bins', None) is not None:
+        batch_sizes._mbx_bins = None
 
 
 def note_bins(batch_sizes: torch.Tensor, bins: torch.Tensor):
@@ -48,10 +76,7 @@ def note_bins(batch_sizes: torch.Tensor, bins: torch.Tensor):
     it over, and the products of this step do not compute it again."""
     if batch_sizes.is_cuda and bins.dtype == torch.int32 and bins.device == batch_sizes.device \
             and bins.numel() == batch_sizes.numel() and not torch.cuda.is_current_stream_capturing():
-        try:
-            batch_sizes._mbx_bins = (bins.view(-1), batch_sizes._version)
-        except Exception:
-            pass
+        _remember(batch_sizes, (bins.view(-1), batch_sizes._version, None))
 
 
 def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None, _record_as=None):
@@ -70,9 +95,9 @@ def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None, _record_as=None
         raise ValueError('gmm: trans_a and trans_b cannot both be set')
     dt = _lib.dtype_of(a)
     a, b = a.contiguous(), b.contiguous()
-    bins = _device_bins(batch_sizes, a.device)
-    groups = bins.shape[0]
     rows = a.shape[0]
+    bins = _device_bins(batch_sizes, a.device, rows)
+    groups = bins.shape[0]
     if trans_a:
         if b.ndim != 2 or b.shape[0] != rows:
             raise ValueError('gmm(trans_a): b must be [rows, n]')
@@ -113,7 +138,7 @@ def gmm_dual(a, b, a2, b2, batch_sizes, trans_b=False, c=None):
     if a.ndim != 2 or b.ndim != 3 or a.dtype != b.dtype:
         raise ValueError('gmm_dual: a must be [rows, k] and b [num_groups, ., .] of the same dtype')
     a, b, a2, b2 = a.contiguous(), b.contiguous(), a2.contiguous(), b2.contiguous()
-    bins = _device_bins(batch_sizes, a.device)
+    bins = _device_bins(batch_sizes, a.device, a.shape[0])
     groups, rows, k = bins.shape[0], a.shape[0], a.shape[1]
     n, layout = (b.shape[1], _lib.NT) if trans_b else (b.shape[2], _lib.NN)
     if b.shape[0] != groups or (b.shape[2] if trans_b else b.shape[1]) != k:

@@ -70,13 +70,22 @@ class _RouterLinear(torch.autograd.Function):
         return sizes
 
     @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
     def forward(ctx: Any, x: torch.Tensor, weight: torch.Tensor):
+        # Under autocast the product runs in x's 16-bit type, as torch's own linear would; the cast weight is
+        # what the backward multiplies with, and the weight gradient goes back in the parameter's type (fp32
+        # master weights).  Outside autocast mismatched types are an error, as for torch.nn.Linear.
+        ctx.weight_dtype = weight.dtype
+        if weight.dtype != x.dtype and torch.is_autocast_enabled():
+            weight = weight.to(x.dtype)
         ctx.save_for_backward(x, weight)
         return torch.nn.functional.linear(x, weight)
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
     def backward(ctx: Any, grad: torch.Tensor):
         x, weight = ctx.saved_tensors
+        grad = grad.to(x.dtype)
         dx = grad @ weight if ctx.needs_input_grad[0] else None
         dw = None
         if ctx.needs_input_grad[1]:
@@ -84,7 +93,7 @@ class _RouterLinear(torch.autograd.Function):
             sizes = _RouterLinear.piece_sizes(x.shape[0])
             pieces = sizes.shape[0]
             parts = gg.gmm(grad.contiguous(), x.contiguous(), sizes, trans_a=True, _record_as='router_wgrad')   # [pieces, E, h]
-            dw = parts[0] if pieces == 1 else parts.float().sum(0).to(weight.dtype)
+            dw = (parts[0] if pieces == 1 else parts.float().sum(0)).to(ctx.weight_dtype)
         return dx, dw
 
 
@@ -156,6 +165,9 @@ class LearnedRouter(torch.nn.Module):
         else:
             logits = self.layer(x2d)
         _save_router_logits(logits, self.args)
+        if logits.is_cuda and logits.dtype != torch.float32 and torch.is_autocast_enabled():
+            # autocast runs softmax in fp32 (router.py:98 under torch.autocast): scores and weights come out in fp32
+            logits = logits.float()
         if FUSED_SOFTMAX_TOPK and _SoftmaxTopK.supported(logits, self.args.moe_top_k):
             scores, expert_weights, expert_indices = _SoftmaxTopK.apply(
                 logits, self.args.moe_top_k, self.args.moe_normalize_expert_weights or 0)

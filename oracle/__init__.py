@@ -32,3 +32,6 @@ from oracle.gmm import gmm  # noqa: F401
 from oracle.layers import (  # noqa: F401
     gelu_tanh_backward, router_forward, dmoe_forward,
 )
+from oracle.losses import (  # noqa: F401
+    load_balancing_loss, layer_load_balancing_loss, router_zloss, uniform_expert_assignment,
+)

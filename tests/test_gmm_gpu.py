@@ -121,10 +121,47 @@ def test_gmm_c_argument_and_errors(gg):
         gg.backend.gmm(a, b.float(), sizes)
     with pytest.raises(ValueError):
         gg.backend.gmm(a, b, sizes, trans_b=True)
-    short = torch.tensor([60, 20])                                # rows past the last bin are left alone
-    c2 = torch.full((128, 32), 7.0).bfloat16().cuda()
-    gg.backend.gmm(a, b, short, c=c2)
+    short = torch.tensor([60, 20])
+    with pytest.raises(ValueError):                               # sizes on the host are checked against the operand
+        gg.backend.gmm(a, b, short)
+    with pytest.raises(ValueError):
+        gg.backend.gmm(a, b, torch.tensor([130, -2]))
+    with pytest.raises(ValueError):
+        gg.backend.gmm(a, a, short, trans_a=True)
+    c2 = torch.full((128, 32), 7.0).bfloat16().cuda()             # sizes on the device cannot be: rows past the last
+    gg.backend.gmm(a, b, short.cuda(), c=c2)                      # bin are left alone
     assert bool((c2[80:] == 7.0).all()) and rel_err(c2[:80].cpu(), oracle.gmm(a[:80].cpu(), b.cpu(), short)) < TOL
+
+
+@pytest.mark.parametrize('dtype,k,n', [(torch.bfloat16, 256, 512), (torch.bfloat16, 72, 40), (torch.float32, 64, 64),
+                                       (torch.bfloat16, 1 << 16, 64)])
+@pytest.mark.parametrize('mode', ['nn', 'nt', 'tn'])
+def test_gmm_bins_that_do_not_match_the_operands_stay_in_range(gg, dtype, k, n, mode):
+    """Device-side sizes that add up to more rows than the operands have (a stale table), or that are negative:
+    the values are then unspecified, but no kernel reads or writes outside the operands -- the rows behind the
+    output and a guard region around it keep their canary."""
+    if k > 4096 and mode != 'nn':
+        pytest.skip('the long-k case exercises the register-staged NN fallback only')
+    rows, groups = 700, 4
+    a = torch.randn(rows, k, device='cuda').to(dtype)
+    if mode == 'tn':
+        b = torch.randn(rows, n, device='cuda').to(dtype)
+        shape = (groups, k, n)
+    else:
+        b = torch.randn(groups, n, k, device='cuda').to(dtype) if mode == 'nt' else torch.randn(groups, k, n, device='cuda').to(dtype)
+        shape = (rows, n)
+    numel = shape[0] * shape[1] * (shape[2] if len(shape) == 3 else 1)
+    for sizes in ([300, 300, 300, 300], [900, 0, 0, 0], [200, -50, 400, 5000], [-7, 2000, -2000, 100]):
+        guard = 4096
+        buf = torch.full((numel + 2 * guard,), 3.0, device='cuda', dtype=dtype)
+        c = buf[guard:guard + numel].view(shape)
+        gg.backend.gmm(a, b, torch.tensor(sizes, dtype=torch.int32, device='cuda'), trans_a=mode == 'tn', trans_b=mode == 'nt', c=c)
+        torch.cuda.synchronize()
+        assert bool((buf[:guard] == 3.0).all()) and bool((buf[guard + numel:] == 3.0).all())
+    # a table that does match still gives the product
+    good = torch.tensor([100, 0, 250, 350], dtype=torch.int32, device='cuda')
+    got = gg.backend.gmm(a, b, good, trans_a=mode == 'tn', trans_b=mode == 'nt')
+    assert rel_err(got.float(), _ref_gpu(a, b, good.cpu(), mode == 'tn', mode == 'nt')) < TOL
 
 
 BIG = [  # name, groups, rows, hidden, ffn, skew

@@ -24,7 +24,10 @@ def syn():
     return synthetic
 
 
-def _oracle_step(w, inp, routing_given):
+def _oracle_step(w, inp, routing_given, top_experts=None):
+    """fp32 forward + backward of the oracle.  With the router in the chain, `top_experts` (the layer's own choice:
+    a 16-bit router breaks near-ties differently from fp32) replaces the oracle's top-k; the weights are then the
+    oracle's own fp32 scores at those experts, renormalised as router.py:100-106 does."""
     x = inp['x'].clone().requires_grad_(True)
     rw = inp['router_weight'].clone().requires_grad_(True)
     w1, w2 = inp['w1'].clone().requires_grad_(True), inp['w2'].clone().requires_grad_(True)
@@ -33,7 +36,12 @@ def _oracle_step(w, inp, routing_given):
         ew = inp['expert_weights'].clone().requires_grad_(True)
         te = inp['top_experts']
     else:
-        _, ew, te = oracle.router_forward(x, rw, w.top_k, w.normalize)
+        scores, ew, te = oracle.router_forward(x, rw, w.top_k, w.normalize)
+        if top_experts is not None:
+            te = top_experts
+            ew = scores.gather(1, te)
+            if w.normalize:
+                ew = ew / torch.norm(ew, p=w.normalize, dim=-1, keepdim=True)
     out, tpe = oracle.dmoe_forward(x, ew, te, w1, w2, v1, num_experts=w.experts, top_k=w.top_k,
                                    activation=w.activation())
     out.backward(inp['grad'])
@@ -55,6 +63,8 @@ CASES = [  # tokens, hidden, ffn, experts, top_k, mlp_type, mlp_impl, routing
     (512, 256, 512, 8, 2, 'mlp', 'sparse', 'logits'),
     (512, 256, 512, 8, 2, 'glu', 'sparse', 'logits'),
     (300, 72, 136, 5, 3, 'mlp', 'grouped', 'logits'),          # sizes off the MFMA fast path
+    (2048, 256, 512, 8, 2, 'glu', 'grouped', 'router'),        # enough tokens for the router's grouped weight gradient
+    (1536, 128, 256, 16, 1, 'mlp', 'sparse', 'router'),
 ]
 
 
@@ -75,20 +85,18 @@ def test_dmoe_forward_backward_vs_oracle(syn, tokens, hidden, ffn, experts, top_
             if inp[k] is not None:
                 inp[k] = inp[k].to(dtype).float()
     given = routing != 'router'
-    want, want_tpe, want_grads, te = _oracle_step(w, inp, given)
-
     layer = syn.build_layer(w, inp, memory_optimized=memopt)
     x = inp['x'].to(dtype).cuda().requires_grad_(True)
     grad = inp['grad'].to(dtype).cuda()
     if given:
         ew = inp['expert_weights'].to(dtype).cuda().requires_grad_(True)
         routing_t = (inp['scores'].to(dtype).cuda(), ew, inp['top_experts'].cuda())
+        own_choice = None
     else:
         routing_t = None
-        # a bf16 router may pick other experts than the fp32 oracle on near-ties: route with the oracle's choice
-        scores, ew_r, te_r = layer.router(x)
-        if not torch.equal(te_r.cpu(), te):
-            pytest.skip('router tie broken differently in reduced precision; covered by the given-routing cases')
+        with torch.no_grad():   # the experts the layer's own router picks for these inputs
+            own_choice = layer.router(x)[2].cpu()
+    want, want_tpe, want_grads, te = _oracle_step(w, inp, given, own_choice)
     out = syn.layer_step(layer, w, x, grad, routing_t)
 
     tol = 1e-4 if dtype == torch.float32 else 1e-2                 # f16 has three more mantissa bits than bf16: same bound
@@ -204,6 +212,36 @@ def test_router_softmax_topk_backward(dtype, experts, top_k, norm_p, with_score_
     assert rel_err(x.grad, xr.grad) < (1e-5 if dtype == torch.float32 else 1e-2)
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_router_softmax_topk_with_nan_and_inf_logits(dtype):
+    """A NaN or +inf logit makes its row of scores NaN (as torch's softmax does); torch.topk ranks NaN above every
+    number and still returns expert indices.  The fused kernel does too: indices stay inside [0, E), distinct per
+    token, and the other rows are untouched."""
+    from megablocks_amd.layers.router import _SoftmaxTopK
+    tokens, experts, top_k = 64, 8, 2
+    torch.manual_seed(0)
+    logits = torch.randn(tokens, experts, device='cuda').to(dtype)
+    clean = _SoftmaxTopK.apply(logits, top_k, 1)
+    bad = logits.clone()
+    bad[3, 5] = float('nan')
+    bad[10, 0] = float('inf')
+    bad[20, :] = float('nan')
+    s, w, i = _SoftmaxTopK.apply(bad, top_k, 1)
+    assert int(i.min()) >= 0 and int(i.max()) < experts
+    assert bool((i[:, 0] != i[:, 1]).all())
+    ref_s = bad.float().softmax(-1)
+    for t in (3, 10, 20):
+        assert bool(torch.isnan(s[t]).all()) and bool(torch.isnan(ref_s[t]).all()) and bool(torch.isnan(w[t]).all())
+        assert i[t].tolist() == [0, 1]                              # equal ranks are taken in ascending expert index
+    keep = torch.ones(tokens, dtype=torch.bool, device='cuda')
+    keep[[3, 10, 20]] = False
+    for got, want in zip((s, w, i), clean):
+        assert torch.equal(got[keep], want[keep])
+    # downstream: every slot lands in a bin, so the permuted buffers have no unowned rows
+    import megablocks_amd.ops as ops
+    assert int(ops.histogram(i.flatten().int(), experts).sum()) == tokens * top_k
+
+
 def test_router_falls_back_to_torch_for_many_experts():
     from megablocks_amd.layers.arguments import Arguments
     from megablocks_amd.layers.router import LearnedRouter
@@ -270,6 +308,67 @@ def test_full_size_layer_properties(syn, name):
                     h = h * (v1[e].float() @ xt)
                 want[r] += ew[t, j] * (w2[e].float().t() @ h)
         assert rel_err(out[rows], want) < 2e-2
+
+    # Reference values for the backward, in fp32 on the GPU from the definition (autograd): the weight gradients
+    # of one expert that has tokens, and the input gradient of the sampled tokens (with the router's share where
+    # the router is part of the step).
+    g1 = dict(zip(['x', 'w1', 'w2'] + (['v1'] if v1 is not None else []) + (['router'] if routing_t is None else []), g1))
+    flat_te = te.flatten()
+    counts = torch.bincount(flat_te, minlength=w.experts)
+    e = int(torch.nonzero(counts > 0).flatten()[w.experts // 2 % int((counts > 0).sum())])
+    slots = torch.nonzero(flat_te == e).flatten()
+    xe = x.detach()[slots // w.top_k].float()
+    ge = grad[slots // w.top_k].float() * ew.flatten()[slots].unsqueeze(1)      # what reaches the expert's output rows
+    pw = [w1[e].detach().float().requires_grad_(True), w2[e].detach().float().requires_grad_(True)]
+    if v1 is not None:
+        pw.append(v1[e].detach().float().requires_grad_(True))
+    h = act(xe @ pw[0].t())
+    if v1 is not None:
+        h = h * (xe @ pw[2].t())
+    ((h @ pw[1]) * ge).sum().backward()
+    f0, f1 = e * w.ffn, (e + 1) * w.ffn
+    assert rel_err(g1['w1'][f0:f1], pw[0].grad) < 1e-2
+    assert rel_err(g1['w2'][f0:f1], pw[1].grad) < 1e-2
+    if v1 is not None:
+        assert rel_err(g1['v1'][f0:f1], pw[2].grad) < 1e-2
+
+    xs = x.detach()[rows].float().requires_grad_(True)
+    if routing_t is None:
+        sc = (xs @ layer.router.layer.weight.detach().float().t()).softmax(-1)
+        ws = sc.gather(1, te[rows])
+        if w.normalize:
+            ws = ws / torch.norm(ws, p=w.normalize, dim=-1, keepdim=True)
+    else:
+        ws = ew[rows]
+    total = 0
+    for r, t in enumerate(rows):
+        for j in range(w.top_k):
+            ex = int(te[t, j])
+            hh = act(w1[ex].detach().float() @ xs[r])
+            if v1 is not None:
+                hh = hh * (v1[ex].detach().float() @ xs[r])
+            total = total + ws[r, j] * ((w2[ex].detach().float().t() @ hh) * grad[t].float()).sum()
+    total.backward()
+    assert rel_err(g1['x'][rows], xs.grad) < 2e-2
+
+
+def test_c1_full_size_fp32_vs_oracle(syn):
+    """Workload c1 (4096 tokens, hidden 1024, ffn 4096, 8 experts, top-2, fp32) at full size against the CPU oracle:
+    forward and every gradient, 1e-4."""
+    w = syn.WORKLOADS['c1']
+    inp = syn.make_inputs(w, seed=0)
+    layer = syn.build_layer(w, inp)
+    x = inp['x'].cuda().requires_grad_(True)
+    with torch.no_grad():
+        own_choice = layer.router(x)[2].cpu()
+    want, want_tpe, want_grads, _ = _oracle_step(w, inp, False, own_choice)
+    out = syn.layer_step(layer, w, x, inp['grad'].cuda(), None)
+    assert torch.equal(own_choice, oracle.router_forward(inp['x'], inp['router_weight'], w.top_k, w.normalize)[2])
+    assert out.dtype == torch.float32 and rel_err(out, want) < 1e-4
+    assert rel_err(x.grad, want_grads['x']) < 1e-4
+    assert rel_err(layer.experts.mlp.w1.grad, want_grads['w1']) < 1e-4
+    assert rel_err(layer.experts.mlp.w2.grad, want_grads['w2']) < 1e-4
+    assert rel_err(layer.router.layer.weight.grad, want_grads['router']) < 5e-4
 
 
 def test_routing_bookkeeping_is_bit_exact(syn):
@@ -474,19 +573,23 @@ def test_autocast_with_fp32_parameters_equals_the_bf16_layer(mlp_type, mlp_impl,
         for p16, p32 in zip(half.parameters(), master.parameters()):
             assert p32.dtype == torch.float32 and p16.dtype == torch.bfloat16
             p16.copy_(p32)
-    x = torch.randn(64, 4, 256, device='cuda')
+    x = torch.randn(512, 4, 256, device='cuda')          # 2048 tokens: the router's weight gradient takes the grouped kernel
     x32 = x.clone().requires_grad_(True)
     x16 = x.bfloat16().requires_grad_(True)
-    grad = torch.randn(64, 4, 256, device='cuda').bfloat16()
+    grad = torch.randn(512, 4, 256, device='cuda').bfloat16()
     with torch.autocast('cuda', dtype=torch.bfloat16):
+        scores, weights, _ = master.router(x32.detach().bfloat16())
         out = master(x32)
     out.backward(grad)
     want = half(x16)
     want.backward(grad)
-    assert out.dtype == torch.bfloat16 and torch.equal(out, want)
-    assert x32.grad.dtype == torch.float32 and rel_err(x32.grad, x16.grad) < 1e-6
-    for p32, p16 in zip(master.parameters(), half.parameters()):
-        assert p32.grad.dtype == torch.float32 and rel_err(p32.grad, p16.grad) < 1e-6
+    # autocast runs the router's softmax in fp32 (router.py:98 under torch.autocast), so scores and expert weights are
+    # fp32 there and bf16 in the bf16 layer: equal up to that rounding, not bit for bit
+    assert scores.dtype == torch.float32 and weights.dtype == torch.float32
+    assert out.dtype == torch.bfloat16 and rel_err(out, want) < 5e-3
+    assert x32.grad.dtype == torch.float32 and rel_err(x32.grad, x16.grad) < 5e-3
+    for (name, p32), p16 in zip(master.named_parameters(), half.parameters()):
+        assert p32.grad.dtype == torch.float32 and rel_err(p32.grad, p16.grad) < (2e-2 if 'router' in name else 5e-3), name
 
 
 def test_parameter_names_and_shapes_are_the_reference_checkpoint_layout():
@@ -526,6 +629,136 @@ def test_forward_shapes_bias_and_losses():
     router.clear_router_zloss()
     layer2 = dMoE(dataclasses.replace(args, return_bias=False))
     assert layer2(x.detach()).shape == x.shape
+
+
+@pytest.mark.parametrize('dtype,in_fp32', [(torch.float32, False), (torch.bfloat16, True), (torch.bfloat16, False)])
+@pytest.mark.parametrize('tokens,hs,ne,top_k,layers', [(96, 128, 4, 2, 1), (2048, 256, 8, 2, 1), (300, 64, 16, 4, 2)])
+def test_auxiliary_losses_match_oracle(dtype, in_fp32, tokens, hs, ne, top_k, layers):
+    """batched_load_balancing_loss (moe.py:32-89), ParallelMLP.load_balancing_loss (moe.py:138-150) and
+    batched_router_zloss (router.py:25-42): the values the layers report and the router weight gradient they
+    produce, against the oracle fed with the same routing decision."""
+    from megablocks_amd.layers import moe, router
+    from megablocks_amd.layers.dmoe import dMoE
+    torch.manual_seed(tokens + ne)
+    lw, zw = 0.1, 1e-3
+    args = _args(hidden_size=hs, ffn_hidden_size=2 * hs, moe_num_experts=ne, moe_top_k=top_k, moe_loss_weight=lw,
+                 moe_zloss_weight=zw, num_layers=layers, bf16=dtype == torch.bfloat16, moe_lbl_in_fp32=in_fp32,
+                 moe_zloss_in_fp32=in_fp32, moe_normalize_expert_weights=1 if top_k > 1 else None)
+    moe.clear_load_balancing_loss()
+    router.clear_router_zloss()
+    models = [dMoE(args) for _ in range(layers)]
+    for m in models:
+        m.train()
+    xs = [torch.randn(tokens, 1, hs, device='cuda').to(dtype) for _ in range(layers)]
+    outs = [m(x) for m, x in zip(models, xs)]
+    saved = moe.get_load_balancing_loss()
+    assert len(saved) == layers and all(t.shape == (ne,) and sc.shape == (tokens, ne) for t, sc in saved)
+    lbl = moe.batched_load_balancing_loss(args)
+    zloss = router.batched_router_zloss(args)
+    assert zloss.shape == (layers,)
+    per_layer = models[0].experts.load_balancing_loss(saved[0][0], saved[0][1])
+    (lbl + zloss.sum()).backward()
+
+    # oracle: fp32 router on the same (rounded) inputs, counts from the layer's own expert choice
+    rws = [m.router.layer.weight.detach().float().cpu().requires_grad_(True) for m in models]
+    logits = [x.view(tokens, hs).float().cpu() @ rw.t() for x, rw in zip(xs, rws)]
+    scores = [lg.softmax(-1) for lg in logits]
+    counts = [t.cpu() for t, _ in saved]
+    for c, sc, (_, got_sc) in zip(counts, scores, saved):
+        assert int(c.sum()) == tokens * top_k
+        assert rel_err(got_sc, sc) < (1e-5 if dtype == torch.float32 else 1e-2)
+    want_lbl = oracle.load_balancing_loss(counts, scores, num_experts=ne, top_k=top_k, loss_weight=lw, num_layers=layers)
+    want_z = oracle.router_zloss(logits, zloss_weight=zw)
+    # 16-bit scores / logits reduced in 16 bits (the reference's default, moe_lbl_in_fp32 = moe_zloss_in_fp32 = False)
+    # carry a few rounding steps of 2^-9 each
+    tol = 1e-5 if dtype == torch.float32 else (1e-2 if in_fp32 else 3e-2)
+    loss_dtype = torch.float32 if in_fp32 else dtype
+    assert lbl.dtype == loss_dtype and abs(float(lbl) - float(want_lbl)) < tol * abs(float(want_lbl))
+    assert zloss.dtype == loss_dtype and rel_err(zloss, want_z) < tol
+    want_one = oracle.layer_load_balancing_loss(counts[0], scores[0], top_k=top_k)
+    assert abs(float(per_layer) - float(want_one)) < tol * abs(float(want_one))
+    (want_lbl + want_z.sum()).backward()
+    for m, rw in zip(models, rws):
+        assert rel_err(m.router.layer.weight.grad, rw.grad) < (1e-4 if dtype == torch.float32 else (2e-2 if in_fp32 else 5e-2))
+    del outs
+    moe.clear_load_balancing_loss()
+    router.clear_router_zloss()
+    assert moe.get_load_balancing_loss() == [] and moe.batched_load_balancing_loss(_args(moe_loss_weight=0.0)) == 0.0
+
+
+def test_load_balancing_loss_closed_forms_on_the_layer():
+    """Evenly loaded experts give loss_weight whatever the scores (uniform_expert_assignment makes them even);
+    the wrong number of saved layers raises as moe.py:42-60 does."""
+    from megablocks_amd.layers import moe
+    from megablocks_amd.layers.dmoe import dMoE
+    moe.clear_load_balancing_loss()
+    args = _args(moe_num_experts=8, moe_top_k=2, moe_loss_weight=0.25, uniform_expert_assignment=True)
+    layer = dMoE(args)
+    layer.train()
+    layer(torch.randn(64, 4, 128, device='cuda').bfloat16())
+    tpe, _ = moe.get_load_balancing_loss()[0]
+    assert tpe.tolist() == [64] * 8
+    assert abs(float(moe.batched_load_balancing_loss(args)) - 0.25) < 1e-3
+    layer(torch.randn(64, 4, 128, device='cuda').bfloat16())
+    with pytest.raises(ValueError):
+        moe.batched_load_balancing_loss(args)          # two saved layers, num_layers = 1
+    moe.clear_load_balancing_loss()
+    layer.eval()
+    layer(torch.randn(64, 4, 128, device='cuda').bfloat16())
+    assert moe.get_load_balancing_loss() == []         # saved in training mode only (moe.py:430-431)
+
+
+@pytest.mark.parametrize('mlp_impl', ['grouped', 'sparse'])
+def test_uniform_expert_assignment_routes_round_robin(mlp_impl):
+    """router.py:49-58,108-113: expert of slot i is i mod E (the weights stay the router's top-k scores); the layer
+    output is the oracle's for that assignment."""
+    from megablocks_amd.layers.dmoe import dMoE
+    torch.manual_seed(11)
+    tokens, hs, ne, top_k = 200, 128, 8, 2
+    layer = dMoE(_args(hidden_size=hs, ffn_hidden_size=256, moe_num_experts=ne, moe_top_k=top_k, mlp_impl=mlp_impl,
+                       uniform_expert_assignment=True))
+    x = torch.randn(tokens, 1, hs, device='cuda').bfloat16()
+    scores, weights, top = layer.router(x)
+    assert top.dtype == torch.int64 and torch.equal(top.cpu(), oracle.uniform_expert_assignment((tokens, top_k), ne))
+    assert torch.equal(weights, torch.topk(scores, top_k, dim=-1).values)
+    out = layer(x)
+    m = layer.experts.mlp
+    want, tpe = oracle.dmoe_forward(x.view(tokens, hs).float().cpu(), weights.float().cpu(), top.cpu(),
+                                    m.w1.detach().float().cpu(), m.w2.detach().float().cpu(), num_experts=ne, top_k=top_k)
+    assert tpe.tolist() == [tokens * top_k // ne] * ne
+    assert rel_err(out.view(tokens, hs), want) < 1e-2
+
+
+def test_router_jitter():
+    """router.py:81-85,93-94: in training mode the router input is multiplied element-wise by uniform noise from
+    [1 - eps, 1 + eps); nothing is drawn in eval mode or when moe_jitter_eps is None."""
+    from megablocks_amd.layers.router import LearnedRouter
+    eps = 0.25
+    args = _args(hidden_size=256, moe_num_experts=8, moe_top_k=2, moe_jitter_eps=eps, bf16=False)
+    router = LearnedRouter(args)
+    x = torch.randn(4096, 256, device='cuda')
+    noise = router.jitter(x)
+    assert noise.shape == x.shape and noise.dtype == x.dtype
+    assert float(noise.min()) >= 1 - eps and float(noise.max()) <= 1 + eps
+    assert abs(float(noise.mean()) - 1.0) < 2e-3 and abs(float(noise.std()) - 2 * eps / 12 ** 0.5) < 2e-3
+    rw = router.layer.weight.detach().cpu()
+    router.eval()
+    s_eval, w_eval, i_eval = router(x)
+    want_s, want_w, want_i = oracle.router_forward(x.cpu(), rw, 2)
+    assert torch.allclose(s_eval.cpu(), want_s, rtol=1e-4, atol=1e-6) and torch.equal(i_eval.cpu(), want_i)
+    router.train()
+    torch.manual_seed(5)
+    s_train, w_train, i_train = router(x)
+    torch.manual_seed(5)
+    jittered = x * router.jitter(x)                     # the same draw
+    want_s, want_w, want_i = oracle.router_forward(jittered.cpu(), rw, 2)
+    assert torch.allclose(s_train.cpu(), want_s, rtol=1e-4, atol=1e-6) and torch.equal(i_train.cpu(), want_i)
+    assert torch.allclose(w_train.cpu(), want_w, rtol=1e-4, atol=1e-6)
+    assert not torch.equal(s_train, s_eval)
+    state = torch.cuda.get_rng_state()
+    LearnedRouter(_args(hidden_size=256, moe_num_experts=8, moe_jitter_eps=None)).train()(x.bfloat16())
+    router.eval()(x)
+    assert torch.equal(state, torch.cuda.get_rng_state())      # no draw without jitter
 
 
 def test_memory_optimized_requires_all_grads():

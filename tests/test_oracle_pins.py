@@ -449,3 +449,89 @@ def test_c_oracle_topology_replicate_route(rc):
         got = rc.route(te, experts, oracle.routing.sort_end_bit(experts), 128)
         for w, t in zip(want, got):
             assert torch.equal(w.view(-1), t.view(-1))
+
+
+# ---------------------------------------------------------------- auxiliary losses
+def _lbl_loop(counts_per_layer, scores_per_layer, ne, top_k, weight):
+    """moe.py:32-89 element by element in Python floats."""
+    layers = len(counts_per_layer)
+    tokens = len(scores_per_layer[0])
+    dot = 0.0
+    for counts, scores in zip(counts_per_layer, scores_per_layer):
+        for e in range(ne):
+            col = sum(row[e] for row in scores)
+            dot += counts[e] * (col / tokens if tokens else col)
+    return ne * weight / (layers * tokens * top_k) * dot
+
+
+@pytest.mark.parametrize('tokens,ne,top_k,layers', [(7, 3, 1, 1), (16, 4, 2, 1), (33, 8, 3, 2), (5, 2, 2, 3)])
+def test_load_balancing_loss_loop(tokens, ne, top_k, layers):
+    g = torch.Generator().manual_seed(tokens * ne)
+    scores = [torch.randn(tokens, ne, generator=g).softmax(-1) for _ in range(layers)]
+    counts = [oracle.histogram(torch.topk(s, top_k, -1).indices.flatten().int(), ne) for s in scores]
+    want = _lbl_loop([c.tolist() for c in counts], [s.tolist() for s in scores], ne, top_k, 0.1)
+    got = oracle.load_balancing_loss(counts, scores, num_experts=ne, top_k=top_k, loss_weight=0.1)
+    assert abs(float(got) - want) <= 1e-6 * abs(want)
+    if layers == 1:   # the per-layer form of moe.py:138-150 is the same quantity without the weight
+        one = oracle.layer_load_balancing_loss(counts[0], scores[0], top_k=top_k)
+        assert abs(float(one) * 0.1 - want) <= 1e-6 * abs(want)
+
+
+def test_load_balancing_loss_closed_forms():
+    ne, top_k, tokens, w = 8, 2, 64, 0.25
+    g = torch.Generator().manual_seed(1)
+    scores = torch.randn(tokens, ne, generator=g).softmax(-1)
+    # evenly loaded experts: <counts, mean scores> = tokens * top_k / E * sum_e mean_e = tokens * top_k / E,
+    # whatever the scores are (each row of a softmax sums to one) -> loss = loss_weight
+    even = torch.full((ne,), tokens * top_k // ne, dtype=torch.int32)
+    assert abs(float(oracle.load_balancing_loss(even, scores, num_experts=ne, top_k=top_k, loss_weight=w)) - w) < 1e-6
+    # everything routed to one expert whose score is 1 for every token -> loss = E * loss_weight
+    onehot = torch.zeros(tokens, ne)
+    onehot[:, 3] = 1
+    counts = torch.zeros(ne, dtype=torch.int32)
+    counts[3] = tokens * top_k
+    assert abs(float(oracle.load_balancing_loss(counts, onehot, num_experts=ne, top_k=top_k, loss_weight=w)) - ne * w) < 1e-5
+    # two layers with num_layers = 2: the mean of the two single-layer losses
+    s2 = torch.randn(tokens, ne, generator=g).softmax(-1)
+    c1 = oracle.histogram(torch.topk(scores, top_k, -1).indices.flatten().int(), ne)
+    c2 = oracle.histogram(torch.topk(s2, top_k, -1).indices.flatten().int(), ne)
+    both = oracle.load_balancing_loss([c1, c2], [scores, s2], num_experts=ne, top_k=top_k, loss_weight=w)
+    a = oracle.load_balancing_loss(c1, scores, num_experts=ne, top_k=top_k, loss_weight=w)
+    b = oracle.load_balancing_loss(c2, s2, num_experts=ne, top_k=top_k, loss_weight=w)
+    assert abs(float(both) - 0.5 * (float(a) + float(b))) < 1e-6
+    assert oracle.load_balancing_loss(c1, scores, num_experts=ne, top_k=top_k, loss_weight=0) == 0.0
+    with pytest.raises(ValueError):
+        oracle.load_balancing_loss([c1], [scores], num_experts=ne, top_k=top_k, loss_weight=w, num_layers=2)
+    # the gradient reaches the scores only: d loss / d scores[t, e] = scale * counts[e] / tokens
+    s = scores.clone().requires_grad_(True)
+    oracle.load_balancing_loss(c1, s, num_experts=ne, top_k=top_k, loss_weight=w).backward()
+    want = (ne * w / (tokens * top_k)) * c1.float() / tokens
+    assert torch.allclose(s.grad, want.expand(tokens, ne), rtol=1e-6, atol=0)
+
+
+def test_router_zloss_loop_and_closed_form():
+    import math
+    tokens, ne, w = 9, 5, 1e-3
+    g = torch.Generator().manual_seed(2)
+    logits = torch.randn(tokens, ne, generator=g) * 3
+    want = w * sum(math.log(sum(math.exp(v) for v in row)) ** 2 for row in logits.tolist()) / tokens
+    got = oracle.router_zloss(logits, zloss_weight=w)
+    assert got.shape == (1,) and abs(float(got[0]) - want) <= 1e-6 * want
+    # constant logits c over E experts: logsumexp = c + ln E
+    for c in (-2.0, 0.0, 3.5):
+        z = oracle.router_zloss(torch.full((4, ne), c), zloss_weight=w)
+        want_c = w * (c + math.log(ne)) ** 2
+        assert abs(float(z[0]) - want_c) <= 1e-6 * want_c
+    # one value per router; large logits do not overflow
+    z = oracle.router_zloss([logits, logits + 100.0], zloss_weight=w)
+    assert z.shape == (2,) and torch.isfinite(z).all() and abs(float(z[0]) - want) <= 1e-6 * want
+    assert oracle.router_zloss(logits, zloss_weight=0) == 0
+    # 16-bit logits are widened first (router.py:36-37)
+    zb = oracle.router_zloss(logits.bfloat16(), zloss_weight=w)
+    assert zb.dtype == torch.float32
+
+
+def test_uniform_expert_assignment():
+    got = oracle.uniform_expert_assignment((5, 2), 4)
+    assert got.tolist() == [[0, 1], [2, 3], [0, 1], [2, 3], [0, 1]]
+    assert oracle.histogram(oracle.uniform_expert_assignment((64, 2), 8).flatten().int(), 8).tolist() == [16] * 8
