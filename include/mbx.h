@@ -112,6 +112,21 @@ int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
                 void* out, const int32_t* slot_rows, void* scratch, size_t scratch_bytes,
                 mbx_stream_t stream);
 
+/* mbx_scatter for callers that cannot allocate device memory and have no buffer to lend: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * scatter allocates its [tokens, top_k, hidden] temporary through torch).  Same arguments and results as
+ * mbx_scatter with slot_rows = NULL, except that the slot -> row map is built in a buffer that is part of the
+ * library image (MBX_STATIC_SCATTER_MAX_SLOTS int32 entries = 4 MiB on every GPU the library runs on, held until the
+ * process ends) instead of in caller-provided scratch.  It calls no allocator.  tokens * top_k above
+ * MBX_STATIC_SCATTER_MAX_SLOTS returns MBX_ERANGE.  All calls on one GPU share that one buffer: calls that may
+ * overlap on a GPU (different streams, different threads) race and must be ordered by the caller.  The buffer's
+ * address is looked up on the first call on each device; make that call outside stream capture. */
+#define MBX_STATIC_SCATTER_MAX_SLOTS (1 << 20)
+int mbx_scatter_static(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
+                       const int32_t* indices, const int32_t* bin_ids, const int32_t* bins,
+                       const int32_t* padded_bins, int num_bins, const void* weights, int w_dtype,
+                       void* out, mbx_stream_t stream);
+
 /* megablocks/backend/kernels.py:217-307 `scatter_wgrad` / `padded_scatter_wgrad`:
  * wgrad[indices[i]] = <x[row(i)], grad[indices[i] / top_k]> (fp32 accumulate, stored
  * in the type of x). */

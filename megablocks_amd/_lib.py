@@ -34,6 +34,7 @@ _SIGNATURES = {
     'mbx_gather': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _vp, _vp]),
     'mbx_slot_rows': (_i, [_vp, _vp, _vp, _vp, _i, _i64, _vp, _vp]),
     'mbx_scatter': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _sz, _vp]),
+    'mbx_scatter_static': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp]),
     'mbx_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     'mbx_scatter_backward': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i64, _vp, _vp]),
     'mbx_binned_gather': (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _vp]),

@@ -4,6 +4,8 @@
 // multiple of 16 bytes and the buffers are 16-byte aligned.
 #include "common.h"
 
+#include <mutex>
+
 namespace mbx {
 namespace {
 
@@ -603,6 +605,30 @@ int mbx_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k, 
   return launch_status();
 }
 
+// The slot -> row map of mbx_scatter_static: device memory that is part of the loaded code object, so that the
+// entry point never allocates.  Every GPU the library runs on holds its own copy (4 MiB) at its own address until
+// the process ends; in host code the array's name is only a handle for hipGetSymbolAddress.
+static __device__ __align__(256) int32_t g_static_slot_rows[MBX_STATIC_SCATTER_MAX_SLOTS];
+
+// Device address of g_static_slot_rows on the current device, looked up once per device.
+static int static_slot_rows(int32_t** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static int32_t* address[kMaxDevices];
+  int dev = 0;
+  MBX_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return MBX_EINVAL;
+  std::lock_guard<std::mutex> guard(lock);
+  if (!address[dev]) {
+    void* p = nullptr;
+    MBX_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_slot_rows)));
+    if (!p) return MBX_EINVAL;
+    address[dev] = (int32_t*)p;
+  }
+  *out = address[dev];
+  return 0;
+}
+
 static void build_slot_rows(const int32_t* indices, const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins,
                             int num_bins, int64_t n_slots, int32_t* inv, hipStream_t s) {
   const unsigned fb = (unsigned)(ceil_div(n_slots, 256) < 2048 ? ceil_div(n_slots, 256) : 2048);
@@ -617,6 +643,21 @@ int mbx_slot_rows(const int32_t* indices, const int32_t* bin_ids, const int32_t*
   if (!indices || !slot_rows || (padded_bins && !bins)) return MBX_EINVAL;
   if (n_slots > 0x7fffffff) return MBX_ERANGE;
   build_slot_rows(indices, bin_ids, bins, padded_bins, num_bins, n_slots, slot_rows, as_stream(stream));
+  return launch_status();
+}
+
+// The combine launch of mbx_scatter / mbx_scatter_static: `inv` is the slot -> row map.
+static int launch_combine(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* inv,
+                          const void* weights, int w_dtype, void* out, hipStream_t s) {
+  const bool vec = can_vec(dtype, hidden, x, out);
+#define CALL(DT, V)                                                                                                             \
+  do {                                                                                                                          \
+    if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
+    else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
+    else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
+  } while (0)
+  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
+#undef CALL
   return launch_status();
 }
 
@@ -637,16 +678,25 @@ int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
     build_slot_rows(indices, bin_ids, bins, padded_bins, num_bins, n_slots, (int32_t*)scratch, s);
     inv = (const int32_t*)scratch;
   }
-  const bool vec = can_vec(dtype, hidden, x, out);
-#define CALL(DT, V)                                                                                                             \
-  do {                                                                                                                          \
-    if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
-    else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
-    else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
-  } while (0)
-  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
-#undef CALL
-  return launch_status();
+  return launch_combine(x, dtype, tokens, hidden, top_k, inv, weights, w_dtype, out, s);
+}
+
+int mbx_scatter_static(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
+                       const int32_t* bin_ids, const int32_t* bins, const int32_t* padded_bins, int num_bins,
+                       const void* weights, int w_dtype, void* out, mbx_stream_t stream) {
+  if (tokens < 0 || hidden < 0 || top_k <= 0 || num_bins < 0 || bad_dtype(dtype)) return MBX_EINVAL;
+  if (weights && bad_dtype(w_dtype)) return MBX_EINVAL;
+  if (tokens == 0 || hidden == 0) return 0;
+  if (!x || !out || !indices || (padded_bins && !bins)) return MBX_EINVAL;
+  const int64_t n_slots = tokens * top_k;
+  if (n_slots > MBX_STATIC_SCATTER_MAX_SLOTS) return MBX_ERANGE;   // more slots than the static map holds
+  int32_t* map = nullptr;
+  const int rc = static_slot_rows(&map);
+  if (rc) return rc;
+  hipStream_t s = as_stream(stream);
+  // every entry the combine reads is rewritten here (fill, then the inverse map): nothing of the previous call is used
+  build_slot_rows(indices, bin_ids, bins, padded_bins, num_bins, n_slots, map, s);
+  return launch_combine(x, dtype, tokens, hidden, top_k, map, weights, w_dtype, out, s);
 }
 
 int mbx_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int hidden, int top_k,
