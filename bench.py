@@ -22,13 +22,22 @@ if ROOT not in sys.path:
 
 MFMA_PEAK = {'bf16': 2.5e15, 'f16': 2.5e15, 'f32': 157.3e12}
 HBM_PEAK = 8e12
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
-# keyed by (workload, kernel); None until measured for the workload at hand.
-MEASURED_TRAFFIC = {
-    # workload c3, rocprofv3 FETCH_SIZE (x2.00, the factor a plain 1 GiB copy shows) + WRITE_SIZE, bytes per launch;
-    # see profiles/gmm_dmoe_c3_mixtral_hbm_traffic.txt
-    ('c3', 'gmm_nn'): 4.94e9, ('c3', 'gmm_nt'): 6.41e9, ('c3', 'gmm_tn'): 4.90e9, ('c3', 'gmm_nn_dual'): 9.90e9,
-}
+# HBM bytes per launch of the grouped-GEMM kernels as rocprofv3 counted them (FETCH_SIZE scaled by what a plain copy of
+# known size shows, plus WRITE_SIZE): read from the machine-readable companion of the counter summaries under
+# profiles/, so the figure printed is the one of the committed profile and names it.
+TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+
+
+def measured_traffic(workload, kernel):
+    """(bytes per launch or None, where it comes from / why there is none)."""
+    try:
+        table = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError) as exc:
+        return None, f'{os.path.relpath(TRAFFIC_FILE, ROOT)} unreadable: {exc}'
+    entry = table.get('workloads', {}).get(workload, {}).get(kernel)
+    if entry is None:
+        return None, f'no counter run of {kernel} on {workload} in {os.path.relpath(TRAFFIC_FILE, ROOT)}'
+    return entry['bytes_per_launch'], entry.get('source')
 
 
 def parse():
@@ -48,6 +57,9 @@ def parse():
     ap.add_argument('--operand-patterns', action='store_true',
                     help='also time the grouped GEMM launches on all-zero and all-one operands (same shapes): what the '
                          'same instruction stream gives when the operands cost no switching power')
+    ap.add_argument('--mfma-ceiling', action='store_true',
+                    help='also run a loop of matrix-core instructions alone (no LDS, no memory) on all-zero, all-one and '
+                         'N(0,1) bf16 operands: the rate and shader clock the power limit allows on such values')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also launch one plain 1 GiB device copy (a known-size reference for HBM byte counters)')
     return ap.parse_args()
@@ -307,6 +319,62 @@ def operand_pattern_leg(w, inp):
     return res
 
 
+def mfma_ceiling_leg():
+    """A loop of matrix-core instructions alone (libmbx_probe.so: operands and accumulators stay in registers; no LDS
+    reads, no memory traffic), about a second per case, on operands that are all zero, all one, and N(0,1) bf16
+    values, for the 32x32x16 instruction the grouped GEMM uses and for 16x16x32.  The shader clock is measured inside
+    the kernel (cycle counter against the 100 MHz wall clock).  On values that switch few bits the loop runs at the
+    nominal peak; on random values the power limit lowers the clock, and what is left is the most any bf16 kernel
+    can show on such data."""
+    import ctypes
+
+    import torch
+
+    lib = ctypes.CDLL(os.path.join(ROOT, 'megablocks_amd', 'libmbx_probe.so'))
+    lib.mbx_probe_mfma.restype = ctypes.c_int
+    lib.mbx_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                   ctypes.c_void_p, ctypes.c_void_p]
+    dev = torch.device('cuda', 0)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    blocks = cus                                   # one workgroup of four waves per compute unit: one wave per SIMD
+    n_vec = 1 << 16
+    sink = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    res = {'what': 'MFMA-only loop, one wave per SIMD on every compute unit, operands in registers', 'blocks': blocks, 'cases': {}}
+    for kind, kname in ((0, 'mfma_32x32x16_bf16'), (1, 'mfma_16x16x32_bf16')):
+        for pattern in ('zeros', 'ones', 'normal'):
+            if pattern == 'zeros':
+                ops = torch.zeros(n_vec * 8, dtype=torch.bfloat16, device=dev)
+            elif pattern == 'ones':
+                ops = torch.ones(n_vec * 8, dtype=torch.bfloat16, device=dev)
+            else:
+                ops = torch.randn(n_vec * 8, device=dev, generator=torch.Generator(device=dev).manual_seed(0)).to(torch.bfloat16)
+
+            def launch(iters):
+                rc = lib.mbx_probe_mfma(ops.data_ptr(), n_vec, kind, blocks, iters, sink.data_ptr(), clocks.data_ptr(), stream)
+                if rc:
+                    raise RuntimeError(f'mbx_probe_mfma failed: {rc}')
+            launch(2000)
+            torch.cuda.synchronize()
+            iters = 400000                          # 16 MFMAs of 32 (or 64 of 8) cycles per iteration: about 0.1 s per launch
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            launches = 10
+            e0.record()
+            for _ in range(launches):
+                launch(iters)
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / launches
+            flops = blocks * 4.0 * iters * 16 * 32768
+            cyc, wall = clocks.tolist()
+            res['cases'][f'{kname}/{pattern}'] = dict(
+                ms_per_launch=round(ms, 3), tflops=round(flops / (ms * 1e-3) / 1e12, 1),
+                frac_of_mfma_peak=round(flops / (ms * 1e-3) / MFMA_PEAK['bf16'], 4),
+                shader_clock_mhz=round(cyc / wall * 100.0) if wall else None)
+    return res
+
+
 def cpu_leg(args, w, inp_full):
     """The CPU formulation (oracle) of the same layer, fp32, forward+backward, on a bounded sample."""
     import torch
@@ -316,12 +384,12 @@ def cpu_leg(args, w, inp_full):
 
     cores = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    # aim at roughly 10-30 s of CPU work: scale the token count to about 2e12 FLOP per step
+    # The whole workload where a step is a few seconds of CPU work, else half of its tokens (all experts and their
+    # full weights either way: the work per token is unchanged); --cpu-tokens overrides.
     if args.cpu_tokens:
         T = args.cpu_tokens
     else:
-        per_token = w.gemm_flops() / w.tokens
-        T = int(min(w.tokens, max(256, 2.0e12 // per_token)))
+        T = w.tokens if w.gemm_flops() <= 4e12 else w.tokens // 2
     inp = inp_full if T == w.tokens else synthetic.make_inputs(w, tokens=T, seed=0)
     act = w.activation()
 
@@ -342,13 +410,13 @@ def cpu_leg(args, w, inp_full):
 
     step()  # warm-up
     times = []
-    for _ in range(2):
+    for _ in range(3):
         t0 = time.perf_counter()
         step()
         times.append(time.perf_counter() - t0)
     t = statistics.median(times)
     return dict(value=round(T / t, 1), unit='tokens/s', cores=cores, kind='port',
-                sample=f'{T} of {w.tokens} tokens of workload {w.name}, fp32, fwd+bwd, 1 warm-up + 2 timed steps '
+                sample=f'{T} of {w.tokens} tokens of workload {w.name}, fp32, fwd+bwd, 1 warm-up + 3 timed steps '
                        f'(median {t:.2f} s), torch {torch.get_num_threads()} threads',
                 seconds_per_step=round(t, 3))
 
@@ -383,13 +451,15 @@ def main():
     dom_name, dom = max(gemm.items(), key=lambda kv: kv[1]['avg_ms'] * kv[1]['launches'])
     # The kernel is bound by whichever roofline its arithmetic intensity puts lower (the ridge of the part is
     # MFMA peak / HBM peak = 312 FLOP per byte in bf16): c2's 256-row experts stream their weights.
+    traffic, traffic_source = measured_traffic(w.name if not args.tokens else None, dom_name)
     if dom['flops_per_launch'] / dom['bytes_per_launch'] >= MFMA_PEAK[dn] / HBM_PEAK:
         roofline = dict(bound='mfma', kernel=dom_name, achieved=dom['tflops'], peak=MFMA_PEAK[dn] / 1e12, unit='TFLOP/s',
-                        frac=dom['frac_of_mfma_peak'], traffic=MEASURED_TRAFFIC.get((w.name, dom_name)),
+                        frac=dom['frac_of_mfma_peak'], traffic=traffic, traffic_source=traffic_source,
+                        algorithmic_bytes_per_launch=dom['bytes_per_launch'],
                         flops_per_launch=dom['flops_per_launch'], avg_launch_ms=dom['avg_ms'])
     else:
         roofline = dict(bound='hbm', kernel=dom_name, achieved=dom['gbps'], peak=HBM_PEAK / 1e9, unit='GB/s',
-                        frac=dom['frac_of_hbm_peak'], traffic=MEASURED_TRAFFIC.get((w.name, dom_name)),
+                        frac=dom['frac_of_hbm_peak'], traffic=traffic, traffic_source=traffic_source,
                         bytes_per_launch=dom['bytes_per_launch'], avg_launch_ms=dom['avg_ms'])
     all_gemm_tflops = w.gemm_flops() / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None
 
@@ -419,6 +489,8 @@ def main():
         out['library_gemm'] = library_gemm_leg(w, inp)
     if args.operand_patterns:
         out['operand_patterns'] = operand_pattern_leg(w, inp)
+    if args.mfma_ceiling:
+        out['mfma_ceiling'] = mfma_ceiling_leg()
     if not args.no_cpu:
         del layer
         torch.cuda.empty_cache()

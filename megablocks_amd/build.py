@@ -1,4 +1,5 @@
-"""Builds libmbx.so (the HIP kernels + C ABI) in-tree for gfx950 with hipcc.
+"""Builds libmbx.so (the HIP kernels + C ABI) and libmbx_probe.so (measurement aids for bench.py) in-tree for
+gfx950 with hipcc.
 
     python megablocks_amd/build.py            # compile what is out of date
     python megablocks_amd/build.py --force    # recompile everything
@@ -14,9 +15,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
 BUILD = os.path.join(HERE, 'build')
 LIB = os.path.join(HERE, 'libmbx.so')
+PROBE_LIB = os.path.join(HERE, 'libmbx_probe.so')
+PROBE_SOURCE = 'probe.hip'
 SOURCES = ['routing.hip', 'permute.hip', 'gmm.hip', 'elementwise.hip', 'router.hip']
 HEADERS = [os.path.join(CSRC, 'common.h'), os.path.join(CSRC, 'gmm_dma.h'),
-           os.path.join(os.path.dirname(HERE), 'include', 'mbx.h')]
+           os.path.join(os.path.dirname(HERE), 'include', 'mbx.h'), os.path.join(os.path.dirname(HERE), 'include', 'mbx_probe.h')]
 ARCH = 'gfx950'
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from scalar float code.
 FLAGS = ['-O3', '-fPIC', '-std=c++17', f'--offload-arch={ARCH}', '-Xclang', '-target-feature', '-Xclang',
@@ -54,11 +57,18 @@ def build(force: bool = False, verbose: bool = False) -> str:
             if verbose:
                 print(' '.join(cmd), flush=True)
             procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    probe_src = os.path.join(CSRC, PROBE_SOURCE)
+    probe_cmd = None
+    if force or not os.path.exists(PROBE_LIB) or os.path.getmtime(PROBE_LIB) < max(os.path.getmtime(probe_src), newest_header):
+        probe_cmd = [hipcc] + FLAGS + ['-shared', probe_src, '-o', PROBE_LIB]
+        if verbose:
+            print(' '.join(probe_cmd), flush=True)
+        procs.append((probe_cmd, subprocess.Popen(probe_cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     for cmd, p in procs:
         out, _ = p.communicate()
         if p.returncode != 0:
             raise RuntimeError(f'command failed: {" ".join(cmd)}\n{out}')
-    if procs or force or not os.path.exists(LIB):
+    if [c for c, _ in procs if c is not probe_cmd] or force or not os.path.exists(LIB):
         _run([hipcc, '-shared', '-fPIC', f'--offload-arch={ARCH}', '-o', LIB] + objs)
     return LIB
 
