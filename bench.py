@@ -357,7 +357,7 @@ def mfma_ceiling_leg():
                     raise RuntimeError(f'mbx_probe_mfma failed: {rc}')
             launch(2000)
             torch.cuda.synchronize()
-            iters = 400000                          # 16 MFMAs of 32 (or 64 of 8) cycles per iteration: about 0.1 s per launch
+            iters = 400000 if kind == 0 else 200000  # 512 (or 1024) matrix-core cycles per iteration: about 0.1 s per launch
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             launches = 10
             e0.record()
@@ -366,7 +366,7 @@ def mfma_ceiling_leg():
             e1.record()
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1) / launches
-            flops = blocks * 4.0 * iters * 16 * 32768
+            flops = blocks * 4.0 * iters * (16 * 32768 if kind == 0 else 64 * 16384)   # 16 MFMAs of 32x32x16 or 64 of 16x16x32 per iteration
             cyc, wall = clocks.tolist()
             res['cases'][f'{kname}/{pattern}'] = dict(
                 ms_per_launch=round(ms, 3), tflops=round(flops / (ms * 1e-3) / 1e12, 1),

@@ -14,6 +14,8 @@
 // experts cost nothing (NN/NT) or produce an all-zero block (TN).
 #include "common.h"
 
+#include <cstdlib>
+
 namespace mbx {
 namespace {
 
@@ -30,6 +32,16 @@ __device__ __forceinline__ f32x16 mfma32(const u32x4& a, const u32x4& b, const f
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
   else
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ f32x4 mfma16(const u32x4& a, const u32x4& b, const f32x4& c) {
+  if (DT == MBX_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
 }
 
 // One operand of the product as seen by a workgroup.
@@ -481,6 +493,26 @@ typedef dma::Tile<256, 256, 2, 2, 64, 2> TileDma;
 // an expert when it is at most half full, for the tail of a launch, and for launches of small experts;
 // its smaller stages allow a three-deep ring.
 typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;   // 4 x 16 KiB + 3 x 32 KiB
+// the same two tiles on the 16 x 16 x 32 instruction
+typedef dma::Tile<256, 256, 2, 2, 64, 2, 16> TileDma16;
+typedef dma::Tile<128, 256, 1, 4, 64, 3, 16> TileDmaSmallM16;
+
+// Which instruction the direct-to-LDS kernels multiply with.  32 x 32 x 16 unless MBX_MFMA=16 is set in the
+// environment (read once).  On operands with random mantissas the power limit lets a loop of 16 x 16 x 32 MFMAs alone
+// run at 2.0 PFLOP/s where 32 x 32 x 16 reaches 1.76 (it moves half the accumulator registers per FLOP), and the
+// 16 x 16 x 32 kernels do hold a shader clock of 1.9 - 2.0 GHz on such operands where the others drop to 1.55 - 1.65.
+// But a wave alone on its SIMD issues one independent instruction every four cycles (eight when it depends on the
+// one before, and more where vector-ALU, LDS and scalar instructions alternate), an MFMA takes two of those slots,
+// and a 16-cycle MFMA leaves room for two more where a 32-cycle one leaves six: with 128 instead of 64 MFMAs per K
+// tile the loads, LDS reads and address arithmetic of a K tile no longer fit behind them, and the higher clock only
+// just makes up for the idle matrix-core cycles (c3 in the layer: NT +0.7 %, NN -1.4 %, TN -4 %).
+static inline bool use_mfma16() {
+  static const bool choice = [] {
+    const char* v = getenv("MBX_MFMA");
+    return v && v[0] == '1' && v[1] == '6';
+  }();
+  return choice;
+}
 
 template <int DT, bool A_MC, bool B_MC, typename T>
 constexpr size_t lds_bytes() {
@@ -670,6 +702,14 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     if (dma_ok) {
       // TN: the half-height tile only when the product has at most 128 rows (it is slower otherwise)
       const bool small_m = layout == MBX_TN ? k <= TileDmaSmallM::BM : half_height_only(rows, num_groups, n);
+      if (use_mfma16()) {
+        if (small_m) {
+          if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+          return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+        }
+        if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+        return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+      }
       if (small_m) {
         if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
         return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
@@ -701,6 +741,14 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   const bool small_m = half_height_only(rows, num_groups, n);
+  if (use_mfma16()) {
+    if (small_m) {
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+    }
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+  }
   if (small_m) {
     if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
     return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);

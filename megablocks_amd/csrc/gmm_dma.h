@@ -35,13 +35,19 @@ namespace dma {
 // B load can be (the B stage to refill is still being read), so that global -> LDS loads leave the
 // compute unit at an even rate: the texture-address unit takes some 20 cycles per wave-wide load, is
 // shared by the four waves, and a wave whose load has to queue cannot issue its next MFMA either.
-template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_>
+// MF_: rows / columns of the matrix-core instruction: 32 (v_mfma_f32_32x32x16, 16 accumulator registers per product
+// tile, reduction length 16) or 16 (v_mfma_f32_16x16x32: 4 registers, reduction length 32).  Same peak rate, same LDS
+// bytes per FLOP for a given wave tile; the 16 x 16 x 32 form moves half the accumulator registers per FLOP.
+template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_, int MF_ = 32>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1;
-  static constexpr int KS = BK / 16;                                           // MFMA k-steps per tile
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1, MF = MF_;
+  static constexpr int KSTEP = MF == 32 ? 16 : 32;                             // reduction length of one MFMA
+  static constexpr int KS = BK / KSTEP;                                        // MFMA k-steps per tile
   static constexpr int WAVES = WM * WN, THREADS = WAVES * kWave;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
-  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int TM = WTM / MF, TN = WTN / MF;
+  typedef typename std::conditional<MF == 32, f32x16, f32x4>::type Acc;        // one product tile of a lane
+  static_assert(MF == 32 || MF == 16, "matrix-core instruction shape");
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int A_INSTRS = A_BYTES / 1024, B_INSTRS = B_BYTES / 1024;  // wave-wide 1 KiB loads per tile
   static constexpr int LA = A_INSTRS / WAVES, LB = B_INSTRS / WAVES;          // ... per wave
@@ -91,29 +97,46 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
 // Per-lane byte offset (inside an operand tile) of the MFMA operand of the 32 rows/cols starting
 // at `r`, k-step 0.  KC: k-step s is the same address with bits 5.. XORed by 32 s.  MC: 16 rows (of
 // COLS columns) further per k-step.
-template <bool MC, int BK, int COLS>
+// MF = 16 (16 x 16 x 32 instruction): lane l holds row / column l % 16 and the eight k values 8 (l / 16) ..; k-step s is
+// 32 k further (KC: bits 6.. XORed by 64 s; MC: 32 rows).  The MC layout for this shape swizzles the pair index by
+// 2 (k & 3) ^ ((k >> 3) & 1): the two 16-lane groups a transposing read serves per cycle hold k rows 8 apart.
+template <bool MC, int BK, int COLS, int MF = 32>
 __device__ __forceinline__ uint32_t frag_lane_offset(int r) {
   const int lane = lane_id();
   if (!MC) {
-    const int row = lane & 31;
-    const int swz = BK == 64 ? (row >> 1) & 7 : (row >> 2) & 3;
-    return (uint32_t)((r + row) * (BK * 2) + (((lane >> 5) ^ swz) << 4));
+    if (MF == 32) {
+      const int row = lane & 31;
+      const int swz = BK == 64 ? (row >> 1) & 7 : (row >> 2) & 3;
+      return (uint32_t)((r + row) * (BK * 2) + (((lane >> 5) ^ swz) << 4));
+    } else {
+      static_assert(MF == 32 || BK == 64, "16 x 16 x 32 operands are read from 128-byte rows");
+      const int row = lane & 15;
+      const int swz = (row >> 1) & 7;
+      return (uint32_t)((r + row) * (BK * 2) + (((lane >> 4) ^ swz) << 4));
+    }
   } else {
     const int g = lane >> 4, s = lane & 15;
-    const int k = (g >> 1) * 8 + (s >> 2);
-    const int pair = (r >> 4) + (g & 1);
-    return (uint32_t)(k * (COLS * 2) + ((pair ^ (2 * ((s >> 2) & 3))) << 5) + ((s & 3) << 3));
+    if (MF == 32) {
+      const int k = (g >> 1) * 8 + (s >> 2);
+      const int pair = (r >> 4) + (g & 1);
+      return (uint32_t)(k * (COLS * 2) + ((pair ^ (2 * ((s >> 2) & 3))) << 5) + ((s & 3) << 3));
+    } else {
+      const int k = g * 8 + (s >> 2);
+      const int pair = r >> 4;
+      return (uint32_t)(k * (COLS * 2) + ((pair ^ (2 * ((s >> 2) & 3)) ^ (g & 1)) << 5) + ((s & 3) << 3));
+    }
   }
 }
 
 // IMM: constant byte offset of the 32-row tile inside a KC operand tile (goes into the instruction).
-template <bool MC, int KS, int IMM = 0, int COLS = 256>
+template <bool MC, int KS, int IMM = 0, int COLS = 256, int MF = 32>
 __device__ __forceinline__ u32x4 read_frag(uint32_t tile_addr, uint32_t lane_off) {
+  constexpr int KSTEP = MF == 32 ? 16 : 32;
   if (!MC) {
-    return lds_read_b128<IMM>(tile_addr + (lane_off ^ (KS * 32)));
+    return lds_read_b128<IMM>(tile_addr + (lane_off ^ (KS * KSTEP * 2)));
   } else {
-    const u32x2 lo = lds_read_tr16_b64<KS * 16 * COLS * 2>(tile_addr + lane_off);
-    const u32x2 hi = lds_read_tr16_b64<KS * 16 * COLS * 2 + 4 * COLS * 2>(tile_addr + lane_off);
+    const u32x2 lo = lds_read_tr16_b64<KS * KSTEP * COLS * 2>(tile_addr + lane_off);
+    const u32x2 hi = lds_read_tr16_b64<KS * KSTEP * COLS * 2 + 4 * COLS * 2>(tile_addr + lane_off);
     u32x4 v;
     v[0] = lo[0]; v[1] = lo[1]; v[2] = hi[0]; v[3] = hi[1];
     return v;
@@ -123,8 +146,11 @@ __device__ __forceinline__ u32x4 read_frag(uint32_t tile_addr, uint32_t lane_off
 // ---- global -> LDS ----
 // Byte offset (from the operand's buffer base) fetched by this lane in the wave's first load of
 // tile 0; `r0` is the tile origin in the non-reduction dimension, `ld_bytes` the row pitch.
-template <bool MC, int BK, int COLS>
-__device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t ld_bytes) {
+// MF = 16: the MC swizzle has the extra term (k >> 3) & 1 (see frag_lane_offset).  With 256 columns a load holds
+// k = 2 j, 2 j + 1 for load number j = wave + 4 q of the tile, so that term is the parity of q (`odd`); with 128
+// columns (k = 4 j ..) it is (wave >> 1) & 1.
+template <bool MC, int BK, int COLS, int MF = 32>
+__device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t ld_bytes, bool odd = false) {
   const int lane = lane_id();
   if (!MC) {
     if (BK == 64) {  // 8 rows x 8 chunks per instruction; instruction j holds rows 8j .. 8j + 7
@@ -139,22 +165,37 @@ __device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t 
   } else if (COLS == 256) {   // 2 k-rows x 32 chunks per instruction; instruction j holds k = 2j, 2j + 1
     const int kl = lane >> 5, pc = lane & 31;
     const int k3 = (2 * (wave & 1) + kl) & 3;                     // (2j + kl) & 3 with j = wave (mod 2)
-    const int c = ((((pc >> 1) ^ (2 * k3)) << 1) | (pc & 1));
+    const int x = (2 * k3) ^ ((MF == 16 && odd) ? 1 : 0);
+    const int c = ((((pc >> 1) ^ x) << 1) | (pc & 1));
     return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
   } else {                    // 128 columns: 4 k-rows x 16 chunks per instruction; instruction j holds k = 4j .. 4j + 3
     static_assert(!MC || COLS == 256 || COLS == 128, "strided operand tile width");
     const int kl = lane >> 4, pc = lane & 15;
-    const int c = ((((pc >> 1) ^ (2 * kl)) << 1) | (pc & 1));
+    const int x = (2 * kl) ^ (MF == 16 ? (wave >> 1) & 1 : 0);
+    const int c = ((((pc >> 1) ^ x) << 1) | (pc & 1));
     return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
   }
 }
 
 // One wait for all LDS reads in flight, tied to the operand registers of a k-step so that the MFMAs
 // that consume them cannot be scheduled above it.
+template <int N>
+__device__ __forceinline__ void tie_frags(u32x4 (&f)[N]) {   // no instruction: orders later users of f behind the preceding wait
+  static_assert(N == 4 || N == 8, "operand registers per k-step");
+  if constexpr (N == 8) {
+    asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
+  } else {
+    asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
+  }
+}
+
 template <int NA, int NB>
 __device__ __forceinline__ void wait_frags(u32x4 (&a)[NA], u32x4 (&b)[NB]) {
-  static_assert(NA <= 4 && NB <= 4 && NA >= 2 && NB >= 2, "operand registers per k-step");
-  if constexpr (NA == 4 && NB == 4) {
+  static_assert(NA <= 8 && NB <= 8 && NA >= 2 && NB >= 2, "operand registers per k-step");
+  if constexpr (NA == 8) {   // an asm statement takes at most 30 operands, and "+v" counts twice
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+    tie_frags(b);
+  } else if constexpr (NA == 4 && NB == 4) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
   } else if constexpr (NA == 4 && NB == 2) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]));
@@ -180,7 +221,8 @@ struct Args {
 // acc = (clear ? 0 : acc) + A_tile * B_tile over all K tiles.  On return no load is in flight and no LDS
 // read is pending, but other waves may still be reading the last stages.
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
-__device__ __forceinline__ void block_multiply(const Args& g, f32x16 (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
+__device__ __forceinline__ void block_multiply32(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
+  static_assert(T::MF == 32, "the schedule below is written for the 32 x 32 x 16 instruction");
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -391,17 +433,253 @@ __device__ __forceinline__ void block_multiply(const Args& g, f32x16 (&acc)[T::T
 #undef MBX_STEP
 }
 
+// acc += a-fragment x b-fragment with v_mfma_f32_16x16x32, written as inline asm with the accumulator tied to one
+// register tuple ("+a": an AGPR tuple, source and destination): with the builtin, whose destination may differ from
+// its accumulator source, the register allocator gave the 64 four-register tiles of a wave other registers at the
+// bottom of the main loop than at its top and moved all of them back every iteration (some 400 copies).  The
+// compiler does not know that this statement is a matrix-core instruction, so the wait states the instruction set
+// asks for around reads and writes of the accumulators by other instructions are put in by hand (mfma16_settle).
+template <int DT>
+__device__ __forceinline__ void mfma16_acc(f32x4& acc, const u32x4& a, const u32x4& b) {
+  if (DT == MBX_BF16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+// more wait states than any hazard between a vector-ALU access and a matrix-core access of the same register needs
+__device__ __forceinline__ void mfma16_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+
+// The same product with v_mfma_f32_16x16x32: two k-steps of 32 per K tile, TM x TN = 8 x 8 product tiles of 16 x 16
+// per wave (the same 128 x 128 wave tile and 256 accumulator registers; 8 + 8 operand fragments per k-step, double
+// buffered: 128 registers).  Iteration kt multiplies K tile kt and issues
+//   k-step 0: the second half of B tile kt + SB - 1 -> B stage (kt - 1) % SB, the first half of A tile kt + SB -> A stage (kt - 1) % SA
+//   barrier: every wave has both k-steps of tile kt in registers and tile kt + 1 has landed
+//   k-step 1: the second half of that A tile, the first half of B tile kt + SB -> B stage kt % SB (free since the barrier)
+// i.e. the loads in the order of the 32 x 32 x 16 schedule, one wave-wide load per eight MFMAs.
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
+__device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
+  static_assert(T::MF == 16 && T::KS == 2, "two k-steps of 32 per K tile");
+  const lds_ptr lds = (lds_ptr)lds_generic;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
+
+  constexpr int BK = T::BK, SA = T::SA, SB = T::SB, LA = T::LA, LB = T::LB;
+  constexpr uint32_t B_RING = (uint32_t)SA * T::A_BYTES;
+  // a 256-column MC operand takes its lane offsets from the parity of the load's index inside the tile
+  constexpr bool A_QDEP = A_MC && T::BM == 256, B_QDEP = B_MC && T::BN == 256;
+  static_assert((LA / 2) % 2 == 0 && (LB / 2) % 2 == 0, "every group of loads starts at an even load index");
+  const uint32_t a_lane = load_lane_offset<A_MC, BK, T::BM, 16>(wave, g.a_r0, g.a_ld_bytes, false);
+  const uint32_t b_lane = load_lane_offset<B_MC, BK, T::BN, 16>(wave, g.b_r0, g.b_ld_bytes, false);
+  const uint32_t a_lane1 = A_QDEP ? load_lane_offset<A_MC, BK, T::BM, 16>(wave, g.a_r0, g.a_ld_bytes, true) : a_lane;
+  const uint32_t b_lane1 = B_QDEP ? load_lane_offset<B_MC, BK, T::BN, 16>(wave, g.b_r0, g.b_ld_bytes, true) : b_lane;
+  const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
+  const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
+  constexpr uint32_t A_ROWS = (uint32_t)(1024 / ((A_MC ? T::BM : BK) * 2)), B_ROWS = (uint32_t)(1024 / ((B_MC ? T::BN : BK) * 2));
+  const uint32_t a_jstep = A_ROWS * g.a_ld_bytes, b_jstep = B_ROWS * g.b_ld_bytes;
+  auto scalar_off = [&](bool is_b, int kt, int q) -> uint32_t {
+    const uint32_t j = (uint32_t)(wave + q * T::WAVES);
+    const uint32_t v = is_b ? (uint32_t)kt * b_step + j * b_jstep : (uint32_t)kt * a_step + j * a_jstep;
+    return v | (kt < g.nk ? 0u : 0x80000000u);
+  };
+  __amdgpu_buffer_rsrc_t ra = g.rsrc_a, rb = g.rsrc_b;
+  auto lds_off = [&](bool is_b, int stage, int q) -> uint32_t {
+    return (is_b ? B_RING + (uint32_t)stage * T::B_BYTES : (uint32_t)stage * T::A_BYTES) + (uint32_t)(wave + q * T::WAVES) * 1024u;
+  };
+  auto issue = [&](bool is_b, uint32_t sc, uint32_t dst, bool odd) {
+    if (is_b) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? b_lane1 : b_lane) + sc), 0, 0, 0);
+    } else {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? a_lane1 : a_lane) + sc), 0, 0, 0);
+    }
+  };
+  auto issue_group = [&](bool is_b, int kt, int stage, int q0, int count) {   // prologue
+    uint32_t sc = scalar_off(is_b, kt, q0), dst = lds_off(is_b, stage, q0);
+#pragma unroll
+    for (int i = 0; i < count; ++i) {
+      issue(is_b, sc, dst, ((q0 + i) & 1) != 0);
+      sc += T::WAVES * (is_b ? b_jstep : a_jstep);
+      dst += T::WAVES * 1024u;
+    }
+  };
+
+  constexpr int KC_TILE = 16 * BK * 2;   // bytes of a 16-row fragment of a KC operand tile
+  uint32_t fa_off[A_MC ? T::TM : 1], fb_off[B_MC ? T::TN : 1];
+  if (A_MC) {
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true, BK, T::BM, 16>(wm + i * 16);
+  } else {
+    fa_off[0] = frag_lane_offset<false, BK, T::BM, 16>(wm);
+  }
+  if (B_MC) {
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) fb_off[j] = frag_lane_offset<true, BK, T::BN, 16>(wn + j * 16);
+  } else {
+    fb_off[0] = frag_lane_offset<false, BK, T::BN, 16>(wn);
+  }
+
+  u32x4 fa[2][T::TM], fb[2][T::TN];
+  constexpr int NF = T::TM + T::TN, NP = T::TM * T::TN;
+#define MBX_READ_ONE16(KSTEP, BUF, A_ADDR, B_ADDR, M)                                                            \
+  do {                                                                                                           \
+    if constexpr ((M) < T::TM) {                                                                                 \
+      constexpr int i_ = (M);                                                                                    \
+      if constexpr (A_MC) fa[BUF][i_] = read_frag<true, KSTEP, 0, T::BM, 16>(A_ADDR, fa_off[A_MC ? i_ : 0]);     \
+      else fa[BUF][i_] = read_frag<false, KSTEP, i_ * KC_TILE, 256, 16>(A_ADDR, fa_off[0]);                      \
+    } else if constexpr ((M) < NF) {                                                                             \
+      constexpr int j_ = (M) - T::TM;                                                                            \
+      if constexpr (B_MC) fb[BUF][j_] = read_frag<true, KSTEP, 0, T::BN, 16>(B_ADDR, fb_off[B_MC ? j_ : 0]);     \
+      else fb[BUF][j_] = read_frag<false, KSTEP, j_ * KC_TILE, 256, 16>(B_ADDR, fb_off[0]);                      \
+    }                                                                                                            \
+  } while (0)
+  // One k-step: NP MFMAs of 16 cycles on register buffer CUR_BUF.  A wave issues about one instruction every four
+  // cycles, so the gap behind an MFMA has room for three more before the matrix core runs dry; everything else
+  // a k-step has to do is dealt out over the gaps accordingly:
+  //   gaps 0 .. NF - 1: the operand reads of the next k-step into the other buffer, one fragment per gap;
+  //   from gap NF on, every LEVERY-th gap: one global -> LDS load (N1 of operand G1_B at (G1_SC, G1_DST), then N2 of
+  //   operand G2_B), with the update of its running offsets in the gap behind it;
+  //   the scalar bookkeeping P0 .. P4 (at most three instructions each) in the gaps between the first loads.
+#define MBX_STEP16(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, G1_B, G1_SC, G1_DST, N1, G2_B, G2_SC, G2_DST, N2, P0, P1, P2, P3, P4)  \
+  do {                                                                                                           \
+    constexpr int nl_ = (N1) + (N2), load0_ = NF, every_ = (NP - load0_) / nl_;                                  \
+    static_assert(every_ >= 3, "not enough MFMAs per k-step to deal the loads and the bookkeeping over");        \
+    wait_frags(fa[CUR_BUF], fb[CUR_BUF]);                                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                           \
+    static_for<NP>([&](auto mi_) {                                                                               \
+      constexpr int m_ = decltype(mi_)::value;                                                                   \
+      constexpr int i_ = m_ / T::TN, j_ = (i_ & 1) ? T::TN - 1 - m_ % T::TN : m_ % T::TN;                        \
+      mfma16_acc<DT>(acc[i_][j_], fb[CUR_BUF][j_], fa[CUR_BUF][i_]);                                             \
+      MBX_READ_ONE16(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                             \
+      if constexpr (m_ >= load0_ && (m_ - load0_) % every_ == 0 && (m_ - load0_) / every_ < nl_) {               \
+        constexpr int l_ = (m_ - load0_) / every_;                                                               \
+        if constexpr (l_ < (N1)) issue(G1_B, G1_SC, G1_DST, (l_ & 1) != 0);                                      \
+        else issue(G2_B, G2_SC, G2_DST, ((l_ - (N1)) & 1) != 0);                                                 \
+      }                                                                                                          \
+      if constexpr (m_ > load0_ && (m_ - load0_ - 1) % every_ == 0 && (m_ - load0_ - 1) / every_ < nl_) {        \
+        constexpr int l_ = (m_ - load0_ - 1) / every_;                                                           \
+        if constexpr (l_ < (N1)) {                                                                               \
+          G1_SC += T::WAVES * ((G1_B) ? b_jstep : a_jstep);                                                      \
+          G1_DST += T::WAVES * 1024u;                                                                            \
+        } else {                                                                                                 \
+          G2_SC += T::WAVES * ((G2_B) ? b_jstep : a_jstep);                                                      \
+          G2_DST += T::WAVES * 1024u;                                                                            \
+        }                                                                                                        \
+      }                                                                                                          \
+      if constexpr (m_ == load0_ + 2) P0();                                                                      \
+      if constexpr (m_ == load0_ + every_ + 2) P1();                                                             \
+      if constexpr (m_ == load0_ + 2 * every_ + 2) P2();                                                         \
+      if constexpr (m_ == load0_ + 3 * every_ + 2) P3();                                                         \
+      if constexpr (every_ >= 4 && m_ == load0_ + 3) P4();                                                       \
+      if constexpr (every_ < 4 && m_ == load0_ + 3 * every_ + 3) P4();                                           \
+      __builtin_amdgcn_sched_barrier(0);                                                                         \
+    });                                                                                                          \
+  } while (0)
+
+  const int nk = g.nk;
+  constexpr int WAIT_PROLOGUE = (SB - 2) * (LA + LB) + LA + LB / 2;
+  constexpr int WAIT_LOOP = (SB - 1) * LA + (SB - 2) * LB - LA / 2;   // the second half of the newest A tile is issued after the wait
+  if (nk > 0) {
+#pragma unroll
+    for (int t = 0; t < SB - 1; ++t) {
+      issue_group(false, t, t, 0, LA);
+      issue_group(true, t, t, 0, LB);
+    }
+    issue_group(false, SB - 1, SB - 1, 0, LA);
+    issue_group(true, SB - 1, SB - 1, 0, LB / 2);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  if (clear) {
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+  }
+  if (nk > 0) {
+    wait_vmcnt<WAIT_PROLOGUE>();
+    __builtin_amdgcn_s_barrier();
+    mfma16_settle();   // the accumulators were written by vector-ALU instructions
+    static_for<NF>([&](auto mi_) { constexpr int m_ = decltype(mi_)::value; MBX_READ_ONE16(0, 0, lds_base, lds_base + B_RING, m_); });
+
+    constexpr uint32_t A_RING_END = (uint32_t)SA * T::A_BYTES, B_RING_END = B_RING + (uint32_t)SB * T::B_BYTES;
+    uint32_t a_rd = lds_base, b_rd = lds_base + B_RING, a_rd_next = 0, b_rd_next = 0;
+    uint32_t a_dst0 = lds_off(false, SA - 1, 0), b_dst0 = lds_off(true, 0, 0);
+    uint32_t a_sc0 = (uint32_t)SB * a_step + (uint32_t)wave * a_jstep, b_sc0 = (uint32_t)SB * b_step + (uint32_t)wave * b_jstep;
+    const uint32_t a_dst_end = A_RING_END + (uint32_t)wave * 1024u, b_dst_end = B_RING_END + (uint32_t)wave * 1024u;
+    uint32_t sc_b = scalar_off(true, SB - 1, LB / 2), dst_b = lds_off(true, SB - 1, LB / 2), sc_a = 0, dst_a = 0;
+    uint32_t past = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+      // k-step 0.  Group 1: the rest of B tile kt + SB - 1 (N1 = LB / 2 loads); group 2: the first half of A tile
+      // kt + SB, whose offsets p0 / p1 set up before its first load (gap NF + N1 * LEVERY).
+      auto p0 = [&]() { past = kt + SB < nk ? 0u : 0x80000000u; };
+      auto p1 = [&]() {
+        sc_a = a_sc0 | past;
+        dst_a = a_dst0;
+        if (DUAL) ra = kt + SB >= g.nk1 ? g.rsrc_a2 : g.rsrc_a;
+      };
+      auto p2 = [&]() {   // the stages k-step 1 reads the next tile's first operands from
+        a_rd_next = a_rd + T::A_BYTES;
+        a_rd_next = a_rd_next >= lds_base + A_RING_END ? lds_base : a_rd_next;
+      };
+      auto p3 = [&]() {
+        b_rd_next = b_rd + T::B_BYTES;
+        b_rd_next = b_rd_next >= lds_base + B_RING_END ? lds_base + B_RING : b_rd_next;
+      };
+      auto nop = [&]() {};
+      MBX_STEP16(0, 1, a_rd, b_rd, true, sc_b, dst_b, LB / 2, false, sc_a, dst_a, LA / 2, p0, p1, p2, p3, nop);
+      wait_frags(fa[1], fb[1]);
+      wait_vmcnt<WAIT_LOOP>();
+      __builtin_amdgcn_s_barrier();
+      // k-step 1.  Group 1: the second half of that A tile; group 2: the first half of B tile kt + SB (into the
+      // stage the barrier has just freed), whose offsets q1 sets up; q0 / q2 move on to K tile kt + SB + 1.
+      auto q0 = [&]() {   // sc_a / dst_a were taken from these in k-step 0
+        a_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * a_jstep : a_sc0 + a_step;
+        a_dst0 += T::A_BYTES;
+        a_dst0 = a_dst0 >= a_dst_end ? a_dst0 - A_RING_END : a_dst0;
+      };
+      auto q1 = [&]() {
+        sc_b = b_sc0 | past;
+        dst_b = b_dst0;
+        if (DUAL) rb = kt + SB >= g.nk1 ? g.rsrc_b2 : g.rsrc_b;
+      };
+      auto q2 = [&]() {
+        b_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * b_jstep : b_sc0 + b_step;
+        b_dst0 += T::B_BYTES;
+        b_dst0 = b_dst0 >= b_dst_end ? b_dst0 - (uint32_t)SB * T::B_BYTES : b_dst0;
+      };
+      MBX_STEP16(1, 0, a_rd_next, b_rd_next, false, sc_a, dst_a, LA / 2, true, sc_b, dst_b, LB / 2, q0, q1, q2, nop, nop);   // past the last tile this reads stale LDS into dead registers
+      a_rd = a_rd_next;
+      b_rd = b_rd_next;
+    }
+    wait_vmcnt<0>();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    mfma16_settle();   // the last products must have reached the accumulators before anything else reads them
+  }
+#undef MBX_READ_ONE16
+#undef MBX_STEP16
+}
+
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
+__device__ __forceinline__ void block_multiply(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds) {
+  if constexpr (T::MF == 32) block_multiply32<DT, A_MC, B_MC, T, DUAL>(g, acc, clear, lds);
+  else block_multiply16<DT, A_MC, B_MC, T, DUAL>(g, acc, clear, lds);
+}
+
 // c[m][n] = acc for m < m_lim, n < n_lim, where m = m_base + (row inside the tile) and
 // n = n_base + (column inside the tile).  Uses the LDS of the operand rings as a staging buffer.
 template <int DT, typename T>
-__device__ __forceinline__ void block_store(const f32x16 (&acc)[T::TM][T::TN], uint16_t* __restrict__ c, int64_t ldc,
+__device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][T::TN], uint16_t* __restrict__ c, int64_t ldc,
                                             int m_base, int m_lim, int n_base, int n_lim, char* lds_generic) {
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
   const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
   // accumulator (i, j), register r of lane l holds c[m][n] with
-  //   m = m_base + wm + 32 i + (l % 32),  n = n_base + wn + 32 j + 8 (r / 4) + 4 (l / 32) + (r % 4)
+  //   32 x 32 x 16: m = m_base + wm + 32 i + (l % 32),  n = n_base + wn + 32 j + 8 (r / 4) + 4 (l / 32) + (r % 4)
+  //   16 x 16 x 32: m = m_base + wm + 16 i + (l % 16),  n = n_base + wn + 16 j + 4 (l / 16) + r
+  // i.e. runs of four consecutive columns per lane: Q runs per product tile, at column run_col(q), of row tile_row.
+  constexpr int MF = T::MF, Q = MF == 32 ? 4 : 1;
+  const int tile_row = MF == 32 ? (lane & 31) : (lane & 15);
+  auto run_col = [&](int q) -> int { return MF == 32 ? q * 8 + (lane >> 5) * 4 : (lane >> 4) * 4; };
   if ((ldc % 8 == 0) && (((uintptr_t)c & 15u) == 0)) {
     // Staged through LDS (free by now) so that every global store instruction writes whole rows of the
     // tile: 64 lanes x 16 bytes = two 512-byte row segments, instead of 32 scattered 16-byte pieces.
@@ -409,16 +687,17 @@ __device__ __forceinline__ void block_store(const f32x16 (&acc)[T::TM][T::TN], u
     constexpr int ROW = T::BN * 2 + 16;   // bytes; the 16-byte pad spreads the rows of a column over the banks
 #pragma unroll
     for (int i = 0; i < T::TM; ++i) {
-      const int ml = wm + i * 32 + (lane & 31);
+      const int ml = wm + i * MF + tile_row;
 #pragma unroll
       for (int j = 0; j < T::TN; ++j) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int nl = wn + j * 32 + q * 8 + (lane >> 5) * 4;
-          const f32x16& v = acc[i][j];
+        for (int q = 0; q < Q; ++q) {
+          const int nl = wn + j * MF + run_col(q);
+          const typename T::Acc& v = acc[i][j];
+          const int o = MF == 32 ? q * 4 : 0;                    // first register of the run
           u32x2 w;
-          w[0] = pack2<DT>(v[q * 4 + 0], v[q * 4 + 1]);
-          w[1] = pack2<DT>(v[q * 4 + 2], v[q * 4 + 3]);
+          w[0] = pack2<DT>(v[o + 0], v[o + 1]);
+          w[1] = pack2<DT>(v[o + 2], v[o + 3]);
           *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
         }
       }
@@ -475,24 +754,25 @@ __device__ __forceinline__ void block_store(const f32x16 (&acc)[T::TM][T::TN], u
     const bool n_vec = (ldc % 4 == 0) && (((uintptr_t)c & 7u) == 0);
 #pragma unroll
     for (int i = 0; i < T::TM; ++i) {
-      const int m = m_base + wm + i * 32 + (lane & 31);
+      const int m = m_base + wm + i * MF + tile_row;
       if (m >= m_lim) continue;
       uint16_t* crow = c + (int64_t)m * ldc;
 #pragma unroll
       for (int j = 0; j < T::TN; ++j) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n_base + wn + j * 32 + q * 8 + (lane >> 5) * 4;
-          const f32x16& v = acc[i][j];
+        for (int q = 0; q < Q; ++q) {
+          const int n = n_base + wn + j * MF + run_col(q);
+          const typename T::Acc& v = acc[i][j];
+          const int o = MF == 32 ? q * 4 : 0;
           if (n + 3 < n_lim && n_vec) {
             u32x2 w;
-            w[0] = pack2<DT>(v[q * 4 + 0], v[q * 4 + 1]);
-            w[1] = pack2<DT>(v[q * 4 + 2], v[q * 4 + 3]);
+            w[0] = pack2<DT>(v[o + 0], v[o + 1]);
+            w[1] = pack2<DT>(v[o + 2], v[o + 3]);
             *(u32x2*)(crow + n) = w;
           } else {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-              if (n + t < n_lim) crow[n + t] = (uint16_t)(pack2<DT>(v[q * 4 + t], 0.f) & 0xffffu);
+              if (n + t < n_lim) crow[n + t] = (uint16_t)(pack2<DT>(v[o + t], 0.f) & 0xffffu);
           }
         }
       }
@@ -504,7 +784,7 @@ __device__ __forceinline__ void block_store(const f32x16 (&acc)[T::TM][T::TN], u
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
 __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
                                            int n_base, int n_lim, char* lds) {
-  f32x16 acc[T::TM][T::TN];
+  typename T::Acc acc[T::TM][T::TN];
   block_multiply<DT, A_MC, B_MC, T, DUAL>(g, acc, true, lds);
   block_store<DT, T>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds);
 }
@@ -643,7 +923,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "tail tile");
+  static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
   constexpr bool kSplit = T::BM != TS::BM;
   static_assert(!kSplit || T::BM == 2 * TS::BM, "tail tile");
   const int P = gridDim.x, run = P / kXcds;
@@ -738,7 +1018,7 @@ __device__ __forceinline__ void tn_tile(Args& g, const uint16_t* __restrict__ a,
   } else {
     // The reduction runs over the expert's rows in segments of at most seg_rows rows, each with buffers
     // of its own that cover exactly its rows.
-    f32x16 acc[TT::TM][TT::TN];
+    typename TT::Acc acc[TT::TM][TT::TN];
     int first = start;
     for (;;) {
       const int64_t left = end - first;

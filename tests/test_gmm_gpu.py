@@ -479,3 +479,48 @@ def test_fused_gated_activation_matches_the_two_step_formulation(dtype, act_name
     assert rel_err(out.cpu(), wantf) < (1e-5 if dtype == torch.float32 else 1e-2)
     odd = torch.randn(5, 3).to(dtype).cuda()             # not a multiple of 16 bytes: plain torch ops
     assert torch.equal(gated_activation(fn, odd, odd), fn(odd) * odd)
+
+
+_MFMA16_CHECK = r'''
+import sys, torch
+sys.path.insert(0, sys.argv[1])
+from megablocks_amd import grouped_gemm_util as gg
+torch.manual_seed(0)
+def rel(a, b):
+    return float((a.double() - b.double()).norm() / b.double().norm())
+worst = 0.0
+for dtype in (torch.bfloat16, torch.float16):
+    for groups, rows, k, n in ((8, 4096, 512, 768), (5, 1500, 320, 264), (64, 8192, 1024, 512), (3, 900, 1408, 2048)):
+        cuts = torch.sort(torch.randint(0, rows + 1, (groups - 1,)))[0]
+        sizes = torch.diff(torch.cat([torch.zeros(1, dtype=torch.int64), cuts, torch.tensor([rows])]))
+        if groups > 2:
+            sizes[2] += sizes[1]; sizes[1] = 0                      # an empty group
+        a = torch.randn(rows, k, device='cuda').to(dtype)
+        a2 = torch.randn(rows, k, device='cuda').to(dtype)
+        bn = (torch.randn(groups, k, n, device='cuda') * 0.1).to(dtype)
+        bn2 = (torch.randn(groups, k, n, device='cuda') * 0.1).to(dtype)
+        bt = bn.transpose(1, 2).contiguous()
+        g = torch.randn(rows, n, device='cuda').to(dtype)
+        bounds = torch.cumsum(sizes, 0).tolist()
+        want_nn = torch.cat([a[lo:hi].float() @ bn[e].float() for e, (lo, hi) in enumerate(zip([0] + bounds[:-1], bounds))])
+        want_dual = want_nn + torch.cat([a2[lo:hi].float() @ bn2[e].float() for e, (lo, hi) in enumerate(zip([0] + bounds[:-1], bounds))])
+        want_tn = torch.stack([a[lo:hi].float().t() @ g[lo:hi].float() for lo, hi in zip([0] + bounds[:-1], bounds)])
+        worst = max(worst, rel(gg.backend.gmm(a, bn, sizes), want_nn), rel(gg.backend.gmm(a, bt, sizes, trans_b=True), want_nn),
+                    rel(gg.backend.gmm(a, g, sizes, trans_a=True), want_tn), rel(gg.gmm_dual(a, bn, a2, bn2, sizes), want_dual))
+        assert int(torch.count_nonzero(gg.backend.gmm(a, g, sizes, trans_a=True)[1])) == 0 or groups <= 2
+print('worst', worst)
+assert worst < 1e-2, worst
+'''
+
+
+def test_gmm_on_the_16x16x32_instruction():
+    """MBX_MFMA=16 selects the main loop built on v_mfma_f32_16x16x32 (read once per process, hence the child
+    process): the three layouts and the two-pair product against fp32 torch."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, MBX_MFMA='16')
+    proc = subprocess.run([sys.executable, '-c', _MFMA16_CHECK, root], env=env, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    assert 'worst' in proc.stdout
