@@ -28,6 +28,7 @@ typedef void* mbx_stream_t; /* a hipStream_t; NULL = the default stream */
 enum mbx_itype { MBX_I16 = 0, MBX_I32 = 1, MBX_I64 = 2 };
 enum mbx_dtype { MBX_BF16 = 0, MBX_F16 = 1, MBX_F32 = 2 };
 enum mbx_layout { MBX_NN = 0, MBX_NT = 1, MBX_TN = 2 };
+enum mbx_activation { MBX_ACT_SILU = 0, MBX_ACT_GELU_TANH = 1 };
 
 #define MBX_EINVAL (-1)   /* bad enum / negative size / null pointer */
 #define MBX_ESCRATCH (-2) /* scratch buffer too small */
@@ -196,6 +197,24 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
                  const int32_t* bins, int num_groups, int64_t rows, int k, int n, int layout,
                  mbx_stream_t stream);
 
+/* The first product of the expert MLP with its activation, megablocks/layers/mlp.py:521-522 / 414-416
+ * (`x = gmm(x, w1, batch_sizes, trans_b=True); x = activation_fn(x)`), in one launch:
+ *   c[r_e] = a[r_e] @ b[e]^T (b is [E, n, k]),   c_act = act(c)
+ * where act is applied in the product's epilogue to c as stored (rounded to `dtype`), i.e. to the value the
+ * reference's separate activation kernel reads.  Both outputs are [rows, n].  act: MBX_ACT_GELU_TANH.
+ * MBX_EUNSUPPORTED (the caller runs mbx_gmm and the activation itself): fp32, another activation, k not a multiple of 64,
+ * n not a multiple of 8, operands or outputs not 16-byte aligned, one expert's weights of 2 GiB or more. */
+int mbx_gmm_act(const void* a, const void* b, void* c, void* c_act, int dtype, const int32_t* bins,
+                int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
+
+/* The activation gradient of the expert MLP's backward, megablocks/layers/mlp.py:478-483 with
+ * megablocks/layers/gelu.py:9-13 (`dact = gmm(ddsd_out, w2, trans_b=True); dsdd_out = gelu_backward_(dact, sdd_out)`),
+ * in one launch:   c[r_e] = round(a[r_e] @ b[e]^T) * act'(pre[r_e])
+ * with `pre` the saved first product ([rows, n], read in the epilogue).  The product is rounded to `dtype` before the
+ * multiplication, as the reference's two steps round it.  Same restrictions and return codes as mbx_gmm_act. */
+int mbx_gmm_dact(const void* a, const void* b, const void* pre, void* c, int dtype, const int32_t* bins,
+                 int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
+
 /* megablocks/layers/gelu.py:9-13 `_gelu_backward_inplace(g, x)`: g *= d/dx gelu_tanh(x). */
 int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel,
                               mbx_stream_t stream);
@@ -204,7 +223,6 @@ int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel,
  * (`activation_fn(x1) * x2`) in one pass: out = round(round(act(a)) * b), i.e. with the same two
  * roundings as the reference's two element-wise ops.  act: 0 = SiLU, 1 = tanh-GELU.  numel must be a
  * multiple of 16 bytes' worth of elements and the buffers 16-byte aligned (else MBX_EINVAL). */
-enum mbx_activation { MBX_ACT_SILU = 0, MBX_ACT_GELU_TANH = 1 };
 int mbx_glu_forward(const void* a, const void* b, void* out, int dtype, int act, int64_t numel,
                     mbx_stream_t stream);
 

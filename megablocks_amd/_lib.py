@@ -42,6 +42,8 @@ _SIGNATURES = {
     'mbx_binned_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _vp]),
     'mbx_gmm': (_i, [_vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_dual': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
+    'mbx_gmm_act': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
+    'mbx_gmm_dact': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gelu_backward_inplace': (_i, [_vp, _vp, _i, _i64, _vp]),
     'mbx_glu_forward': (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp]),
     'mbx_glu_backward': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _vp]),

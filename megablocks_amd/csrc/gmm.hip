@@ -580,9 +580,11 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
 // Launch of the direct-to-LDS kernels (k a multiple of 64 for NN / NT; sizes as dma_sizes_ok() allows).
 // TS is the tile the tail of an NN / NT launch is cut into (TS = T: never cut).
 // a2 / b2 non-null (NN / NT only): c = a @ b[e] + a2 @ b2[e], the second pair shaped like the first.
+// epi / extra (NT, one operand pair only): dma::kEpiAct with the second output, dma::kEpiDact with the second input.
 template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
-            int layout, hipStream_t s, const void* a2 = nullptr, const void* b2 = nullptr) {
+            int layout, hipStream_t s, const void* a2 = nullptr, const void* b2 = nullptr, int epi = dma::kEpiNone,
+            void* extra = nullptr) {
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
   const uint16_t* ap2 = (const uint16_t*)a2;
@@ -614,17 +616,26 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
   if (tiles > 0x7fffffff) return MBX_ERANGE;
   const unsigned grid = (unsigned)persistent_grid(tiles);
-#define MBX_LAUNCH_ROWS(B_MC, DUAL)                                                                   \
+#define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI)                                                              \
   do {                                                                                                \
-    auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL>;                                          \
+    auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL, EPI>;                                     \
     int rc = allow_lds(kern, lds);                                                                    \
     if (rc) return rc;                                                                                \
-    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2);  \
+    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra);  \
   } while (0)
+  if (epi != dma::kEpiNone) {
+    if (layout != MBX_NT || dual || !extra) return MBX_EINVAL;
+    if constexpr (T::MF == 32) {
+      if (epi == dma::kEpiAct) MBX_LAUNCH_ROWS(false, false, dma::kEpiAct); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDact);
+      return launch_status();
+    } else {
+      return MBX_EUNSUPPORTED;
+    }
+  }
   if (layout == MBX_NT) {
-    if (dual) MBX_LAUNCH_ROWS(false, true); else MBX_LAUNCH_ROWS(false, false);
+    if (dual) MBX_LAUNCH_ROWS(false, true, dma::kEpiNone); else MBX_LAUNCH_ROWS(false, false, dma::kEpiNone);
   } else {
-    if (dual) MBX_LAUNCH_ROWS(true, true); else MBX_LAUNCH_ROWS(true, false);
+    if (dual) MBX_LAUNCH_ROWS(true, true, dma::kEpiNone); else MBX_LAUNCH_ROWS(true, false, dma::kEpiNone);
   }
 #undef MBX_LAUNCH_ROWS
   return launch_status();
@@ -755,6 +766,38 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
   }
   if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
   return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+}
+
+// The NT product with an activation epilogue (epi: dma::kEpiAct / dma::kEpiDact), for the shapes the direct-to-LDS
+// kernels take; anything else is MBX_EUNSUPPORTED and the caller runs the product and the element-wise pass.
+static int gmm_nt_epilogue(const void* a, const void* b, void* c, void* extra, int dtype, const int32_t* bins, int num_groups,
+                           int64_t rows, int k, int n, int act, int epi, mbx_stream_t stream) {
+  if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
+  if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
+  if (act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
+  if (num_groups == 0 || rows == 0 || n == 0) return 0;
+  if (!bins || !c || !extra || (k > 0 && (!a || !b))) return MBX_EINVAL;
+  if (rows > 0x7fffffff) return MBX_ERANGE;
+  const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(extra) && k > 0 &&
+                  k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n) && !use_mfma16();
+  if (!ok) return MBX_EUNSUPPORTED;
+  hipStream_t s = as_stream(stream);
+  if (half_height_only(rows, num_groups, n)) {
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+    return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+  }
+  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+  return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+}
+
+int mbx_gmm_act(const void* a, const void* b, void* c, void* c_act, int dtype, const int32_t* bins, int num_groups,
+                int64_t rows, int k, int n, int act, mbx_stream_t stream) {
+  return gmm_nt_epilogue(a, b, c, c_act, dtype, bins, num_groups, rows, k, n, act, dma::kEpiAct, stream);
+}
+
+int mbx_gmm_dact(const void* a, const void* b, const void* pre, void* c, int dtype, const int32_t* bins, int num_groups,
+                 int64_t rows, int k, int n, int act, mbx_stream_t stream) {
+  return gmm_nt_epilogue(a, b, c, (void*)pre, dtype, bins, num_groups, rows, k, n, act, dma::kEpiDact, stream);
 }
 
 int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel, mbx_stream_t stream) {

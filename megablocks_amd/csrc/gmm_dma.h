@@ -664,11 +664,99 @@ __device__ __forceinline__ void block_multiply(const Args& g, typename T::Acc (&
   else block_multiply16<DT, A_MC, B_MC, T, DUAL>(g, acc, clear, lds);
 }
 
+// ---- activation in the epilogue (tanh-GELU: megablocks/layers/arguments.py:19, megablocks/layers/gelu.py:9-13) ----
+// Both are evaluated in fp32 on the value as stored (rounded to the 16-bit type), which is what the reference's
+// separate element-wise kernels see, and through one exponential and one reciprocal instead of a library tanh:
+//   gelu_tanh(x) = 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  tanh(u) = 1 - 2 / (1 + exp(2u)),  u = 0.79788456 (x + 0.044715 x^3)
+// Evaluated on the eight values of a 16-byte chunk at a time, stage by stage: a wave alone on its SIMD issues a
+// dependent instruction only every eight cycles, an independent one every four, so the eight chains are interleaved.
+__device__ __forceinline__ void sigmoid_2u8(const float (&x)[8], float (&x2)[8], float (&s)[8]) {   // s = 1 / (1 + exp(-2u))
+  float z[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x2[i] = x[i] * x[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = -0.102943240f * x2[i] - 2.30220819f;      // -(2 * 0.79788456) (1 + 0.044715 x^2) log2(e)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = z[i] * x[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = __builtin_amdgcn_exp2f(z[i]);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = 1.f + z[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = __builtin_amdgcn_rcpf(z[i]);
+}
+__device__ __forceinline__ void gelu_tanh_fwd8(float (&x)[8]) {                // x <- gelu_tanh(x) = x s
+  float x2[8], s[8];
+  sigmoid_2u8(x, x2, s);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x[i] = x[i] * s[i];
+}
+// g <- g * d/dx gelu_tanh(x).  With t = tanh(u) = 2 s - 1 the expression of gelu.py:9-13,
+// 0.5 x (1 - t^2) (0.79788456 + 0.1070322243 x^2) + 0.5 (1 + t), is s (1 + x (1 - s) (1.59576912 + 0.2140644486 x^2)).
+__device__ __forceinline__ void gelu_tanh_bwd8(float (&g)[8], const float (&x)[8]) {
+  float x2[8], s[8], q[8];
+  sigmoid_2u8(x, x2, s);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q[i] = 0.2140644486f * x2[i] + 1.59576912f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q[i] = q[i] * x[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x2[i] = 1.f - s[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q[i] = q[i] * x2[i] + 1.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = s[i] * q[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) g[i] = g[i] * s[i];
+}
+
+// What the store of an output tile does besides storing it:
+//   kEpiNone  nothing;
+//   kEpiAct   also stores gelu_tanh of the (rounded) tile to a second output of the same shape;
+//   kEpiDact  multiplies the (rounded) tile by d/dx gelu_tanh of a second input of the same shape before storing it.
+enum { kEpiNone = 0, kEpiAct = 1, kEpiDact = 2 };
+
+// the eight 16-bit values of a 16-byte chunk as fp32 and back (rounded)
+template <int DT>
+__device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {
+  typedef typename Elem<DT>::type E;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    f[2 * w] = Elem<DT>::to_f32(__builtin_bit_cast(E, (uint16_t)(v[w] & 0xffffu)));
+    f[2 * w + 1] = Elem<DT>::to_f32(__builtin_bit_cast(E, (uint16_t)(v[w] >> 16)));
+  }
+}
+template <int DT>
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
+  u32x4 r;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) r[w] = pack2<DT>(f[2 * w], f[2 * w + 1]);
+  return r;
+}
+template <int DT>
+__device__ __forceinline__ u32x4 gelu_fwd_chunk(const u32x4& v) {
+  float x[8];
+  unpack8<DT>(v, x);
+  gelu_tanh_fwd8(x);
+  return pack8<DT>(x);
+}
+template <int DT>
+__device__ __forceinline__ u32x4 gelu_bwd_chunk(const u32x4& gv, const u32x4& xv) {
+  float g[8], x[8];
+  unpack8<DT>(gv, g);
+  unpack8<DT>(xv, x);
+  gelu_tanh_bwd8(g, x);
+  return pack8<DT>(g);
+}
+
 // c[m][n] = acc for m < m_lim, n < n_lim, where m = m_base + (row inside the tile) and
 // n = n_base + (column inside the tile).  Uses the LDS of the operand rings as a staging buffer.
-template <int DT, typename T>
+// `extra` (EPI != kEpiNone; laid out like c, same pitch, 16-byte aligned like c): the second output of kEpiAct, the
+// second input of kEpiDact.  Those two take the staged path only (the launch checks pitch and alignment).
+template <int DT, typename T, int EPI = kEpiNone>
 __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][T::TN], uint16_t* __restrict__ c, int64_t ldc,
-                                            int m_base, int m_lim, int n_base, int n_lim, char* lds_generic) {
+                                            int m_base, int m_lim, int n_base, int n_lim, char* lds_generic,
+                                            uint16_t* __restrict__ extra = nullptr) {
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
@@ -721,6 +809,31 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
     uint32_t off = ((uint32_t)m * (uint32_t)ldc + (uint32_t)n) * 2u;   // outputs are below 2 GiB
     const uint32_t off_step = (uint32_t)ROW_STEP * (uint32_t)ldc * 2u;
     char* const cb = (char*)c;
+    char* const eb = (char*)extra;
+    // kEpiDact: the chunks of the second input that belong to a batch are fetched one batch ahead (the registers of
+    // the accumulators are free by now), so that their latency is behind the arithmetic and the stores of the batch
+    // before; rows or columns outside the tile's part of c are not fetched (zeros: their results are not stored)
+    u32x4 pre[EPI == kEpiDact ? BATCH : 1], pre_next[EPI == kEpiDact ? BATCH : 1];
+    auto fetch_pre = [&](u32x4 (&dst)[EPI == kEpiDact ? BATCH : 1], int m0, uint32_t off0) {
+      if constexpr (EPI == kEpiDact) {
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          const u32x4 zero = {0u, 0u, 0u, 0u};
+          dst[u] = zero;
+          if (m0 + u * ROW_STEP < m_lim && n < n_lim) {
+            const uint16_t* src = (const uint16_t*)(eb + (off0 + (uint32_t)u * off_step));
+            if (n + 8 <= n_lim) {
+              dst[u] = __builtin_nontemporal_load((const u32x4*)src);
+            } else {
+#pragma unroll
+              for (int t = 0; t < 8; ++t)
+                if (n + t < n_lim) dst[u][t >> 1] |= (uint32_t)src[t] << ((t & 1) * 16);
+            }
+          }
+        }
+      }
+    };
+    fetch_pre(pre_next, m, off);
 #pragma unroll 1
     for (int b = 0; b < ITERS; b += BATCH) {
       u32x4 v[BATCH];
@@ -728,22 +841,44 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
         constexpr int u = decltype(ui)::value;
         v[u] = lds_read_b128<u * ROW_STEP * ROW>(rd_addr + (uint32_t)(b * ROW_STEP * ROW));
       });
+      if constexpr (EPI == kEpiDact) {
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) pre[u] = pre_next[u];
+        if (b + BATCH < ITERS) fetch_pre(pre_next, m + BATCH * ROW_STEP, off + BATCH * off_step);
+      }
       asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+      if constexpr (EPI == kEpiDact) {
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) v[u] = gelu_bwd_chunk<DT>(v[u], pre[u]);
+      }
       if (full_n) {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u)
-          if (m + u * ROW_STEP < m_lim) __builtin_nontemporal_store(v[u], (u32x4*)(cb + (off + (uint32_t)u * off_step)));
+          if (m + u * ROW_STEP < m_lim) {
+            __builtin_nontemporal_store(v[u], (u32x4*)(cb + (off + (uint32_t)u * off_step)));
+            if constexpr (EPI == kEpiAct) {
+              const u32x4 y = gelu_fwd_chunk<DT>(v[u]);
+              __builtin_nontemporal_store(y, (u32x4*)(eb + (off + (uint32_t)u * off_step)));
+            }
+          }
       } else {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) {
           if (m + u * ROW_STEP >= m_lim || n >= n_lim) continue;
           uint16_t* dst = (uint16_t*)(cb + (off + (uint32_t)u * off_step));
+          u32x4 y = v[u];
+          if constexpr (EPI == kEpiAct) y = gelu_fwd_chunk<DT>(v[u]);
+          uint16_t* dst2 = (uint16_t*)(eb + (off + (uint32_t)u * off_step));
           if (n + 8 <= n_lim) {
             *(u32x4*)dst = v[u];
+            if constexpr (EPI == kEpiAct) *(u32x4*)dst2 = y;
           } else {
 #pragma unroll
             for (int t = 0; t < 8; ++t)
-              if (n + t < n_lim) dst[t] = (uint16_t)(v[u][t >> 1] >> ((t & 1) * 16));
+              if (n + t < n_lim) {
+                dst[t] = (uint16_t)(v[u][t >> 1] >> ((t & 1) * 16));
+                if constexpr (EPI == kEpiAct) dst2[t] = (uint16_t)(y[t >> 1] >> ((t & 1) * 16));
+              }
           }
         }
       }
@@ -781,12 +916,12 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
 }
 
 // c = A_tile * B_tile over all K tiles (the whole product of one output tile)
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, int EPI = kEpiNone>
 __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
-                                           int n_base, int n_lim, char* lds) {
+                                           int n_base, int n_lim, char* lds, uint16_t* __restrict__ extra = nullptr) {
   typename T::Acc acc[T::TM][T::TN];
   block_multiply<DT, A_MC, B_MC, T, DUAL>(g, acc, true, lds);
-  block_store<DT, T>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds);
+  block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra);
 }
 
 // Buffer sizes stay below 2 GiB: bit 31 of a byte offset marks a load that must fetch nothing.
@@ -917,11 +1052,12 @@ struct RowTiles {
 // the tail then costs little more than half a round.  TS = T switches this off.
 // DUAL: c = a @ b[e] + a2 @ b2[e] in one pass (k is the reduction length of each pair, at least
 // (SB + 1) K tiles), as one reduction over 2 k.
-template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false>
+// EPI: see block_store; `extra` is its second output / input, [rows, n] like c.
+template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false, int EPI = kEpiNone>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
-                const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2) {
+                const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
   constexpr bool kSplit = T::BM != TS::BM;
@@ -968,12 +1104,13 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
     g.b_r0 = tn * T::BN;
     uint16_t* const c_tile = c + (int64_t)row0 * n;
+    uint16_t* const e_tile = EPI != kEpiNone ? extra + (int64_t)row0 * n : nullptr;
     // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
     use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
     if (use_ts) {
-      block_gemm<DT, false, B_MC, TS, DUAL>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds);
+      block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile);
     } else {
-      block_gemm<DT, false, B_MC, T, DUAL>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds);
+      block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile);
     }
     tile_done();
   }

@@ -5,6 +5,7 @@ bf16/f16 MFMA kernels of libmbx.so.
 `batch_sizes` may be the host int64 tensor the reference passes (mlp.py:502) or, to avoid
 the device-to-host copy, a device tensor of per-expert row counts.
 """
+import os
 import types
 
 import torch
@@ -158,6 +159,87 @@ def gmm_dual(a, b, a2, b2, batch_sizes, trans_b=False, c=None):
         c += gmm(a2, b2, batch_sizes, trans_b=trans_b)
         return c
     _lib.check(rc, 'gmm_dual')
+    return c
+
+
+ACT_GELU_TANH = 1   # mbx_activation of include/mbx.h
+# False: gmm_act / gmm_dact run the product and the element-wise pass as two launches (what they do anyway for shapes
+# the epilogue kernels do not take); a switch for measurements
+ACTIVATION_EPILOGUES = os.environ.get('MBX_ACTIVATION_EPILOGUES', '1') != '0'
+# The epilogue costs every output tile some 19 k (activation) to 37 k (its gradient) cycles in which the matrix cores
+# idle; the separate pass it replaces costs a trip of the [rows, n] tensor through memory.  Tensors that fit the
+# part's 256 MiB Infinity Cache make that trip cheaply (c2's 128 MiB intermediate: the layer step is 2 % faster with
+# the two passes), so the epilogues are used from this size on (c5's 1.5 GiB: 3.7 % faster with them).
+ACTIVATION_EPILOGUE_MIN_BYTES = 256 << 20
+
+
+def _use_epilogue(fuse, a, rows, n):
+    if a.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    if fuse is None:
+        return ACTIVATION_EPILOGUES and rows * n * a.element_size() >= ACTIVATION_EPILOGUE_MIN_BYTES
+    return bool(fuse)
+
+
+def _nt_operands(a, b, batch_sizes, what):
+    _lib.require_cuda(a, b)
+    if a.ndim != 2 or b.ndim != 3 or a.dtype != b.dtype:
+        raise ValueError(f'{what}: a must be [rows, k] and b [num_groups, n, k] of the same dtype')
+    a, b = a.contiguous(), b.contiguous()
+    bins = _device_bins(batch_sizes, a.device, a.shape[0])
+    if b.shape[0] != bins.shape[0] or b.shape[2] != a.shape[1]:
+        raise ValueError(f'{what}: b does not match a and batch_sizes')
+    return a, b, bins
+
+
+def gmm_act(a, b, batch_sizes, fuse=None):
+    """(c, gelu_tanh(c)) with c[r_e] = a[r_e] @ b[e].T: the first product of the expert MLP and its activation
+    (mlp.py:521-522), the activation applied in the product's epilogue where the library has a kernel for the shape
+    (16-bit types, k a multiple of 64, n of 8) and the output is large enough for that to pay (`fuse` None; True /
+    False force the choice), else as a separate element-wise pass."""
+    a, b, bins = _nt_operands(a, b, batch_sizes, 'gmm_act')
+    rows, k, n, groups = a.shape[0], a.shape[1], b.shape[1], bins.shape[0]
+    c = torch.empty((rows, n), dtype=a.dtype, device=a.device)
+    c_act = torch.empty_like(c)
+    rc = _lib.EUNSUPPORTED
+    if _use_epilogue(fuse, a, rows, n):
+        with _lib.device_of(a), _lib.record('gmm_nt_act', rows=rows, k=k, n=n, elem=a.element_size(), groups=groups) as rec:
+            rc = lib.mbx_gmm_act(_lib.ptr(a), _lib.ptr(b), _lib.ptr(c), _lib.ptr(c_act), _lib.dtype_of(a), _lib.ptr(bins),
+                                 groups, rows, k, n, ACT_GELU_TANH, _lib.stream())
+            if rc == _lib.EUNSUPPORTED:
+                rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        gmm(a, b, batch_sizes, trans_b=True, c=c)
+        return c, torch.nn.functional.gelu(c, approximate='tanh')
+    _lib.check(rc, 'gmm_act')
+    return c, c_act
+
+
+def gmm_dact(a, b, pre, batch_sizes, c=None, fuse=None):
+    """round(a[r_e] @ b[e].T) * d/dx gelu_tanh(pre[r_e]): the activation gradient of the expert MLP's backward
+    (mlp.py:478-483 with gelu.py:9-13) with the multiplication in the product's epilogue where the library has a
+    kernel for the shape, else as `gmm` and `gelu_backward_`.  Written to `c` when given (which may not be `pre`)."""
+    a, b, bins = _nt_operands(a, b, batch_sizes, 'gmm_dact')
+    rows, k, n, groups = a.shape[0], a.shape[1], b.shape[1], bins.shape[0]
+    _lib.require_cuda(pre, c)
+    if tuple(pre.shape) != (rows, n) or pre.dtype != a.dtype or not pre.is_contiguous():
+        raise ValueError('gmm_dact: pre has the wrong shape, dtype or layout')
+    if c is None:
+        c = torch.empty((rows, n), dtype=a.dtype, device=a.device)
+    elif tuple(c.shape) != (rows, n) or c.dtype != a.dtype or not c.is_contiguous() or c.data_ptr() == pre.data_ptr():
+        raise ValueError('gmm_dact: c has the wrong shape, dtype or layout')
+    rc = _lib.EUNSUPPORTED
+    if _use_epilogue(fuse, a, rows, n):
+        with _lib.device_of(a), _lib.record('gmm_nt_dact', rows=rows, k=k, n=n, elem=a.element_size(), groups=groups) as rec:
+            rc = lib.mbx_gmm_dact(_lib.ptr(a), _lib.ptr(b), _lib.ptr(pre), _lib.ptr(c), _lib.dtype_of(a), _lib.ptr(bins),
+                                  groups, rows, k, n, ACT_GELU_TANH, _lib.stream())
+            if rc == _lib.EUNSUPPORTED:
+                rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        from megablocks_amd.layers.gelu import gelu_backward_
+        gmm(a, b, batch_sizes, trans_b=True, c=c)
+        return gelu_backward_(c, pre)
+    _lib.check(rc, 'gmm_dact')
     return c
 
 

@@ -139,6 +139,44 @@ class Topology:
         return self.column_indices.numel()
 
 
+class GroupedGeluMLP(torch.autograd.Function):
+    """GroupedMLP.forward with the default activation (mlp.py:499-523: gmm, tanh-GELU, gmm) and the backward autograd
+    derives for it, with the two element-wise passes moved into the epilogues of the products next to them: the
+    first product also writes its activation (`gmm_act`), and the gradient of the activation's input comes out of
+    the `ddsd_out @ w2^T` product directly (`gmm_dact`).  Saves what autograd would save: x, the first product and its
+    activation."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
+    def forward(ctx, x, w1, w2, batch_sizes):
+        if ctx._fwd_used_autocast:
+            x, w1, w2 = x.to(ctx._dtype), w1.to(ctx._dtype), w2.to(ctx._dtype)
+        x, w1, w2 = x.contiguous(), w1.contiguous(), w2.contiguous()
+        sdd_out, activation_fn_out = gg.gmm_act(x, w1, batch_sizes)
+        dsd_out = gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+        ctx.save_for_backward(w1, w2, batch_sizes, x, sdd_out, activation_fn_out)
+        return dsd_out
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
+    def backward(ctx: Any, ddsd_out: torch.Tensor):
+        w1, w2, batch_sizes, x, sdd_out, activation_fn_out = ctx.saved_tensors
+        ddsd_out = ddsd_out.contiguous()
+        dx = dw1 = dw2 = None
+        if ctx.needs_input_grad[2]:
+            dw2 = gg.backend.gmm(activation_fn_out, ddsd_out, batch_sizes, trans_a=True)
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            dsdd_out = gg.gmm_dact(ddsd_out, w2, sdd_out, batch_sizes)
+            if ctx.needs_input_grad[1]:
+                dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
+            if ctx.needs_input_grad[0]:
+                dx = gg.backend.gmm(dsdd_out, w1, batch_sizes)
+        return dx, dw1, dw2, None
+
+
+grouped_gelu_mlp = GroupedGeluMLP.apply
+
+
 class MemoryOptimizedGroupedMLP(torch.autograd.Function):
     """GroupedMLP with a hand-scheduled backward that recomputes the activation and reuses
     buffers (mlp.py:397-493)."""
@@ -150,8 +188,11 @@ class MemoryOptimizedGroupedMLP(torch.autograd.Function):
             x, w1, w2 = x.to(ctx._dtype), w1.to(ctx._dtype), w2.to(ctx._dtype)
         if not x.is_contiguous() or not w1.is_contiguous() or not w2.is_contiguous():
             raise ValueError("Expected contiguous 'x', 'w1' and 'w2'.")
-        sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
-        activation_fn_out = activation_fn(sdd_out)
+        if activation_fn is DEFAULT_ACTIVATION_FN:
+            sdd_out, activation_fn_out = gg.gmm_act(x, w1, batch_sizes)
+        else:
+            sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
+            activation_fn_out = activation_fn(sdd_out)
         dsd_out = gg.backend.gmm(activation_fn_out, w2, batch_sizes)
         ctx.x_shape = x.shape
         ctx.sdd_out_shape = sdd_out.shape
@@ -181,9 +222,9 @@ class MemoryOptimizedGroupedMLP(torch.autograd.Function):
         dw2 = gg.backend.gmm(activation_fn_out.detach(), ddsd_out, batch_sizes, trans_a=True)
 
         if default_act:
-            # d(activation output) overwrites the recomputed activation, then becomes d(sdd_out) in place.
-            dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True, c=activation_fn_out)
-            dsdd_out = gelu.gelu_backward_(dactivation_fn_out, sdd_out)
+            # d(sdd_out) overwrites the recomputed activation: the product ddsd_out @ w2^T with the closed-form GELU
+            # gradient (gelu.py:9-13) in its epilogue
+            dsdd_out = gg.gmm_dact(ddsd_out, w2, sdd_out, batch_sizes, c=activation_fn_out)
         else:
             dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True)
             activation_fn_out.backward(dactivation_fn_out)
@@ -234,6 +275,8 @@ class SparseMLP(torch.nn.Module):
         w1, w2 = self._expert_views(self.w1, self.w2)
         if self.args.memory_optimized_mlp:
             return memory_optimized_grouped_mlp(x, w1, w2, batch_sizes, self.args.activation_fn)
+        if self.args.activation_fn is DEFAULT_ACTIVATION_FN and x.is_cuda:
+            return grouped_gelu_mlp(x, w1, w2, batch_sizes)
         x = gg.ops.gmm(x, w1, batch_sizes, trans_b=True)
         x = self.args.activation_fn(x)
         return gg.ops.gmm(x, w2, batch_sizes)

@@ -524,3 +524,50 @@ def test_gmm_on_the_16x16x32_instruction():
     proc = subprocess.run([sys.executable, '-c', _MFMA16_CHECK, root], env=env, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert 'worst' in proc.stdout
+
+
+EPILOGUE = [  # groups, rows, k, n -- full and half-height tiles, partial last column tile, shapes off the fused path
+    (8, 4096, 1024, 4096), (64, 16384, 1024, 1024), (5, 1500, 320, 264), (3, 700, 128, 1408), (1, 37, 64, 8),
+    (4, 1000, 72, 256), (16, 6000, 2048, 520),
+]
+
+
+@pytest.mark.parametrize('groups,rows,k,n', EPILOGUE)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+def test_gmm_with_activation_epilogues(gg, groups, rows, k, n, dtype):
+    """gmm_act: (x @ w1^T, gelu_tanh of it) in one launch; gmm_dact: round(dy @ w2^T) * gelu_tanh'(pre).  Against the
+    two-step formulation of mlp.py:521-522 and mlp.py:478-483 / gelu.py:9-13 in fp32 with the reference's roundings."""
+    torch.manual_seed(groups * 7 + n)
+    sizes = _sizes(groups, rows, seed=rows + k, empty=(1,) if groups > 2 else ())
+    a = torch.randn(rows, k, device='cuda').to(dtype)
+    b = (torch.randn(groups, n, k, device='cuda') * (1.5 / k ** 0.5)).to(dtype)      # pre-activations of order one
+    ref = _ref_gpu(a, b, sizes, False, True)
+    want_pre = ref.to(dtype)
+    want_act = torch.nn.functional.gelu(want_pre.float(), approximate='tanh')
+    guard = torch.full((rows + 64, n), 5.0, device='cuda', dtype=dtype)
+    pre, act = gg.gmm_act(a, b, sizes, fuse=True)
+    assert pre.shape == (rows, n) and act.shape == (rows, n) and pre.dtype == dtype and act.dtype == dtype
+    tol = 1e-4 if dtype == torch.float32 else TOL
+    assert rel_err(pre.float(), ref) < tol
+    assert torch.equal(pre, gg.backend.gmm(a, b, sizes, trans_b=True))         # the product itself is the same kernel's
+    # the activation is taken of the stored product: one rounding step of the output type away from the fp32 formula
+    assert rel_err(act.float(), torch.nn.functional.gelu(pre.float(), approximate='tanh')) < (1e-6 if dtype == torch.float32 else 3e-3)
+    assert rel_err(act.float(), want_act) < tol
+
+    dy = torch.randn(rows, k, device='cuda').to(dtype)
+    x_pre = (torch.randn(rows, n, device='cuda') * 1.5).to(dtype)
+    prod = _ref_gpu(dy, b, sizes, False, True).to(dtype).float()
+    want = prod * oracle.gelu_tanh_backward(torch.ones_like(prod).cpu(), x_pre.float().cpu()).cuda()
+    got = gg.gmm_dact(dy, b, x_pre, sizes, fuse=True)
+    assert got.shape == (rows, n) and got.dtype == dtype and rel_err(got.float(), want) < tol
+    out = guard[:rows]
+    assert gg.gmm_dact(dy, b, x_pre, sizes, c=out, fuse=True) is out and torch.equal(out, got)
+    two_step = gg.gmm_dact(dy, b, x_pre, sizes, fuse=False)            # product, then gelu_backward_ in place
+    assert rel_err(two_step.float(), want) < tol and rel_err(got.float(), two_step.float()) < (1e-6 if dtype == torch.float32 else 4e-3)
+    pre2, act2 = gg.gmm_act(a, b, sizes, fuse=False)
+    assert torch.equal(pre2, pre) and rel_err(act.float(), act2.float()) < (1e-6 if dtype == torch.float32 else 4e-3)
+    assert bool((guard[rows:] == 5.0).all())
+    with pytest.raises(ValueError):
+        gg.gmm_dact(dy, b, x_pre, sizes, c=x_pre)                              # the epilogue reads pre while it writes c
+    with pytest.raises(ValueError):
+        gg.gmm_act(a, b[:, :, :k - 8].contiguous(), sizes)

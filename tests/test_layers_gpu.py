@@ -113,6 +113,35 @@ def test_dmoe_forward_backward_vs_oracle(syn, tokens, hidden, ffn, experts, top_
         assert rel_err(layer.router.layer.weight.grad, want_grads['router']) < 5 * tol
 
 
+@pytest.mark.parametrize('mlp_impl,memopt', [('grouped', False), ('grouped', True), ('sparse', False), ('sparse', True)])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_dmoe_mlp_with_activation_epilogues_vs_oracle(syn, monkeypatch, mlp_impl, memopt, dtype):
+    """The GELU expert MLP with the activation and its gradient in the epilogues of the grouped products (taken by
+    itself only for intermediates beyond the Infinity Cache; forced here) against the oracle, forward and backward."""
+    from megablocks_amd import grouped_gemm_util as gg
+    monkeypatch.setattr(gg, 'ACTIVATION_EPILOGUE_MIN_BYTES', 0)
+    w = syn.Workload('t', 1500, 256, 768, 8, 2, 'mlp', mlp_impl, dtype, 'logits')
+    inp = syn.make_inputs(w, seed=5)
+    for k in ('x', 'grad', 'w1', 'w2', 'expert_weights'):
+        inp[k] = inp[k].to(dtype).float()
+    want, _, want_grads, _ = _oracle_step(w, inp, True)
+    layer = syn.build_layer(w, inp, memory_optimized=memopt)
+    x = inp['x'].to(dtype).cuda().requires_grad_(True)
+    ew = inp['expert_weights'].to(dtype).cuda().requires_grad_(True)
+    from megablocks_amd import _lib
+    _lib.profile_hook = []
+    try:
+        out = syn.layer_step(layer, w, x, inp['grad'].to(dtype).cuda(), (inp['scores'].to(dtype).cuda(), ew, inp['top_experts'].cuda()))
+        torch.cuda.synchronize()
+        launched = {name for name, *_ in _lib.profile_hook}
+    finally:
+        _lib.profile_hook = None
+    assert {'gmm_nt_act', 'gmm_nt_dact'} <= launched                      # the epilogue kernels are what ran
+    assert rel_err(out, want) < 1e-2 and rel_err(x.grad, want_grads['x']) < 1e-2
+    assert rel_err(layer.experts.mlp.w1.grad, want_grads['w1']) < 1e-2 and rel_err(layer.experts.mlp.w2.grad, want_grads['w2']) < 1e-2
+    assert rel_err(ew.grad, want_grads['expert_weights']) < 1e-2
+
+
 @pytest.mark.parametrize('tokens,hidden,experts', [(4096, 1024, 64), (5003, 264, 8), (16384, 512, 16)])
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 def test_router_linear_gradients(tokens, hidden, experts, dtype):
