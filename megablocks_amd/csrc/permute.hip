@@ -326,24 +326,37 @@ combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_
         src[j] = (const u32x4*)(x + (int64_t)(live[j] ? row : 0) * hidden);
         scale[j] = __shfl(my_scale, j, kWave);
       }
-      for (int c = lane; c < nvec; c += kWave) {
-        u32x4 v[BATCH];
+      // eight 16-byte loads per lane in flight whatever top_k is: with two experts per token four columns of the
+      // row are worked on together (two loads at a time leave a wave waiting on memory latency most of the time)
+      constexpr int COLS = BATCH == 1 ? 1 : 8 / BATCH;   // BATCH 1: the instantiation for top_k = 1, which never gets here
+      for (int c0 = lane; c0 < nvec; c0 += kWave * COLS) {
+        u32x4 v[COLS][BATCH];
 #pragma unroll
-        for (int j = 0; j < BATCH; ++j)
-          if (live[j]) v[j] = __builtin_nontemporal_load(src[j] + c);   // expert-major rows are read once
-        float acc[EV];
+        for (int u = 0; u < COLS; ++u) {
+          const int c = c0 + u * kWave;
+          if (c >= nvec) continue;
 #pragma unroll
-        for (int i = 0; i < EV; ++i) acc[i] = 0.f;
-#pragma unroll
-        for (int j = 0; j < BATCH; ++j) {
-          if (!live[j]) continue;
-          float f[EV];
-          Vec16<DT>::unpack(v[j], f);
-#pragma unroll
-          for (int i = 0; i < EV; ++i)
-            acc[i] += weights ? Elem<DT>::to_f32(Elem<DT>::from_f32(f[i] * scale[j])) : f[i];
+          for (int j = 0; j < BATCH; ++j)
+            if (live[j]) v[u][j] = __builtin_nontemporal_load(src[j] + c);   // expert-major rows are read once
         }
-        ((u32x4*)dst)[c] = Vec16<DT>::pack(acc);
+#pragma unroll
+        for (int u = 0; u < COLS; ++u) {
+          const int c = c0 + u * kWave;
+          if (c >= nvec) continue;
+          float acc[EV];
+#pragma unroll
+          for (int i = 0; i < EV; ++i) acc[i] = 0.f;
+#pragma unroll
+          for (int j = 0; j < BATCH; ++j) {
+            if (!live[j]) continue;
+            float f[EV];
+            Vec16<DT>::unpack(v[u][j], f);
+#pragma unroll
+            for (int i = 0; i < EV; ++i)
+              acc[i] += weights ? Elem<DT>::to_f32(Elem<DT>::from_f32(f[i] * scale[j])) : f[i];
+          }
+          ((u32x4*)dst)[c] = Vec16<DT>::pack(acc);
+        }
       }
     } else if (VEC) {
       constexpr int EV = Vec16<DT>::kElems;
@@ -652,7 +665,8 @@ static int launch_combine(const void* x, int dtype, int64_t tokens, int hidden, 
   const bool vec = can_vec(dtype, hidden, x, out);
 #define CALL(DT, V)                                                                                                             \
   do {                                                                                                                          \
-    if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
+    if (top_k == 1) combine_kernel<DT, V, 1><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
+    else if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
     else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
     else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
   } while (0)
@@ -799,7 +813,8 @@ int mbx_binned_scatter(const void* x, int dtype, int64_t tokens, int hidden, int
   const bool vec = can_vec(dtype, hidden, x ? x : out, out);
 #define CALL(DT, V)                                                                                                             \
   do {                                                                                                                          \
-    if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
+    if (top_k == 1) combine_kernel<DT, V, 1><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
+    else if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
     else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
     else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
   } while (0)
