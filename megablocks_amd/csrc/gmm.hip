@@ -497,19 +497,18 @@ typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;   // 4 x 16 KiB + 3 x 32
 typedef dma::Tile<256, 256, 2, 2, 64, 2, 16> TileDma16;
 typedef dma::Tile<128, 256, 1, 4, 64, 3, 16> TileDmaSmallM16;
 
-// Which instruction the direct-to-LDS kernels multiply with.  32 x 32 x 16 unless MBX_MFMA=16 is set in the
+// Which instruction the direct-to-LDS kernels multiply with: 16 x 16 x 32 unless MBX_MFMA=32 is set in the
 // environment (read once).  On operands with random mantissas the power limit lets a loop of 16 x 16 x 32 MFMAs alone
 // run at 2.0 PFLOP/s where 32 x 32 x 16 reaches 1.76 (it moves half the accumulator registers per FLOP), and the
-// 16 x 16 x 32 kernels do hold a shader clock of 1.9 - 2.0 GHz on such operands where the others drop to 1.55 - 1.65.
-// But a wave alone on its SIMD issues one independent instruction every four cycles (eight when it depends on the
-// one before, and more where vector-ALU, LDS and scalar instructions alternate), an MFMA takes two of those slots,
-// and a 16-cycle MFMA leaves room for two more where a 32-cycle one leaves six: with 128 instead of 64 MFMAs per K
-// tile the loads, LDS reads and address arithmetic of a K tile no longer fit behind them, and the higher clock only
-// just makes up for the idle matrix-core cycles (c3 in the layer: NT +0.7 %, NN -1.4 %, TN -4 %).
+// 16 x 16 x 32 kernels hold a shader clock of 1.8 - 1.95 GHz on such operands where the others drop to 1.6 - 1.7.
+// The price is issue slots: a wave alone on its SIMD issues one independent instruction every four cycles, an MFMA
+// takes two of those slots, and a 16-cycle MFMA leaves room for two more where a 32-cycle one leaves six, so the
+// loads, LDS reads and address arithmetic of a K tile have to be dealt out one or two to a gap (block_multiply16).
+// Layer step with 16 x 16 x 32 against 32 x 32 x 16, same box, alternating runs: c3 -4.3 %, c4 -3.0 %, c2 -2.2 %.
 static inline bool use_mfma16() {
   static const bool choice = [] {
     const char* v = getenv("MBX_MFMA");
-    return v && v[0] == '1' && v[1] == '6';
+    return !(v && v[0] == '3' && v[1] == '2');
   }();
   return choice;
 }
@@ -625,12 +624,8 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   } while (0)
   if (epi != dma::kEpiNone) {
     if (layout != MBX_NT || dual || !extra) return MBX_EINVAL;
-    if constexpr (T::MF == 32) {
-      if (epi == dma::kEpiAct) MBX_LAUNCH_ROWS(false, false, dma::kEpiAct); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDact);
-      return launch_status();
-    } else {
-      return MBX_EUNSUPPORTED;
-    }
+    if (epi == dma::kEpiAct) MBX_LAUNCH_ROWS(false, false, dma::kEpiAct); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDact);
+    return launch_status();
   }
   if (layout == MBX_NT) {
     if (dual) MBX_LAUNCH_ROWS(false, true, dma::kEpiNone); else MBX_LAUNCH_ROWS(false, false, dma::kEpiNone);
@@ -779,9 +774,17 @@ static int gmm_nt_epilogue(const void* a, const void* b, void* c, void* extra, i
   if (!bins || !c || !extra || (k > 0 && (!a || !b))) return MBX_EINVAL;
   if (rows > 0x7fffffff) return MBX_ERANGE;
   const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(extra) && k > 0 &&
-                  k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n) && !use_mfma16();
+                  k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n);
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
+  if (use_mfma16()) {
+    if (half_height_only(rows, num_groups, n)) {
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+    }
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+  }
   if (half_height_only(rows, num_groups, n)) {
     if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
     return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);

@@ -449,11 +449,14 @@ __device__ __forceinline__ void mfma16_settle() { asm volatile("s_nop 15\n\ts_no
 
 // The same product with v_mfma_f32_16x16x32: two k-steps of 32 per K tile, TM x TN = 8 x 8 product tiles of 16 x 16
 // per wave (the same 128 x 128 wave tile and 256 accumulator registers; 8 + 8 operand fragments per k-step, double
-// buffered: 128 registers).  Iteration kt multiplies K tile kt and issues
-//   k-step 0: the second half of B tile kt + SB - 1 -> B stage (kt - 1) % SB, the first half of A tile kt + SB -> A stage (kt - 1) % SA
-//   barrier: every wave has both k-steps of tile kt in registers and tile kt + 1 has landed
-//   k-step 1: the second half of that A tile, the first half of B tile kt + SB -> B stage kt % SB (free since the barrier)
-// i.e. the loads in the order of the 32 x 32 x 16 schedule, one wave-wide load per eight MFMAs.
+// buffered: 128 registers).  The one barrier of a K tile sits between its two k-steps, when every wave has both
+// k-steps of tile kt in registers: B stage kt % SB is free from then on, A stage kt % SA as well.  Iteration kt issues
+//   k-step 0: A tile kt + SB -> A stage (kt - 1) % SA (free since the barrier of iteration kt - 1)
+//   barrier:  tile kt + 1 has landed
+//   k-step 1: B tile kt + SB -> B stage kt % SB, from the first gaps on
+// so that every load has at least a K tile and a half of MFMAs before the barrier that waits for it (a B load issued
+// just ahead of the barrier that needs it, as a transcription of the 32 x 32 x 16 schedule had it, stalls every K tile
+// for a memory latency).  The prologue loads tiles 0 .. SB - 1 completely.
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
 __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
   static_assert(T::MF == 16 && T::KS == 2, "two k-steps of 32 per K tile");
@@ -516,74 +519,104 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
     fb_off[0] = frag_lane_offset<false, BK, T::BN, 16>(wn);
   }
 
+  if (A_MC) {
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i) fa_off[A_MC ? i : 0] += lds_base;
+  }
+  if (B_MC) {
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) fb_off[B_MC ? j : 0] += lds_base + B_RING;
+  }
+
   u32x4 fa[2][T::TM], fb[2][T::TN];
   constexpr int NF = T::TM + T::TN, NP = T::TM * T::TN;
-#define MBX_READ_ONE16(KSTEP, BUF, A_ADDR, B_ADDR, M)                                                            \
+  constexpr int NSA = (A_MC ? 2 : 1) * T::TM, NSB = (B_MC ? 2 : 1) * T::TN, NS = NSA + NSB;   // read instructions per k-step
+  static_assert(NS <= NP, "one read per gap");
+  // A strided (MC) operand has one lane offset per fragment; adding the stage's address to it for every read would
+  // put a vector-ALU instruction right in front of every LDS read, which costs the wave eight cycles each time.  So
+  // fa_off / fb_off of such an operand hold absolute addresses in the stage that is read next, and are moved on to
+  // the following stage once per K tile (MBX_STEP16's MOVE hook), away from the reads.
+  // One read instruction per gap: a fragment of a KC operand is one ds_read_b128, one of an MC operand two
+  // transposing reads (its k values 0 .. 3 and 4 .. 7) that take a gap each.  Slot R of a k-step's NS read slots:
+#define MBX_READ_SLOT16(KSTEP, BUF, A_ADDR, B_ADDR, R)                                                           \
   do {                                                                                                           \
-    if constexpr ((M) < T::TM) {                                                                                 \
-      constexpr int i_ = (M);                                                                                    \
-      if constexpr (A_MC) fa[BUF][i_] = read_frag<true, KSTEP, 0, T::BM, 16>(A_ADDR, fa_off[A_MC ? i_ : 0]);     \
-      else fa[BUF][i_] = read_frag<false, KSTEP, i_ * KC_TILE, 256, 16>(A_ADDR, fa_off[0]);                      \
-    } else if constexpr ((M) < NF) {                                                                             \
-      constexpr int j_ = (M) - T::TM;                                                                            \
-      if constexpr (B_MC) fb[BUF][j_] = read_frag<true, KSTEP, 0, T::BN, 16>(B_ADDR, fb_off[B_MC ? j_ : 0]);     \
-      else fb[BUF][j_] = read_frag<false, KSTEP, j_ * KC_TILE, 256, 16>(B_ADDR, fb_off[0]);                      \
+    if constexpr ((R) < NSA) {                                                                                   \
+      if constexpr (A_MC) {                                                                                      \
+        constexpr int i_ = (R) / 2, h_ = (R) % 2;                                                                \
+        const u32x2 t_ = lds_read_tr16_b64<(KSTEP) * 32 * T::BM * 2 + h_ * 4 * T::BM * 2>(fa_off[A_MC ? i_ : 0]); \
+        fa[BUF][i_][2 * h_] = t_[0];                                                                             \
+        fa[BUF][i_][2 * h_ + 1] = t_[1];                                                                         \
+      } else {                                                                                                   \
+        fa[BUF][(R)] = read_frag<false, KSTEP, (R) * KC_TILE, 256, 16>(A_ADDR, fa_off[0]);                       \
+      }                                                                                                          \
+    } else if constexpr ((R) < NS) {                                                                             \
+      constexpr int r_ = (R) - NSA;                                                                              \
+      if constexpr (B_MC) {                                                                                      \
+        constexpr int j_ = r_ / 2, h_ = r_ % 2;                                                                  \
+        const u32x2 t_ = lds_read_tr16_b64<(KSTEP) * 32 * T::BN * 2 + h_ * 4 * T::BN * 2>(fb_off[B_MC ? j_ : 0]); \
+        fb[BUF][j_][2 * h_] = t_[0];                                                                             \
+        fb[BUF][j_][2 * h_ + 1] = t_[1];                                                                         \
+      } else {                                                                                                   \
+        fb[BUF][r_] = read_frag<false, KSTEP, r_ * KC_TILE, 256, 16>(B_ADDR, fb_off[0]);                         \
+      }                                                                                                          \
     }                                                                                                            \
   } while (0)
-  // One k-step: NP MFMAs of 16 cycles on register buffer CUR_BUF.  A wave issues about one instruction every four
-  // cycles, so the gap behind an MFMA has room for three more before the matrix core runs dry; everything else
-  // a k-step has to do is dealt out over the gaps accordingly:
-  //   gaps 0 .. NF - 1: the operand reads of the next k-step into the other buffer, one fragment per gap;
-  //   from gap NF on, every LEVERY-th gap: one global -> LDS load (N1 of operand G1_B at (G1_SC, G1_DST), then N2 of
-  //   operand G2_B), with the update of its running offsets in the gap behind it;
-  //   the scalar bookkeeping P0 .. P4 (at most three instructions each) in the gaps between the first loads.
-#define MBX_STEP16(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, G1_B, G1_SC, G1_DST, N1, G2_B, G2_SC, G2_DST, N2, P0, P1, P2, P3, P4)  \
+  constexpr int NMOVE = (A_MC ? T::TM : 0) + (B_MC ? T::TN : 0);
+  constexpr int MOVES_PER_GAP = NS + NMOVE > NP ? 2 : 1;
+  static_assert(NS * MOVES_PER_GAP + NMOVE <= NP * MOVES_PER_GAP, "the address updates fit behind the reads");
+  uint32_t a_delta = 0, b_delta = 0;   // from the stage read now to the next one
+#define MBX_MOVE_ONE16(M)                                                                                        \
   do {                                                                                                           \
-    constexpr int nl_ = (N1) + (N2), load0_ = NF, every_ = (NP - load0_) / nl_;                                  \
-    static_assert(every_ >= 3, "not enough MFMAs per k-step to deal the loads and the bookkeeping over");        \
+    if constexpr (A_MC && (M) < T::TM) fa_off[A_MC ? (M) : 0] += a_delta;                                        \
+    else if constexpr (B_MC && (M) - (A_MC ? T::TM : 0) >= 0 && (M) < NMOVE) fb_off[B_MC ? (M) - (A_MC ? T::TM : 0) : 0] += b_delta; \
+  } while (0)
+  // One k-step: NP MFMAs of 16 cycles on register buffer CUR_BUF.  A wave alone on its SIMD issues an independent
+  // instruction every four cycles and an MFMA takes two such slots, so the gap behind an MFMA has room for two more
+  // before the matrix core runs dry; everything else a k-step has to do is dealt out over the gaps accordingly:
+  //   gaps 0 .. NS - 1: the operand reads of the next k-step into the other buffer, one read instruction per gap;
+  //   from gap LOAD0 on, every EVERY-th gap: one of the NL global -> LDS loads of operand IS_B at (SC, DST), with the
+  //   update of its running offsets in the gap behind it;
+  //   the scalar bookkeeping P0 .. P3 (at most three instructions each) in gaps of their own.
+#define MBX_STEP16(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, IS_B, SC, DST, NL, LOAD0, EVERY, P0, P1, P2, P3, P4, MOVE)  \
+  do {                                                                                                           \
+    static_assert((EVERY) >= 3 && (LOAD0) + ((NL) - 1) * (EVERY) + 2 < NP && (LOAD0) + 3 * (EVERY) + 3 < NP && NS + 1 < NP, "the loads of a k-step and what follows them fit behind its MFMAs"); \
     wait_frags(fa[CUR_BUF], fb[CUR_BUF]);                                                                        \
     __builtin_amdgcn_sched_barrier(0);                                                                           \
     static_for<NP>([&](auto mi_) {                                                                               \
       constexpr int m_ = decltype(mi_)::value;                                                                   \
       constexpr int i_ = m_ / T::TN, j_ = (i_ & 1) ? T::TN - 1 - m_ % T::TN : m_ % T::TN;                        \
       mfma16_acc<DT>(acc[i_][j_], fb[CUR_BUF][j_], fa[CUR_BUF][i_]);                                             \
-      MBX_READ_ONE16(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                             \
-      if constexpr (m_ >= load0_ && (m_ - load0_) % every_ == 0 && (m_ - load0_) / every_ < nl_) {               \
-        constexpr int l_ = (m_ - load0_) / every_;                                                               \
-        if constexpr (l_ < (N1)) issue(G1_B, G1_SC, G1_DST, (l_ & 1) != 0);                                      \
-        else issue(G2_B, G2_SC, G2_DST, ((l_ - (N1)) & 1) != 0);                                                 \
+      MBX_READ_SLOT16(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                            \
+      if constexpr (m_ >= (LOAD0) && (m_ - (LOAD0)) % (EVERY) == 0 && (m_ - (LOAD0)) / (EVERY) < (NL))           \
+        issue(IS_B, SC, DST, (((m_ - (LOAD0)) / (EVERY)) & 1) != 0);                                             \
+      if constexpr (m_ > (LOAD0) && (m_ - (LOAD0) - 1) % (EVERY) == 0 && (m_ - (LOAD0) - 1) / (EVERY) < (NL)) {  \
+        SC += T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                                           \
+        DST += T::WAVES * 1024u;                                                                                 \
       }                                                                                                          \
-      if constexpr (m_ > load0_ && (m_ - load0_ - 1) % every_ == 0 && (m_ - load0_ - 1) / every_ < nl_) {        \
-        constexpr int l_ = (m_ - load0_ - 1) / every_;                                                           \
-        if constexpr (l_ < (N1)) {                                                                               \
-          G1_SC += T::WAVES * ((G1_B) ? b_jstep : a_jstep);                                                      \
-          G1_DST += T::WAVES * 1024u;                                                                            \
-        } else {                                                                                                 \
-          G2_SC += T::WAVES * ((G2_B) ? b_jstep : a_jstep);                                                      \
-          G2_DST += T::WAVES * 1024u;                                                                            \
-        }                                                                                                        \
+      if constexpr (m_ == (LOAD0) + 2) P0();                                                                     \
+      if constexpr (m_ == (LOAD0) + (EVERY) + 2) P1();                                                           \
+      if constexpr (m_ == (LOAD0) + 2 * (EVERY) + 2) P2();                                                       \
+      if constexpr (m_ == (LOAD0) + 3 * (EVERY) + 2) P3();                                                       \
+      if constexpr (m_ == (NS + 1 > (LOAD0) + 3 * (EVERY) + 3 ? NS + 1 : (LOAD0) + 3 * (EVERY) + 3)) P4();   /* behind the k-step's last read and P3 */ \
+      /* the strided operands' read addresses move to the next stage, one per gap, after the k-step's own reads */ \
+      if constexpr ((MOVE) && m_ >= NS && (m_ - NS) * MOVES_PER_GAP < NMOVE) {                                    \
+        MBX_MOVE_ONE16((m_ - NS) * MOVES_PER_GAP);                                                               \
+        if constexpr (MOVES_PER_GAP > 1) MBX_MOVE_ONE16((m_ - NS) * MOVES_PER_GAP + 1);                          \
       }                                                                                                          \
-      if constexpr (m_ == load0_ + 2) P0();                                                                      \
-      if constexpr (m_ == load0_ + every_ + 2) P1();                                                             \
-      if constexpr (m_ == load0_ + 2 * every_ + 2) P2();                                                         \
-      if constexpr (m_ == load0_ + 3 * every_ + 2) P3();                                                         \
-      if constexpr (every_ >= 4 && m_ == load0_ + 3) P4();                                                       \
-      if constexpr (every_ < 4 && m_ == load0_ + 3 * every_ + 3) P4();                                           \
       __builtin_amdgcn_sched_barrier(0);                                                                         \
     });                                                                                                          \
   } while (0)
 
   const int nk = g.nk;
-  constexpr int WAIT_PROLOGUE = (SB - 2) * (LA + LB) + LA + LB / 2;
-  constexpr int WAIT_LOOP = (SB - 1) * LA + (SB - 2) * LB - LA / 2;   // the second half of the newest A tile is issued after the wait
+  constexpr int WAIT_PROLOGUE = (SB - 1) * (LA + LB);        // tile 0 has landed
+  constexpr int WAIT_LOOP = (SB - 2) * (LA + LB) + LA;       // tile kt + 1 has landed: everything up to B tile kt + 1
+  static_assert(SB * (LA + LB) < 64, "vmcnt is a 6-bit counter");
   if (nk > 0) {
 #pragma unroll
-    for (int t = 0; t < SB - 1; ++t) {
+    for (int t = 0; t < SB; ++t) {
       issue_group(false, t, t, 0, LA);
       issue_group(true, t, t, 0, LB);
     }
-    issue_group(false, SB - 1, SB - 1, 0, LA);
-    issue_group(true, SB - 1, SB - 1, 0, LB / 2);
   }
   __builtin_amdgcn_sched_barrier(0);
   if (clear) {
@@ -598,63 +631,79 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
     wait_vmcnt<WAIT_PROLOGUE>();
     __builtin_amdgcn_s_barrier();
     mfma16_settle();   // the accumulators were written by vector-ALU instructions
-    static_for<NF>([&](auto mi_) { constexpr int m_ = decltype(mi_)::value; MBX_READ_ONE16(0, 0, lds_base, lds_base + B_RING, m_); });
+    static_for<NS>([&](auto mi_) { constexpr int m_ = decltype(mi_)::value; MBX_READ_SLOT16(0, 0, lds_base, lds_base + B_RING, m_); });
 
     constexpr uint32_t A_RING_END = (uint32_t)SA * T::A_BYTES, B_RING_END = B_RING + (uint32_t)SB * T::B_BYTES;
-    uint32_t a_rd = lds_base, b_rd = lds_base + B_RING, a_rd_next = 0, b_rd_next = 0;
+    // Running state, all scalar: the stages being multiplied and the next ones (one iteration ahead); LDS offset and
+    // scalar global offset of the first A load of this iteration (tile kt + SB -> stage (kt - 1) % SA) and of the
+    // first B load (tile kt + SB -> stage kt % SB).
+    uint32_t a_rd = lds_base, b_rd = lds_base + B_RING;
+    uint32_t a_rd_next = lds_base + T::A_BYTES, b_rd_next = lds_base + B_RING + T::B_BYTES;
     uint32_t a_dst0 = lds_off(false, SA - 1, 0), b_dst0 = lds_off(true, 0, 0);
     uint32_t a_sc0 = (uint32_t)SB * a_step + (uint32_t)wave * a_jstep, b_sc0 = (uint32_t)SB * b_step + (uint32_t)wave * b_jstep;
     const uint32_t a_dst_end = A_RING_END + (uint32_t)wave * 1024u, b_dst_end = B_RING_END + (uint32_t)wave * 1024u;
-    uint32_t sc_b = scalar_off(true, SB - 1, LB / 2), dst_b = lds_off(true, SB - 1, LB / 2), sc_a = 0, dst_a = 0;
-    uint32_t past = 0;
+    uint32_t past = SB < nk ? 0u : 0x80000000u;
+    uint32_t sc_a = a_sc0 | past, dst_a = a_dst0, sc_b = 0, dst_b = 0;
+    if (DUAL) ra = SB >= g.nk1 ? g.rsrc_a2 : g.rsrc_a;
+    constexpr int A_EVERY = (NP - NF - 3) / LA, B_EVERY = (NP - 4) / LB > 5 ? 5 : (NP - 4) / LB;
     for (int kt = 0; kt < nk; ++kt) {
-      // k-step 0.  Group 1: the rest of B tile kt + SB - 1 (N1 = LB / 2 loads); group 2: the first half of A tile
-      // kt + SB, whose offsets p0 / p1 set up before its first load (gap NF + N1 * LEVERY).
-      auto p0 = [&]() { past = kt + SB < nk ? 0u : 0x80000000u; };
+      // k-step 0: the A loads (offsets set up in the iteration before); p0 / p1 prepare the B loads of k-step 1,
+      // p2 moves the A offsets on to K tile kt + SB + 1
+      auto p0 = [&]() {
+        sc_b = b_sc0 | past;
+        dst_b = b_dst0;
+      };
       auto p1 = [&]() {
-        sc_a = a_sc0 | past;
-        dst_a = a_dst0;
-        if (DUAL) ra = kt + SB >= g.nk1 ? g.rsrc_a2 : g.rsrc_a;
+        if (DUAL) rb = kt + SB >= g.nk1 ? g.rsrc_b2 : g.rsrc_b;
+        b_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * b_jstep : b_sc0 + b_step;
       };
-      auto p2 = [&]() {   // the stages k-step 1 reads the next tile's first operands from
-        a_rd_next = a_rd + T::A_BYTES;
-        a_rd_next = a_rd_next >= lds_base + A_RING_END ? lds_base : a_rd_next;
-      };
-      auto p3 = [&]() {
-        b_rd_next = b_rd + T::B_BYTES;
-        b_rd_next = b_rd_next >= lds_base + B_RING_END ? lds_base + B_RING : b_rd_next;
-      };
-      auto nop = [&]() {};
-      MBX_STEP16(0, 1, a_rd, b_rd, true, sc_b, dst_b, LB / 2, false, sc_a, dst_a, LA / 2, p0, p1, p2, p3, nop);
-      wait_frags(fa[1], fb[1]);
-      wait_vmcnt<WAIT_LOOP>();
-      __builtin_amdgcn_s_barrier();
-      // k-step 1.  Group 1: the second half of that A tile; group 2: the first half of B tile kt + SB (into the
-      // stage the barrier has just freed), whose offsets q1 sets up; q0 / q2 move on to K tile kt + SB + 1.
-      auto q0 = [&]() {   // sc_a / dst_a were taken from these in k-step 0
+      auto p2 = [&]() {
         a_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * a_jstep : a_sc0 + a_step;
         a_dst0 += T::A_BYTES;
         a_dst0 = a_dst0 >= a_dst_end ? a_dst0 - A_RING_END : a_dst0;
       };
-      auto q1 = [&]() {
-        sc_b = b_sc0 | past;
-        dst_b = b_dst0;
-        if (DUAL) rb = kt + SB >= g.nk1 ? g.rsrc_b2 : g.rsrc_b;
-      };
-      auto q2 = [&]() {
-        b_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * b_jstep : b_sc0 + b_step;
+      auto nop = [&]() {};
+      auto p3 = [&]() {
         b_dst0 += T::B_BYTES;
         b_dst0 = b_dst0 >= b_dst_end ? b_dst0 - (uint32_t)SB * T::B_BYTES : b_dst0;
       };
-      MBX_STEP16(1, 0, a_rd_next, b_rd_next, false, sc_a, dst_a, LA / 2, true, sc_b, dst_b, LB / 2, q0, q1, q2, nop, nop);   // past the last tile this reads stale LDS into dead registers
-      a_rd = a_rd_next;
-      b_rd = b_rd_next;
+      a_delta = a_rd_next - a_rd;
+      b_delta = b_rd_next - b_rd;
+      MBX_STEP16(0, 1, a_rd, b_rd, false, sc_a, dst_a, LA, NF, A_EVERY, p0, p1, p2, p3, nop, true);
+      wait_frags(fa[1], fb[1]);
+      wait_vmcnt<WAIT_LOOP>();
+      __builtin_amdgcn_s_barrier();
+      // k-step 1: the B loads from the first gaps on; q0 .. q3 set up the next iteration (its A loads, the stages it
+      // reads after the ones this k-step prefetches from)
+      auto q0 = [&]() { past = kt + 1 + SB < nk ? 0u : 0x80000000u; };
+      auto q1 = [&]() {
+        sc_a = a_sc0 | past;
+        dst_a = a_dst0;
+        if (DUAL) ra = kt + 1 + SB >= g.nk1 ? g.rsrc_a2 : g.rsrc_a;
+      };
+      uint32_t a_rd_nn = 0, b_rd_nn = 0;
+      auto q2 = [&]() {
+        a_rd_nn = a_rd_next + T::A_BYTES;
+        a_rd_nn = a_rd_nn >= lds_base + A_RING_END ? lds_base : a_rd_nn;
+      };
+      auto q3 = [&]() {
+        b_rd_nn = b_rd_next + T::B_BYTES;
+        b_rd_nn = b_rd_nn >= lds_base + B_RING_END ? lds_base + B_RING : b_rd_nn;
+      };
+      auto q4 = [&]() {   // the reads of this k-step have their addresses: on to the next iteration's stages
+        a_rd = a_rd_next;
+        b_rd = b_rd_next;
+        a_rd_next = a_rd_nn;
+        b_rd_next = b_rd_nn;
+      };
+      MBX_STEP16(1, 0, a_rd_next, b_rd_next, true, sc_b, dst_b, LB, 1, B_EVERY, q0, q1, q2, q3, q4, false);   // past the last tile this reads stale LDS into dead registers
     }
     wait_vmcnt<0>();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     mfma16_settle();   // the last products must have reached the accumulators before anything else reads them
   }
-#undef MBX_READ_ONE16
+#undef MBX_READ_SLOT16
+#undef MBX_MOVE_ONE16
 #undef MBX_STEP16
 }
 

@@ -481,7 +481,7 @@ def test_fused_gated_activation_matches_the_two_step_formulation(dtype, act_name
     assert torch.equal(gated_activation(fn, odd, odd), fn(odd) * odd)
 
 
-_MFMA16_CHECK = r'''
+_OTHER_MFMA_CHECK = r'''
 import sys, torch
 sys.path.insert(0, sys.argv[1])
 from megablocks_amd import grouped_gemm_util as gg
@@ -513,15 +513,15 @@ assert worst < 1e-2, worst
 '''
 
 
-def test_gmm_on_the_16x16x32_instruction():
-    """MBX_MFMA=16 selects the main loop built on v_mfma_f32_16x16x32 (read once per process, hence the child
-    process): the three layouts and the two-pair product against fp32 torch."""
+def test_gmm_on_the_32x32x16_instruction():
+    """MBX_MFMA=32 selects the main loop built on v_mfma_f32_32x32x16 instead of the default 16x16x32 one (read once
+    per process, hence the child process): the three layouts and the two-pair product against fp32 torch."""
     import os
     import subprocess
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, MBX_MFMA='16')
-    proc = subprocess.run([sys.executable, '-c', _MFMA16_CHECK, root], env=env, capture_output=True, text=True, timeout=300)
+    env = dict(os.environ, MBX_MFMA='32')
+    proc = subprocess.run([sys.executable, '-c', _OTHER_MFMA_CHECK, root], env=env, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert 'worst' in proc.stdout
 
