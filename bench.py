@@ -384,12 +384,13 @@ def cpu_leg(args, w, inp_full):
 
     cores = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    # The whole workload where a step is a few seconds of CPU work, else half of its tokens (all experts and their
-    # full weights either way: the work per token is unchanged); --cpu-tokens overrides.
+    # The whole workload (c3, the largest default, is about 17 s per step on the 16 host threads of a GPU box, 70 s
+    # for the four steps); a workload beyond 2.5e13 FLOP per step would be cut to half of its tokens (all experts and
+    # their full weights either way: the work per token is unchanged); --cpu-tokens overrides.
     if args.cpu_tokens:
         T = args.cpu_tokens
     else:
-        T = w.tokens if w.gemm_flops() <= 4e12 else w.tokens // 2
+        T = w.tokens if w.gemm_flops() <= 2.5e13 else w.tokens // 2
     inp = inp_full if T == w.tokens else synthetic.make_inputs(w, tokens=T, seed=0)
     act = w.activation()
 

@@ -604,7 +604,11 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (rc) return rc;
     // short reductions (few rows per expert): several tiles per workgroup
     const int64_t avg_rows = rows / (num_groups > 0 ? num_groups : 1);
-    const int chunk = avg_rows >= 1024 ? 1 : avg_rows >= 512 ? 2 : 4;
+    int chunk = avg_rows >= 1024 ? 1 : avg_rows >= 512 ? 2 : 4;
+    // Reductions of a few dozen K tiles still gain from fewer workgroup launches (c3: 2 % of the launch with four
+    // tiles per workgroup), but only where an expert brings every XCD many tiles: with the six tiles per expert and
+    // XCD of a skewed c4, four to a workgroup leave most compute units idle behind the largest expert (2.4 x slower).
+    if (avg_rows >= 1024 && avg_rows < 4096 && dma::tn_tiles_per_group(tiles_m, tiles_n) / kXcds >= 64) chunk = 4;
     const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups, chunk);
     if (grid > 0x7fffffff) return MBX_ERANGE;
     kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, chunk, (int)seg_rows);

@@ -1185,7 +1185,8 @@ static inline int64_t tn_tiles_per_group(int tiles_m, int tiles_n) {
 }
 static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chunk) {
   const int64_t per_xcd = (tn_tiles_per_group(tiles_m, tiles_n) + kXcds - 1) / kXcds;
-  return (per_xcd * num_groups + chunk - 1) / chunk * kXcds;
+  const int64_t span = (int64_t)32 * chunk;   // list entries covered by 32 workgroups of an XCD
+  return (per_xcd * num_groups + span - 1) / span * 32 * kXcds;
 }
 
 // One output tile of expert e's product: rows [g.a_r0, g.a_r0 + TT::BM) x columns [g.b_r0, g.b_r0 + TT::BN) of
@@ -1258,8 +1259,12 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
   g.a_ld_bytes = (uint32_t)k * 2;
   g.b_ld_bytes = (uint32_t)n * 2;
   const int64_t items = (int64_t)per_xcd * num_groups;   // per XCD
-  const int64_t first = (int64_t)(blockIdx.x / kXcds) * chunk;
-  for (int64_t i = first; i < first + chunk && i < items; ++i) {
+  // A workgroup's `chunk` tiles are 32 apart in its XCD's list: the 32 workgroups an XCD runs at a time are then on 32
+  // consecutive tiles (one 8 x 4 block, 12 operand panels) for each of their tiles in turn; with consecutive tiles per
+  // workgroup they would be spread over `chunk` blocks at once.
+  const int64_t member = blockIdx.x / kXcds;
+  const int64_t first = (member / 32) * 32 * chunk + member % 32;
+  for (int64_t i = first; i < first + (int64_t)32 * chunk && i < items; i += 32) {
     const int slot = (int)(i / per_xcd);                  // position of the expert in the longest-first order
     const int t = ((xcd + slot) % kXcds) * per_xcd + (int)(i % per_xcd);     // tile slot inside the expert
     if (t >= per_group) continue;
