@@ -611,7 +611,9 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (avg_rows >= 1024 && avg_rows < 4096 && dma::tn_tiles_per_group(tiles_m, tiles_n) / kXcds >= 64) chunk = 4;
     const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups, chunk);
     if (grid > 0x7fffffff) return MBX_ERANGE;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, chunk, (int)seg_rows);
+    // whole experts per XCD (if the kernel finds them balanced): for reductions of a few K tiles only
+    const int whole_ok = avg_rows < 1024 ? 1 : 0;
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, chunk, (int)seg_rows, whole_ok);
     return launch_status();
   }
   constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;

@@ -335,6 +335,31 @@ def test_gmm_tn_last_row_of_tiles(gg, k, n):
     assert bool((guard[:2048] == 3.0).all()) and bool((guard[2048 + ref.numel():] == 3.0).all())
 
 
+# Short reductions whose experts load the XCDs alike are dealt to XCDs as whole experts (the kernel decides from the
+# row counts): equal experts, equal experts next to empty ones, a count that is no multiple of eight (never balanced:
+# an eighth of every expert per XCD, as for long reductions), nearly equal ones, and one XCD's worth of experts.
+WHOLE_EXPERTS = [[200] * 16, [256, 0] * 8, [320] * 12, [250 + (7 * i) % 13 for i in range(64)], [192] * 8, [64] * 40 + [0] * 24]
+
+
+@pytest.mark.parametrize('rows_per_expert', WHOLE_EXPERTS, ids=lambda r: f'{len(r)}x{r[0]}')
+@pytest.mark.parametrize('k,n', [(1024, 512), (264, 1032), (128, 256)])
+def test_gmm_tn_short_reductions_dealt_by_expert(gg, rows_per_expert, k, n):
+    sizes = torch.tensor(rows_per_expert)
+    rows = int(sizes.sum())
+    torch.manual_seed(rows + k)
+    a = torch.randn(rows, k, device='cuda').bfloat16()
+    b = torch.randn(rows, n, device='cuda').bfloat16()
+    ref = _ref_gpu(a, b, sizes, True, False)
+    guard = torch.full((ref.numel() + 4096,), 3.0, device='cuda').bfloat16()
+    c = guard[2048:2048 + ref.numel()].view(ref.shape)
+    got = gg.backend.gmm(a, b, sizes.cuda(), trans_a=True, c=c)
+    assert rel_err(got, ref) < TOL and max_block_err(got, ref) < 2 * TOL
+    for e, r in enumerate(rows_per_expert):
+        if r == 0:
+            assert torch.count_nonzero(got[e]) == 0
+    assert bool((guard[:2048] == 3.0).all()) and bool((guard[2048 + ref.numel():] == 3.0).all())
+
+
 def _random_shapes(count, seed):
     g = torch.Generator().manual_seed(seed)
     r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
