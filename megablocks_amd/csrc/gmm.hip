@@ -608,12 +608,13 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     // Reductions of a few dozen K tiles still gain from fewer workgroup launches (c3: 2 % of the launch with four
     // tiles per workgroup), but only where an expert brings every XCD many tiles: with the six tiles per expert and
     // XCD of a skewed c4, four to a workgroup leave most compute units idle behind the largest expert (2.4 x slower).
-    if (avg_rows >= 1024 && avg_rows < 4096 && dma::tn_tiles_per_group(tiles_m, tiles_n) / kXcds >= 64) chunk = 4;
-    const int64_t grid = dma::tn_grid(tiles_m, tiles_n, num_groups, chunk);
+    const dma::TnBlocks shape = dma::tn_block_shape(tiles_m, tiles_n);
+    if (avg_rows >= 1024 && avg_rows < 4096 && dma::tn_tiles_per_group(tiles_m, tiles_n, shape) / kXcds >= 64) chunk = 4;
+    const int64_t grid = dma::tn_grid(tiles_m, tiles_n, shape, num_groups, chunk);
     if (grid > 0x7fffffff) return MBX_ERANGE;
     // whole experts per XCD (if the kernel finds them balanced): for reductions of a few K tiles only
     const int whole_ok = avg_rows < 1024 ? 1 : 0;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, chunk, (int)seg_rows, whole_ok);
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, shape.bm, shape.bn, chunk, (int)seg_rows, whole_ok);
     return launch_status();
   }
   constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;

@@ -1179,14 +1179,49 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
 constexpr int kTnBlockM = 8, kTnBlockN = 4;
 // XCD of the expert with rank r (0 = most rows) when whole experts are dealt to XCDs: 0 .. 7, 7 .. 0, 0 .. 7, ...
 __host__ __device__ static inline int serpentine_xcd(int r) { return ((r / kXcds) & 1) ? kXcds - 1 - r % kXcds : r % kXcds; }
-__host__ __device__ static inline int tn_block_m(int tiles_m) { return tiles_m < kTnBlockM ? (tiles_m > 0 ? tiles_m : 1) : kTnBlockM; }
-__host__ __device__ static inline int tn_block_n(int tiles_n) { return tiles_n < kTnBlockN ? (tiles_n > 0 ? tiles_n : 1) : kTnBlockN; }
-static inline int64_t tn_tiles_per_group(int tiles_m, int tiles_n) {
-  const int bm = tn_block_m(tiles_m), bn = tn_block_n(tiles_n);
-  return (int64_t)((tiles_m + bm - 1) / bm) * ((tiles_n + bn - 1) / bn) * (bm * bn);
+// The block shape of a launch: 8 x 4 when an XCD's eighth of an expert is at least a block (32 tiles); for smaller
+// products the shape whose eighths are most compact, so that the workgroups of an XCD, which work on the eighths of
+// several experts at a time, fetch few operand panels per tile (a [1408, 2048] product, 6 x 8 tiles: eighths of 3 x 2
+// tiles with 5 panels each instead of 6 x 1 with 7).  Chosen by trying every shape: first the fewest tiles in the
+// fullest eighth (the XCDs' balance), then the fewest panels over the eight.
+struct TnBlocks { int bm, bn; };
+static inline int64_t tn_tiles_per_group(int tiles_m, int tiles_n, TnBlocks s) {
+  return (int64_t)((tiles_m + s.bm - 1) / s.bm) * ((tiles_n + s.bn - 1) / s.bn) * (s.bm * s.bn);
 }
-static inline int64_t tn_grid(int tiles_m, int tiles_n, int num_groups, int chunk) {
-  const int64_t per_group = tn_tiles_per_group(tiles_m, tiles_n);
+static inline TnBlocks tn_block_shape(int tiles_m, int tiles_n) {
+  TnBlocks best{tiles_m < kTnBlockM ? (tiles_m > 0 ? tiles_m : 1) : kTnBlockM, tiles_n < kTnBlockN ? (tiles_n > 0 ? tiles_n : 1) : kTnBlockN};
+  const int64_t raw = (int64_t)tiles_m * tiles_n;
+  if (raw >= (int64_t)kXcds * kTnBlockM * kTnBlockN || raw <= kXcds) return best;
+  int64_t best_fullest = -1, best_panels = -1;
+  for (int bm = 1; bm <= kTnBlockM && bm <= tiles_m; ++bm) {
+    for (int bn = 1; bn <= kTnBlockM && bn <= tiles_n; ++bn) {
+      if (bm * bn > kTnBlockM * kTnBlockN) continue;
+      const TnBlocks s{bm, bn};
+      const int blocks_m = (tiles_m + bm - 1) / bm;
+      const int per_group = (int)tn_tiles_per_group(tiles_m, tiles_n, s), per_xcd = (per_group + kXcds - 1) / kXcds;
+      int64_t fullest = 0, panels = 0;
+      for (int piece = 0; piece < kXcds; ++piece) {
+        bool row_seen[256] = {}, col_seen[256] = {};   // raw < 256: fewer than 256 tiles in either direction
+        int64_t tiles = 0;
+        for (int t = piece * per_xcd; t < (piece + 1) * per_xcd && t < per_group; ++t) {
+          const int blk = t / (bm * bn), in = t % (bm * bn);
+          const int tm = (blk % blocks_m) * bm + in % bm, tn = (blk / blocks_m) * bn + in / bm;
+          if (tm >= tiles_m || tn >= tiles_n) continue;
+          ++tiles;
+          if (!row_seen[tm]) { row_seen[tm] = true; ++panels; }
+          if (!col_seen[tn]) { col_seen[tn] = true; ++panels; }
+        }
+        fullest = tiles > fullest ? tiles : fullest;
+      }
+      if (best_fullest < 0 || fullest < best_fullest || (fullest == best_fullest && panels < best_panels)) {
+        best_fullest = fullest; best_panels = panels; best = s;
+      }
+    }
+  }
+  return best;
+}
+static inline int64_t tn_grid(int tiles_m, int tiles_n, TnBlocks shape, int num_groups, int chunk) {
+  const int64_t per_group = tn_tiles_per_group(tiles_m, tiles_n, shape);
   const int64_t per_xcd = (per_group + kXcds - 1) / kXcds;
   const int64_t span = (int64_t)32 * chunk;   // list entries covered by 32 workgroups of an XCD
   // entries of an XCD's list: a piece of every expert, or every tile of its share of the experts (the kernel decides)
@@ -1236,11 +1271,10 @@ template <int DT, typename T, typename TS, bool SEGMENTED>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int rows, int k, int n, int tiles_m, int tiles_n,
-              int chunk, int seg_rows, int whole_ok) {
+              int bm, int bn, int chunk, int seg_rows, int whole_ok) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "last-row tile");
   constexpr bool kMixed = T::BM != TS::BM;
-  const int bm = tn_block_m(tiles_m), bn = tn_block_n(tiles_n);
   const int blocks_m = (tiles_m + bm - 1) / bm, blocks_n = (tiles_n + bn - 1) / bn;
   const int per_group = blocks_m * blocks_n * (bm * bn);
   const int per_xcd = (per_group + kXcds - 1) / kXcds;
