@@ -1005,28 +1005,36 @@ __device__ __forceinline__ int clamp_row(int v, int rows) { return v < 0 ? 0 : (
 // search through the bins of that lane's group.
 template <int BM>
 struct RowTiles {
-  int lane_start = 0, lane_end = 0, lane_mt = 0, lane_incl = 0;
-  int total = 0;
-  int per_lane;            // experts per lane: 1 up to 64 experts (the lane then keeps its expert's row range too)
+  // Per lane: one expert up to 64 experts (the lane then keeps its row range too), else a group of per_lane experts.
+  int lane_start = 0, lane_end = 0, lane_mt = 0, lane_incl = 0, lane_short_incl = 0;
+  int total = 0, total_short = 0;   // all tiles; of these, the short last row tiles that come first in the order
+  int per_lane;
   const int32_t* bins;
   int num_groups, tiles_n, rows;
+  bool split;              // short last row tiles (at most BM / 2 rows) may be listed apart, ahead of the others
 
-  static __device__ __forceinline__ int row_tiles(int rows) { return rows > 0 ? (rows + BM - 1) / BM : 0; }
+  // row tiles of an expert that are listed with the full ones, and whether a short one is left over
+  int apart_from;          // full row tiles an expert must have for its short last tile to be listed apart
+  __device__ __forceinline__ int short_tiles(int r) const {
+    return split && r > 0 && r % BM > 0 && r % BM <= BM / 2 && r / BM >= apart_from ? 1 : 0;
+  }
+  __device__ __forceinline__ int long_tiles(int r) const { return r <= 0 ? 0 : (r + BM - 1) / BM - short_tiles(r); }
   // A bin bound as the kernels use it: inside [0, rows] whatever the table holds, so that a table that does not
   // belong to this operand (stale, or of another batch) can make the result wrong but never an access out of range.
   __device__ __forceinline__ int bound(int e) const { return clamp_row(bins[e], rows); }
 
-  __device__ __forceinline__ RowTiles(const int32_t* bins_, int num_groups_, int tiles_n_, int rows_)
-      : bins(bins_), num_groups(num_groups_), tiles_n(tiles_n_), rows(rows_) {
+  __device__ __forceinline__ RowTiles(const int32_t* bins_, int num_groups_, int tiles_n_, int rows_, bool split_, int apart_from_)
+      : bins(bins_), num_groups(num_groups_), tiles_n(tiles_n_), rows(rows_), split(split_), apart_from(apart_from_) {
     per_lane = (num_groups + kWave - 1) / kWave;
     const int lane = lane_id();
     const int first = lane * per_lane;
-    int span = 0;
+    int span = 0, shorts = 0;
     if (per_lane == 1) {
       if (lane < num_groups) {
         lane_end = bound(lane);
         lane_start = lane > 0 ? bound(lane - 1) : 0;
-        lane_mt = row_tiles(lane_end - lane_start);
+        lane_mt = long_tiles(lane_end - lane_start);
+        shorts = short_tiles(lane_end - lane_start);
       }
       span = lane_mt * tiles_n;
     } else if (first < num_groups) {
@@ -1035,23 +1043,57 @@ struct RowTiles {
       int start = lane_start;
       for (int e = first; e < first + per_lane && e < num_groups; ++e) {
         const int end = bound(e);
-        span += row_tiles(end - start) * tiles_n;
+        span += long_tiles(end - start) * tiles_n;
+        shorts += short_tiles(end - start);
         start = end;
       }
       lane_mt = span;
     }
-    int incl = span;
+    int incl = span, sincl = shorts;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
-      const int v = __shfl_up(incl, o, kWave);
-      if (lane >= o) incl += v;
+      const int v = __shfl_up(incl, o, kWave), w = __shfl_up(sincl, o, kWave);
+      if (lane >= o) { incl += v; sincl += w; }
     }
     lane_incl = incl;
-    total = __builtin_amdgcn_readlane(incl, kWave - 1);
+    lane_short_incl = sincl;
+    total_short = __builtin_amdgcn_readlane(sincl, kWave - 1) * tiles_n;
+    total = __builtin_amdgcn_readlane(incl, kWave - 1) + total_short;
   }
 
   // id in [0, total) -> expert, its row range, the row tile and the column tile
   __device__ __forceinline__ void find(int id, int& e, int& start, int& end, int& tm, int& tn) const {
+    if (id < total_short) {
+      // The short last row tiles that are listed apart, expert by expert, column tiles fastest.  A short tile takes
+      // less time than a full one; dealt among the full ones it lets the workgroups of an XCD drift apart, which then
+      // no longer find each other's operand panels in the L2.  Apart, the short tile streams its expert's weights on
+      // its own, so this is only done for experts with many row tiles (apart_from) and by the launches whose long
+      // reductions suffer most from the drift (NN on a Mixtral-shaped layer: L2 misses 4.8 -> 4.0 GB, launch -3 %;
+      // NT, with a quarter of the reduction length, was 1.5 % slower apart, and experts of one or two row tiles, which
+      // are bound by the weights they stream, 18 %).
+      const int j = id / tiles_n;
+      tn = id - j * tiles_n;
+      const uint64_t hit = __ballot(j < lane_short_incl);
+      const int l = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
+      if (per_lane == 1) {
+        e = l;
+        start = __builtin_amdgcn_readlane(lane_start, l);
+        end = __builtin_amdgcn_readlane(lane_end, l);
+      } else {
+        // the j-th short tile overall is number `want` among those of lane l's experts
+        int want = j - (l > 0 ? __builtin_amdgcn_readlane(lane_short_incl, l > 0 ? l - 1 : 0) : 0);
+        start = __builtin_amdgcn_readlane(lane_start, l);
+        end = start;
+        for (e = l * per_lane; e < num_groups; ++e) {
+          end = bound(e);
+          if (short_tiles(end - start) && want-- == 0) break;
+          start = end;
+        }
+      }
+      tm = long_tiles(end - start);
+      return;
+    }
+    id -= total_short;
     int mt;
     const uint64_t hit = __ballot(id < lane_incl);
     const int l = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
@@ -1068,7 +1110,7 @@ struct RowTiles {
       end = start; mt = 0;
       for (e = l * per_lane; e < num_groups; ++e) {
         end = bound(e);
-        mt = row_tiles(end - start);
+        mt = long_tiles(end - start);
         const int span = mt * tiles_n;
         if (id < span) break;
         id -= span;
@@ -1113,7 +1155,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   static_assert(!kSplit || T::BM == 2 * TS::BM, "tail tile");
   const int P = gridDim.x, run = P / kXcds;
   const int xcd = blockIdx.x % kXcds, member = blockIdx.x / kXcds;
-  const RowTiles<T::BM> tiles(bins, num_groups, tiles_n, (int)rows);
+  const RowTiles<T::BM> tiles(bins, num_groups, tiles_n, (int)rows, kSplit && B_MC, 8);
   const int total = tiles.total;
   const int full_rounds = total / P, rest = total - full_rounds * P;
   const bool split = kSplit && rest > 0 && 2 * rest <= P;

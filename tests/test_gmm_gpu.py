@@ -295,6 +295,8 @@ MIXED_ROWS = [  # per-expert row counts around the boundaries between full (256-
     [300] * 48,                       # full and half-height tiles alternate along the tile list, several rounds
     [260, 250] * 40,                  # more than 64 experts
     [130] * 64,                       # on average below the full tile: half-height tiles only
+    [2048 + 37 * (i % 5) for i in range(8)] + [100, 2100, 0, 385],     # many full tiles, a few short last ones
+    [(300, 0, 700, 256, 40)[i % 5] for i in range(150)],             # short last tiles with several experts per lane
 ]
 
 
