@@ -215,6 +215,18 @@ int mbx_gmm_act(const void* a, const void* b, void* c, void* c_act, int dtype, c
 int mbx_gmm_dact(const void* a, const void* b, const void* pre, void* c, int dtype, const int32_t* bins,
                  int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
 
+/* The backward of the GLU experts' gated activation on the product that feeds it, megablocks/layers/glu.py:135-153
+ * (`gmm(ddsd_out, w2, trans_b=True, c=dactivation_fn_out)`, then autograd's gradient of
+ * `activation_fn(sdd_out) * v1_out`, glu.py:120-124), in one launch:
+ *   g = round(a[r_e] @ b[e]^T)        (a = ddsd_out, b = w2 as [E, n, k]: `gmm(ddsd_out, w2, trans_b=True)`)
+ *   d1 = round(g * x2) * act'(x1)     (the gradient of sdd_out;  x1 = sdd_out, x2 = v1_out, all [rows, n])
+ *   d2 = g * round(act(x1))           (the gradient of v1_out)
+ * with the roundings of the separate steps; g itself is not stored.  act: MBX_ACT_SILU or MBX_ACT_GELU_TANH.
+ * MBX_EUNSUPPORTED (the caller runs mbx_gmm and mbx_glu_backward): the cases of mbx_gmm_act, and the 32 x 32 x 16
+ * main loop. */
+int mbx_gmm_dglu(const void* a, const void* b, const void* x1, const void* x2, void* d1, void* d2, int dtype,
+                 const int32_t* bins, int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
+
 /* megablocks/layers/gelu.py:9-13 `_gelu_backward_inplace(g, x)`: g *= d/dx gelu_tanh(x). */
 int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel,
                               mbx_stream_t stream);

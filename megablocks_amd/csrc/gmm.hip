@@ -583,12 +583,12 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
 template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
             int layout, hipStream_t s, const void* a2 = nullptr, const void* b2 = nullptr, int epi = dma::kEpiNone,
-            void* extra = nullptr) {
+            void* extra = nullptr, void* out2 = nullptr) {
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
   const uint16_t* ap2 = (const uint16_t*)a2;
   const uint16_t* bp2 = (const uint16_t*)b2;
-  const bool dual = a2 != nullptr;
+  const bool dual = a2 != nullptr && !dma::epi_is_dglu(epi);
   uint16_t* cp = (uint16_t*)c;
   if (layout == MBX_TN) {
     constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
@@ -627,8 +627,18 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL, EPI>;                                     \
     int rc = allow_lds(kern, lds);                                                                    \
     if (rc) return rc;                                                                                \
-    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra);  \
+    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2);  \
   } while (0)
+  if (dma::epi_is_dglu(epi)) {
+    // a2 carries x2 of the gated activation (not a second operand pair); only the 16 x 16 x 32 tiles are instantiated
+    if (layout != MBX_NT || !extra || !a2 || !out2) return MBX_EINVAL;
+    if constexpr (T::MF == 16) {
+      if (epi == dma::kEpiDgluSilu) MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluSilu); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluGelu);
+      return launch_status();
+    } else {
+      return MBX_EUNSUPPORTED;
+    }
+  }
   if (epi != dma::kEpiNone) {
     if (layout != MBX_NT || dual || !extra) return MBX_EINVAL;
     if (epi == dma::kEpiAct) MBX_LAUNCH_ROWS(false, false, dma::kEpiAct); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDact);
@@ -772,26 +782,30 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
 
 // The NT product with an activation epilogue (epi: dma::kEpiAct / dma::kEpiDact), for the shapes the direct-to-LDS
 // kernels take; anything else is MBX_EUNSUPPORTED and the caller runs the product and the element-wise pass.
+// (kEpiDglu*: pre2 = x2, out2 = the second output; 16 x 16 x 32 main loop only.)
 static int gmm_nt_epilogue(const void* a, const void* b, void* c, void* extra, int dtype, const int32_t* bins, int num_groups,
-                           int64_t rows, int k, int n, int act, int epi, mbx_stream_t stream) {
+                           int64_t rows, int k, int n, int act, int epi, mbx_stream_t stream, const void* pre2 = nullptr,
+                           void* out2 = nullptr) {
   if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
-  if (act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
+  const bool dglu = dma::epi_is_dglu(epi);
+  if (!dglu && act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
   if (num_groups == 0 || rows == 0 || n == 0) return 0;
-  if (!bins || !c || !extra || (k > 0 && (!a || !b))) return MBX_EINVAL;
+  if (!bins || !c || !extra || (k > 0 && (!a || !b)) || (dglu && (!pre2 || !out2))) return MBX_EINVAL;
   if (rows > 0x7fffffff) return MBX_ERANGE;
   const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(extra) && k > 0 &&
-                  k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n);
+                  k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n) && (!dglu || (aligned16(pre2) && aligned16(out2)));
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   if (use_mfma16()) {
     if (half_height_only(rows, num_groups, n)) {
-      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
-      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
+      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
     }
-    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
-    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
+    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
   }
+  if (dglu) return MBX_EUNSUPPORTED;
   if (half_height_only(rows, num_groups, n)) {
     if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
     return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
@@ -808,6 +822,13 @@ int mbx_gmm_act(const void* a, const void* b, void* c, void* c_act, int dtype, c
 int mbx_gmm_dact(const void* a, const void* b, const void* pre, void* c, int dtype, const int32_t* bins, int num_groups,
                  int64_t rows, int k, int n, int act, mbx_stream_t stream) {
   return gmm_nt_epilogue(a, b, c, (void*)pre, dtype, bins, num_groups, rows, k, n, act, dma::kEpiDact, stream);
+}
+
+int mbx_gmm_dglu(const void* a, const void* b, const void* x1, const void* x2, void* d1, void* d2, int dtype,
+                 const int32_t* bins, int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream) {
+  if (act != MBX_ACT_SILU && act != MBX_ACT_GELU_TANH) return MBX_EINVAL;
+  return gmm_nt_epilogue(a, b, d1, (void*)x1, dtype, bins, num_groups, rows, k, n, act,
+                         act == MBX_ACT_SILU ? dma::kEpiDgluSilu : dma::kEpiDgluGelu, stream, x2, d2);
 }
 
 int mbx_gelu_backward_inplace(void* g, const void* x, int dtype, int64_t numel, mbx_stream_t stream) {

@@ -760,10 +760,14 @@ __device__ __forceinline__ void gelu_tanh_bwd8(float (&g)[8], const float (&x)[8
 }
 
 // What the store of an output tile does besides storing it:
-//   kEpiNone  nothing;
-//   kEpiAct   also stores gelu_tanh of the (rounded) tile to a second output of the same shape;
-//   kEpiDact  multiplies the (rounded) tile by d/dx gelu_tanh of a second input of the same shape before storing it.
-enum { kEpiNone = 0, kEpiAct = 1, kEpiDact = 2 };
+//   kEpiNone      nothing;
+//   kEpiAct       also stores gelu_tanh of the (rounded) tile to a second output of the same shape;
+//   kEpiDact      multiplies the (rounded) tile by d/dx gelu_tanh of a second input of the same shape before storing it;
+//   kEpiDgluSilu, kEpiDgluGelu   the tile g is the gradient of act(x1) * x2 (act = SiLU / tanh-GELU) with x1, x2 two
+//                 more inputs of the same shape: stores g * round(act(x1)) and round(g * x2) * act'(x1), two outputs,
+//                 and not g itself.
+enum { kEpiNone = 0, kEpiAct = 1, kEpiDact = 2, kEpiDgluSilu = 3, kEpiDgluGelu = 4 };
+constexpr bool epi_is_dglu(int epi) { return epi == kEpiDgluSilu || epi == kEpiDgluGelu; }
 
 // the eight 16-bit values of a 16-byte chunk as fp32 and back (rounded)
 template <int DT>
@@ -782,6 +786,54 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
   for (int w = 0; w < 4; ++w) r[w] = pack2<DT>(f[2 * w], f[2 * w + 1]);
   return r;
 }
+// The backward of the gated activation act(x1) * x2 on a chunk, with the roundings autograd's separate steps make:
+//   d2 = g * round(act(x1)),   d1 = round(g * x2) * act'(x1)
+// where act(x) = x s and act'(x) = s (1 + x (1 - s) q): SiLU with s = sigmoid(x), q = 1; tanh-GELU with s = sigmoid(2u)
+// and q = 1.59576912 + 0.2140644486 x^2 (see gelu_tanh_bwd8).
+template <int DT, bool GELU>
+__device__ __forceinline__ void dglu_chunk(const u32x4& gv, const u32x4& x1v, const u32x4& x2v, u32x4& d1v, u32x4& d2v) {
+  float g[8], x[8], b[8], s[8], q[8], z[8];
+  unpack8<DT>(gv, g);
+  unpack8<DT>(x1v, x);
+  unpack8<DT>(x2v, b);
+  if (GELU) {
+    sigmoid_2u8(x, z, s);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = 0.2140644486f * z[i] + 1.59576912f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = -1.44269504f * x[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = __builtin_amdgcn_exp2f(z[i]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = 1.f + z[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] = __builtin_amdgcn_rcpf(z[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = x[i] * s[i];                                   // act(x1)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) b[i] = g[i] * b[i];                                   // g x2
+  const u32x4 actv = pack8<DT>(z), gbv = pack8<DT>(b);                              // both rounded to the storage type
+  unpack8<DT>(actv, z);
+  unpack8<DT>(gbv, b);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) g[i] = g[i] * z[i];                                   // d2
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = 1.f - s[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = x[i] * z[i];
+  if (GELU) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = z[i] * q[i];
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = s[i] * z[i] + s[i];                            // act'(x1)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) b[i] = b[i] * z[i];                                   // d1
+  d1v = pack8<DT>(b);
+  d2v = pack8<DT>(g);
+}
 template <int DT>
 __device__ __forceinline__ u32x4 gelu_fwd_chunk(const u32x4& v) {
   float x[8];
@@ -798,14 +850,26 @@ __device__ __forceinline__ u32x4 gelu_bwd_chunk(const u32x4& gv, const u32x4& xv
   return pack8<DT>(g);
 }
 
+// Buffer sizes stay below 2 GiB: bit 31 of a byte offset marks a load that must fetch nothing.
+__device__ __forceinline__ uint32_t clip_bytes(int64_t bytes) {
+  return (uint32_t)(bytes < 0x7fffffff ? bytes : 0x7fffffff);
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
+}
+
 // c[m][n] = acc for m < m_lim, n < n_lim, where m = m_base + (row inside the tile) and
 // n = n_base + (column inside the tile).  Uses the LDS of the operand rings as a staging buffer.
 // `extra` (EPI != kEpiNone; laid out like c, same pitch, 16-byte aligned like c): the second output of kEpiAct, the
-// second input of kEpiDact.  Those two take the staged path only (the launch checks pitch and alignment).
+// second input of kEpiDact, x1 of kEpiDglu*; `pre2` and `out2` (kEpiDglu* only, laid out alike): x2 and the second
+// output (c gets round(g x2) act'(x1), out2 gets g round(act(x1))).  These take the staged path only (the launch
+// checks pitch and alignment).
 template <int DT, typename T, int EPI = kEpiNone>
 __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][T::TN], uint16_t* __restrict__ c, int64_t ldc,
                                             int m_base, int m_lim, int n_base, int n_lim, char* lds_generic,
-                                            uint16_t* __restrict__ extra = nullptr) {
+                                            uint16_t* __restrict__ extra = nullptr, const uint16_t* __restrict__ pre2 = nullptr,
+                                            uint16_t* __restrict__ out2 = nullptr) {
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
@@ -849,7 +913,8 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
     // instruction issue: a tile that is complete in the column direction takes a path with a 32-bit
     // running byte offset and nothing but the row check around each store.  Those stores are
     // non-temporal: the output is not read again by this kernel and need not displace operand panels.
-    constexpr int ITERS = T::BM / ROWS_PER_INSTR / T::WAVES, BATCH = 8;
+    constexpr bool kDglu = epi_is_dglu(EPI), kPre = EPI == kEpiDact || kDglu;
+    constexpr int ITERS = T::BM / ROWS_PER_INSTR / T::WAVES, BATCH = kDglu ? 4 : 8;
     constexpr int ROW_STEP = T::WAVES * ROWS_PER_INSTR;   // rows between consecutive stores of a wave
     static_assert(ITERS % BATCH == 0, "store batches");
     const uint32_t rd_addr = lds_base + (uint32_t)((wave * ROWS_PER_INSTR + rl) * ROW + ch * 16);
@@ -859,74 +924,98 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
     const uint32_t off_step = (uint32_t)ROW_STEP * (uint32_t)ldc * 2u;
     char* const cb = (char*)c;
     char* const eb = (char*)extra;
+    const char* const pb = (const char*)pre2;
+    char* const ob = (char*)out2;
     // kEpiDact: the chunks of the second input that belong to a batch are fetched one batch ahead (the registers of
     // the accumulators are free by now), so that their latency is behind the arithmetic and the stores of the batch
     // before; rows or columns outside the tile's part of c are not fetched (zeros: their results are not stored)
-    u32x4 pre[EPI == kEpiDact ? BATCH : 1], pre_next[EPI == kEpiDact ? BATCH : 1];
-    auto fetch_pre = [&](u32x4 (&dst)[EPI == kEpiDact ? BATCH : 1], int m0, uint32_t off0) {
-      if constexpr (EPI == kEpiDact) {
+    // (kEpiDglu*: both inputs, in batches of four, two batches ahead: a batch of four takes less time than a fetch)
+    u32x4 pre[kPre ? BATCH : 1], pre_next[kPre ? BATCH : 1], preb[kDglu ? BATCH : 1], preb_next[kDglu ? BATCH : 1];
+    u32x4 pre_far[kDglu ? BATCH : 1], preb_far[kDglu ? BATCH : 1];
+    // Buffer loads, bounded by the rows this tile may touch: no branch around a load, so the compiler can count the
+    // loads in flight (around conditional loads it waits for all of them, the ones fetched ahead included); rows past
+    // the end read as zeros, columns past it as whatever follows in the row below — neither is stored.
+    const __amdgpu_buffer_rsrc_t pre_rsrc = make_rsrc(kPre ? eb : nullptr, kPre && m_lim > 0 ? clip_bytes((int64_t)m_lim * ldc * 2) : 0u);
+    const __amdgpu_buffer_rsrc_t preb_rsrc = make_rsrc(kDglu ? pb : nullptr, kDglu && m_lim > 0 ? clip_bytes((int64_t)m_lim * ldc * 2) : 0u);
+    auto fetch_pre = [&](u32x4 (&dst)[kPre ? BATCH : 1], const __amdgpu_buffer_rsrc_t& r, uint32_t off0) {
+      if constexpr (kPre) {
 #pragma unroll
-        for (int u = 0; u < BATCH; ++u) {
-          const u32x4 zero = {0u, 0u, 0u, 0u};
-          dst[u] = zero;
-          if (m0 + u * ROW_STEP < m_lim && n < n_lim) {
-            const uint16_t* src = (const uint16_t*)(eb + (off0 + (uint32_t)u * off_step));
-            if (n + 8 <= n_lim) {
-              dst[u] = __builtin_nontemporal_load((const u32x4*)src);
-            } else {
-#pragma unroll
-              for (int t = 0; t < 8; ++t)
-                if (n + t < n_lim) dst[u][t >> 1] |= (uint32_t)src[t] << ((t & 1) * 16);
-            }
-          }
-        }
+        for (int u = 0; u < BATCH; ++u)
+          dst[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(off0 + (uint32_t)u * off_step), 0, 0));
       }
     };
-    fetch_pre(pre_next, m, off);
+    fetch_pre(pre_next, pre_rsrc, off);
+    if constexpr (kDglu) {
+      fetch_pre(preb_next, preb_rsrc, off);
+      fetch_pre(pre_far, pre_rsrc, off + BATCH * off_step);
+      fetch_pre(preb_far, preb_rsrc, off + BATCH * off_step);
+    }
+    // the second output goes where kEpiAct's does (extra) or to out2 (kEpiDglu*: extra is an input there)
+    constexpr bool kTwoOut = EPI == kEpiAct || kDglu;
+    char* const second = kDglu ? ob : eb;
 #pragma unroll 1
     for (int b = 0; b < ITERS; b += BATCH) {
-      u32x4 v[BATCH];
+      u32x4 v[BATCH], y[kTwoOut ? BATCH : 1];
       static_for<BATCH>([&](auto ui) {
         constexpr int u = decltype(ui)::value;
         v[u] = lds_read_b128<u * ROW_STEP * ROW>(rd_addr + (uint32_t)(b * ROW_STEP * ROW));
       });
-      if constexpr (EPI == kEpiDact) {
+      if constexpr (kPre) {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) pre[u] = pre_next[u];
-        if (b + BATCH < ITERS) fetch_pre(pre_next, m + BATCH * ROW_STEP, off + BATCH * off_step);
+        if constexpr (kDglu) {
+#pragma unroll
+          for (int u = 0; u < BATCH; ++u) {
+            preb[u] = preb_next[u];
+            pre_next[u] = pre_far[u];
+            preb_next[u] = preb_far[u];
+          }
+          fetch_pre(pre_far, pre_rsrc, off + 2 * BATCH * off_step);     // past the tile's rows at the end: not used
+          fetch_pre(preb_far, preb_rsrc, off + 2 * BATCH * off_step);
+        } else {
+          fetch_pre(pre_next, pre_rsrc, off + BATCH * off_step);
+        }
       }
-      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+      if constexpr (BATCH == 8) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+      } else {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+      }
       if constexpr (EPI == kEpiDact) {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) v[u] = gelu_bwd_chunk<DT>(v[u], pre[u]);
+      }
+      if constexpr (kDglu) {
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          const u32x4 gv = v[u];
+          dglu_chunk<DT, EPI == kEpiDgluGelu>(gv, pre[u], preb[u], v[u], y[u]);
+        }
       }
       if (full_n) {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u)
           if (m + u * ROW_STEP < m_lim) {
             __builtin_nontemporal_store(v[u], (u32x4*)(cb + (off + (uint32_t)u * off_step)));
-            if constexpr (EPI == kEpiAct) {
-              const u32x4 y = gelu_fwd_chunk<DT>(v[u]);
-              __builtin_nontemporal_store(y, (u32x4*)(eb + (off + (uint32_t)u * off_step)));
-            }
+            if constexpr (EPI == kEpiAct) y[u] = gelu_fwd_chunk<DT>(v[u]);
+            if constexpr (kTwoOut) __builtin_nontemporal_store(y[u], (u32x4*)(second + (off + (uint32_t)u * off_step)));
           }
       } else {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) {
           if (m + u * ROW_STEP >= m_lim || n >= n_lim) continue;
           uint16_t* dst = (uint16_t*)(cb + (off + (uint32_t)u * off_step));
-          u32x4 y = v[u];
-          if constexpr (EPI == kEpiAct) y = gelu_fwd_chunk<DT>(v[u]);
-          uint16_t* dst2 = (uint16_t*)(eb + (off + (uint32_t)u * off_step));
+          if constexpr (EPI == kEpiAct) y[u] = gelu_fwd_chunk<DT>(v[u]);
+          uint16_t* dst2 = (uint16_t*)(second + (off + (uint32_t)u * off_step));
           if (n + 8 <= n_lim) {
             *(u32x4*)dst = v[u];
-            if constexpr (EPI == kEpiAct) *(u32x4*)dst2 = y;
+            if constexpr (kTwoOut) *(u32x4*)dst2 = y[u];
           } else {
 #pragma unroll
             for (int t = 0; t < 8; ++t)
               if (n + t < n_lim) {
                 dst[t] = (uint16_t)(v[u][t >> 1] >> ((t & 1) * 16));
-                if constexpr (EPI == kEpiAct) dst2[t] = (uint16_t)(y[t >> 1] >> ((t & 1) * 16));
+                if constexpr (kTwoOut) dst2[t] = (uint16_t)(y[kTwoOut ? u : 0][t >> 1] >> ((t & 1) * 16));
               }
           }
         }
@@ -967,20 +1056,13 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
 // c = A_tile * B_tile over all K tiles (the whole product of one output tile)
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, int EPI = kEpiNone>
 __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
-                                           int n_base, int n_lim, char* lds, uint16_t* __restrict__ extra = nullptr) {
+                                           int n_base, int n_lim, char* lds, uint16_t* __restrict__ extra = nullptr,
+                                           const uint16_t* __restrict__ pre2 = nullptr, uint16_t* __restrict__ out2 = nullptr) {
   typename T::Acc acc[T::TM][T::TN];
   block_multiply<DT, A_MC, B_MC, T, DUAL>(g, acc, true, lds);
-  block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra);
+  block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra, pre2, out2);
 }
 
-// Buffer sizes stay below 2 GiB: bit 31 of a byte offset marks a load that must fetch nothing.
-__device__ __forceinline__ uint32_t clip_bytes(int64_t bytes) {
-  return (uint32_t)(bytes < 0x7fffffff ? bytes : 0x7fffffff);
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
-}
 
 // ---- workgroups that compute several tiles ----
 // An NN / NT launch has one workgroup per compute unit (P of them, a multiple of 8); each walks a
@@ -1143,14 +1225,17 @@ struct RowTiles {
 // the tail then costs little more than half a round.  TS = T switches this off.
 // DUAL: c = a @ b[e] + a2 @ b2[e] in one pass (k is the reduction length of each pair, at least
 // (SB + 1) K tiles), as one reduction over 2 k.
-// EPI: see block_store; `extra` is its second output / input, [rows, n] like c.
+// EPI: see block_store; `extra` is its second output / input, [rows, n] like c; kEpiDglu*: `a2` is x2 and `out2` the
+// second output, both [rows, n].
 template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false, int EPI = kEpiNone>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
-                const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra) {
+                const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra,
+                uint16_t* __restrict__ out2) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
+  static_assert(!(DUAL && epi_is_dglu(EPI)), "a2 is the second operand pair's a or the epilogue's x2");
   constexpr bool kSplit = T::BM != TS::BM;
   static_assert(!kSplit || T::BM == 2 * TS::BM, "tail tile");
   const int P = gridDim.x, run = P / kXcds;
@@ -1196,12 +1281,14 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     g.b_r0 = tn * T::BN;
     uint16_t* const c_tile = c + (int64_t)row0 * n;
     uint16_t* const e_tile = EPI != kEpiNone ? extra + (int64_t)row0 * n : nullptr;
+    const uint16_t* const p_tile = epi_is_dglu(EPI) ? a2 + (int64_t)row0 * n : nullptr;   // x2 of the gated activation
+    uint16_t* const o_tile = epi_is_dglu(EPI) ? out2 + (int64_t)row0 * n : nullptr;
     // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
     use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
     if (use_ts) {
-      block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile);
+      block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
     } else {
-      block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile);
+      block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
     }
     tile_done();
   }

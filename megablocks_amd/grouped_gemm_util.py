@@ -243,6 +243,33 @@ def gmm_dact(a, b, pre, batch_sizes, c=None, fuse=None):
     return c
 
 
+def gmm_dglu(a, b, x1, x2, batch_sizes, act, fuse=None):
+    """The gradients (d x1, d x2) of `activation(x1) * x2` where the incoming gradient is g = a[r_e] @ b[e].T: the
+    `gmm(ddsd_out, w2, trans_b=True)` of the GLU experts' backward and the backward of their gated activation
+    (glu.py:135-153) in one launch where the library has a kernel for the shape, else as `gmm` and the element-wise
+    pass.  act: 0 = SiLU, 1 = tanh-GELU."""
+    a, b, bins = _nt_operands(a, b, batch_sizes, 'gmm_dglu')
+    rows, k, n, groups = a.shape[0], a.shape[1], b.shape[1], bins.shape[0]
+    _lib.require_cuda(x1, x2)
+    for t in (x1, x2):
+        if tuple(t.shape) != (rows, n) or t.dtype != a.dtype or not t.is_contiguous():
+            raise ValueError('gmm_dglu: x1 / x2 have the wrong shape, dtype or layout')
+    rc = _lib.EUNSUPPORTED
+    if _use_epilogue(fuse, a, rows, n):
+        d1 = torch.empty((rows, n), dtype=a.dtype, device=a.device)
+        d2 = torch.empty((rows, n), dtype=a.dtype, device=a.device)
+        with _lib.device_of(a), _lib.record('gmm_nt_dglu', rows=rows, k=k, n=n, elem=a.element_size(), groups=groups) as rec:
+            rc = lib.mbx_gmm_dglu(_lib.ptr(a), _lib.ptr(b), _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(d1), _lib.ptr(d2),
+                                  _lib.dtype_of(a), _lib.ptr(bins), groups, rows, k, n, act, _lib.stream())
+            if rc == _lib.EUNSUPPORTED:
+                rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        from megablocks_amd.layers.glu import _glu_backward
+        return _glu_backward(gmm(a, b, batch_sizes, trans_b=True), x1, x2, act)
+    _lib.check(rc, 'gmm_dglu')
+    return d1, d2
+
+
 class GroupedGemm(torch.autograd.Function):
     """Differentiable gmm(a, b, batch_sizes, trans_b): da = gmm(dc, b, trans_b flipped),
     db = the per-group outer product (trans_a)."""

@@ -107,6 +107,50 @@ class GLUProjection(torch.autograd.Function):
         return dx, dw1, dv1, None
 
 
+class GroupedGLUExperts(torch.autograd.Function):
+    """The grouped GLU experts of glu.py:201-205 as one node: the same products and element-wise steps as
+    GLUProjection -> GatedActivation -> gmm, with everything they save, but the backward can then hand the product
+    `ddsd_out @ w2[e]^T` and the backward of the gated activation to one launch (`gg.gmm_dglu`): the gradient of the
+    activation output is never written to memory."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
+    def forward(ctx, x, w1, v1, w2, batch_sizes, act):
+        x = x.contiguous()
+        sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
+        v1_out = gg.backend.gmm(x, v1, batch_sizes, trans_b=True)
+        activation_fn_out = _glu_forward(sdd_out, v1_out, act)
+        ctx.act = act
+        ctx.save_for_backward(x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out)
+        return gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
+    def backward(ctx, ddsd_out):
+        x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out = ctx.saved_tensors
+        ddsd_out = ddsd_out.contiguous()
+        dx = dw1 = dv1 = dw2 = None
+        if ctx.needs_input_grad[3]:
+            dw2 = gg.backend.gmm(activation_fn_out, ddsd_out, batch_sizes, trans_a=True)
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            dsdd_out, dv1_out = gg.gmm_dglu(ddsd_out, w2, sdd_out, v1_out, batch_sizes, ctx.act)
+            if ctx.needs_input_grad[1]:
+                dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
+            if ctx.needs_input_grad[2]:
+                dv1 = gg.backend.gmm(dv1_out, x, batch_sizes, trans_a=True)
+            if ctx.needs_input_grad[0]:
+                dx = gg.gmm_dual(dsdd_out, w1, dv1_out, v1, batch_sizes)
+        return dx, dw1, dv1, dw2, None, None
+
+
+def _one_node(x, w1, v1, w2, act):
+    """Whether the experts can run as GroupedGLUExperts: an activation the library has, 16-bit operands of one type on
+    the GPU, rows the element-wise kernels take."""
+    return (act is not None and x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and
+            w1.dtype == v1.dtype == w2.dtype == x.dtype and (w1.shape[1] * x.element_size()) % 16 == 0 and
+            w1.is_contiguous() and v1.is_contiguous() and w2.is_contiguous())
+
+
 class MemoryOptimizedGroupedGLU(torch.autograd.Function):
     """glu.py:66-167: saves (x, sdd_out, v1_out), recomputes the gated activation in backward."""
 
@@ -152,9 +196,9 @@ class MemoryOptimizedGroupedGLU(torch.autograd.Function):
 
         dw2 = gg.backend.gmm(activation_fn_out.detach(), ddsd_out, batch_sizes, trans_a=True)
         if fused:
-            # the gradient of the activation output overwrites the recomputed activation
-            dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True, c=activation_fn_out)
-            dsdd_out, dv1_out = _glu_backward(dactivation_fn_out, sdd_out, v1_out, act)
+            # one launch where the library has it; else the product (which then overwrites the recomputed activation,
+            # glu.py:138) and the element-wise backward
+            dsdd_out, dv1_out = gg.gmm_dglu(ddsd_out, w2, sdd_out, v1_out, batch_sizes, act)
         else:
             dactivation_fn_out = gg.backend.gmm(ddsd_out, w2, batch_sizes, trans_b=True)
             activation_fn_out.backward(dactivation_fn_out)
@@ -188,7 +232,11 @@ class SparseGLU(SparseMLP):
                 raise NotImplementedError(
                     'Memory optimized implementation not yet supported with GLU with sparse kernels.')
             return memory_optimized_grouped_glu(x, w1, v1, w2, batch_sizes, self.args.activation_fn)
-        x1, x2 = GLUProjection.apply(*gg.autocast_operands(x, w1, v1), batch_sizes)
+        act = _activation_code(self.args.activation_fn)
+        operands = gg.autocast_operands(x, w1, v1, w2)
+        if _one_node(*operands, act):
+            return GroupedGLUExperts.apply(*operands, batch_sizes, act)
+        x1, x2 = GLUProjection.apply(*operands[:3], batch_sizes)
         x1 = gated_activation(self.args.activation_fn, x1, x2)
         return gg.ops.gmm(x1, w2, batch_sizes)
 

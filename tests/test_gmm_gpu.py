@@ -598,3 +598,34 @@ def test_gmm_with_activation_epilogues(gg, groups, rows, k, n, dtype):
         gg.gmm_dact(dy, b, x_pre, sizes, c=x_pre)                              # the epilogue reads pre while it writes c
     with pytest.raises(ValueError):
         gg.gmm_act(a, b[:, :, :k - 8].contiguous(), sizes)
+
+
+@pytest.mark.parametrize('groups,rows,k,n', EPILOGUE)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('act', [0, 1], ids=['silu', 'gelu_tanh'])
+def test_gmm_with_gated_activation_backward_epilogue(gg, groups, rows, k, n, dtype, act):
+    """gmm_dglu: with g = round(dy @ w2^T), (round(g x2) act'(x1), g round(act(x1))) in one launch, against autograd's
+    gradient of act(x1) * x2 in fp32 (glu.py:120-124,135-153) and against the product followed by the element-wise
+    kernel, which it must equal to a rounding step of the output type."""
+    from megablocks_amd.layers.glu import _glu_backward
+    torch.manual_seed(groups * 11 + n + act)
+    sizes = _sizes(groups, rows, seed=rows + k + 1, empty=(1,) if groups > 2 else ())
+    dy = torch.randn(rows, k, device='cuda').to(dtype)
+    b = (torch.randn(groups, n, k, device='cuda') * (1.0 / k ** 0.5)).to(dtype)
+    x1 = (torch.randn(rows, n, device='cuda') * 1.5).to(dtype)
+    x2 = torch.randn(rows, n, device='cuda').to(dtype)
+    g = _ref_gpu(dy, b, sizes, False, True).to(dtype).float()
+    fn = torch.nn.functional.silu if act == 0 else (lambda t: torch.nn.functional.gelu(t, approximate='tanh'))
+    a_, b_ = x1.float().requires_grad_(True), x2.float().requires_grad_(True)
+    (fn(a_) * b_).backward(g)
+    d1, d2 = gg.gmm_dglu(dy, b, x1, x2, sizes, act, fuse=True)
+    tol = 1e-4 if dtype == torch.float32 else TOL
+    assert d1.shape == (rows, n) and d2.shape == (rows, n) and d1.dtype == dtype and d2.dtype == dtype
+    assert rel_err(d1.float(), a_.grad) < tol and rel_err(d2.float(), b_.grad) < tol
+    t1, t2 = _glu_backward(gg.backend.gmm(dy, b, sizes, trans_b=True), x1, x2, act)
+    step = 1e-6 if dtype == torch.float32 else 4e-3
+    assert rel_err(d1.float(), t1.float()) < step and rel_err(d2.float(), t2.float()) < step
+    u1, u2 = gg.gmm_dglu(dy, b, x1, x2, sizes.cuda(), act, fuse=False)
+    assert torch.equal(u1, t1) and torch.equal(u2, t2)
+    with pytest.raises(ValueError):
+        gg.gmm_dglu(dy, b, x1[:, :n - 8].contiguous(), x2, sizes, act)

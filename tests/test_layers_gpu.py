@@ -142,6 +142,37 @@ def test_dmoe_mlp_with_activation_epilogues_vs_oracle(syn, monkeypatch, mlp_impl
     assert rel_err(ew.grad, want_grads['expert_weights']) < 1e-2
 
 
+@pytest.mark.parametrize('mlp_impl,memopt', [('grouped', False), ('grouped', True), ('sparse', False)])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_dmoe_glu_with_the_gate_backward_in_the_epilogue_vs_oracle(syn, monkeypatch, mlp_impl, memopt, dtype):
+    """The gated experts with the backward of the gated activation in the epilogue of the product that feeds it (taken
+    by itself only for intermediates beyond the Infinity Cache; forced here) against the oracle, forward and backward."""
+    from megablocks_amd import grouped_gemm_util as gg
+    monkeypatch.setattr(gg, 'ACTIVATION_EPILOGUE_MIN_BYTES', 0)
+    w = syn.Workload('t', 1500, 256, 768, 8, 2, 'glu', mlp_impl, dtype, 'logits')
+    inp = syn.make_inputs(w, seed=6)
+    for k in ('x', 'grad', 'w1', 'v1', 'w2', 'expert_weights'):
+        inp[k] = inp[k].to(dtype).float()
+    want, _, want_grads, _ = _oracle_step(w, inp, True)
+    layer = syn.build_layer(w, inp, memory_optimized=memopt)
+    x = inp['x'].to(dtype).cuda().requires_grad_(True)
+    ew = inp['expert_weights'].to(dtype).cuda().requires_grad_(True)
+    from megablocks_amd import _lib
+    _lib.profile_hook = []
+    try:
+        out = syn.layer_step(layer, w, x, inp['grad'].to(dtype).cuda(), (inp['scores'].to(dtype).cuda(), ew, inp['top_experts'].cuda()))
+        torch.cuda.synchronize()
+        launched = {name for name, *_ in _lib.profile_hook}
+    finally:
+        _lib.profile_hook = None
+    assert 'gmm_nt_dglu' in launched                                       # the epilogue kernel is what ran
+    assert rel_err(out, want) < 1e-2 and rel_err(x.grad, want_grads['x']) < 1e-2
+    mlp = layer.experts.mlp
+    for name in ('w1', 'v1', 'w2'):
+        assert rel_err(getattr(mlp, name).grad, want_grads[name]) < 1e-2, name
+    assert rel_err(ew.grad, want_grads['expert_weights']) < 1e-2
+
+
 @pytest.mark.parametrize('tokens,hidden,experts', [(4096, 1024, 64), (5003, 264, 8), (16384, 512, 16)])
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 def test_router_linear_gradients(tokens, hidden, experts, dtype):
