@@ -215,6 +215,15 @@ int mbx_gmm_act(const void* a, const void* b, void* c, void* c_act, int dtype, c
 int mbx_gmm_dact(const void* a, const void* b, const void* pre, void* c, int dtype, const int32_t* bins,
                  int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
 
+/* The two first products of the GLU experts and their gated activation, megablocks/layers/glu.py:201-204
+ * (`x1 = gmm(x, w1, trans_b=True); x2 = gmm(x, v1, trans_b=True); x1 = activation_fn(x1) * x2`), in one launch:
+ *   x1[r_e] = a[r_e] @ b1[e]^T,   x2[r_e] = a[r_e] @ b2[e]^T   (b1, b2: [E, n, k]),   h = round(round(act(x1)) * x2)
+ * every workgroup computes the same 128 columns of both products side by side and gates them in the epilogue, from the
+ * values as stored (rounded to `dtype`).  All three outputs are [rows, n].  act: MBX_ACT_SILU or MBX_ACT_GELU_TANH.
+ * MBX_EUNSUPPORTED (the caller runs two mbx_gmm and mbx_glu_forward): as for mbx_gmm_dglu. */
+int mbx_gmm_glu(const void* a, const void* b1, const void* b2, void* x1, void* x2, void* h, int dtype,
+                const int32_t* bins, int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
+
 /* The backward of the GLU experts' gated activation on the product that feeds it, megablocks/layers/glu.py:135-153
  * (`gmm(ddsd_out, w2, trans_b=True, c=dactivation_fn_out)`, then autograd's gradient of
  * `activation_fn(sdd_out) * v1_out`, glu.py:120-124), in one launch:

@@ -588,7 +588,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const uint16_t* bp = (const uint16_t*)b;
   const uint16_t* ap2 = (const uint16_t*)a2;
   const uint16_t* bp2 = (const uint16_t*)b2;
-  const bool dual = a2 != nullptr && !dma::epi_is_dglu(epi);
+  const bool dual = a2 != nullptr && !dma::epi_is_dglu(epi) && !dma::epi_is_glu(epi);
   uint16_t* cp = (uint16_t*)c;
   if (layout == MBX_TN) {
     constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
@@ -618,7 +618,8 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     return launch_status();
   }
   constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
-  const int tiles_n = (int)ceil_div(n, T::BN);
+  // a [w1 | v1] tile covers half as many output columns
+  const int tiles_n = (int)ceil_div(n, dma::epi_is_glu(epi) ? T::BN / 2 : T::BN);
   const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
   if (tiles > 0x7fffffff) return MBX_ERANGE;
   const unsigned grid = (unsigned)persistent_grid(tiles);
@@ -629,6 +630,16 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (rc) return rc;                                                                                \
     kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2);  \
   } while (0)
+  if (dma::epi_is_glu(epi)) {
+    // b2 is the second matrix of the [w1 | v1] tiles (not a second operand pair); 16 x 16 x 32 tiles only
+    if (layout != MBX_NT || !extra || !b2 || !out2 || a2) return MBX_EINVAL;
+    if constexpr (T::MF == 16) {
+      if (epi == dma::kEpiGluSilu) MBX_LAUNCH_ROWS(false, false, dma::kEpiGluSilu); else MBX_LAUNCH_ROWS(false, false, dma::kEpiGluGelu);
+      return launch_status();
+    } else {
+      return MBX_EUNSUPPORTED;
+    }
+  }
   if (dma::epi_is_dglu(epi)) {
     // a2 carries x2 of the gated activation (not a second operand pair); only the 16 x 16 x 32 tiles are instantiated
     if (layout != MBX_NT || !extra || !a2 || !out2) return MBX_EINVAL;
@@ -783,29 +794,32 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
 // The NT product with an activation epilogue (epi: dma::kEpiAct / dma::kEpiDact), for the shapes the direct-to-LDS
 // kernels take; anything else is MBX_EUNSUPPORTED and the caller runs the product and the element-wise pass.
 // (kEpiDglu*: pre2 = x2, out2 = the second output; 16 x 16 x 32 main loop only.)
+// (kEpiGlu*: b2 = the second matrix, extra = the gated activation, out2 = the second product.)
 static int gmm_nt_epilogue(const void* a, const void* b, void* c, void* extra, int dtype, const int32_t* bins, int num_groups,
                            int64_t rows, int k, int n, int act, int epi, mbx_stream_t stream, const void* pre2 = nullptr,
-                           void* out2 = nullptr) {
+                           void* out2 = nullptr, const void* b2 = nullptr) {
   if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
-  const bool dglu = dma::epi_is_dglu(epi);
-  if (!dglu && act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
+  const bool dglu = dma::epi_is_dglu(epi), glu = dma::epi_is_glu(epi);
+  if (!dglu && !glu && act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
   if (num_groups == 0 || rows == 0 || n == 0) return 0;
-  if (!bins || !c || !extra || (k > 0 && (!a || !b)) || (dglu && (!pre2 || !out2))) return MBX_EINVAL;
+  if (!bins || !c || !extra || (k > 0 && (!a || !b)) || (dglu && (!pre2 || !out2)) || (glu && (!out2 || (k > 0 && !b2)))) return MBX_EINVAL;
   if (rows > 0x7fffffff) return MBX_ERANGE;
-  const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(extra) && k > 0 &&
-                  k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n) && (!dglu || (aligned16(pre2) && aligned16(out2)));
+  bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(extra) && k > 0 &&
+            k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n) && (!dglu || (aligned16(pre2) && aligned16(out2)));
+  // the second matrix is addressed from half a tile before its first row: that much more must fit below 2 GiB
+  if (glu) ok = ok && aligned16(b2) && aligned16(out2) && dma_sizes_ok(k, n + TileDma::BN / 2);
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   if (use_mfma16()) {
     if (half_height_only(rows, num_groups, n)) {
-      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
-      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
+      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
     }
-    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
-    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, nullptr, epi, extra, out2);
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
+    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
   }
-  if (dglu) return MBX_EUNSUPPORTED;
+  if (dglu || glu) return MBX_EUNSUPPORTED;
   if (half_height_only(rows, num_groups, n)) {
     if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
     return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
@@ -822,6 +836,13 @@ int mbx_gmm_act(const void* a, const void* b, void* c, void* c_act, int dtype, c
 int mbx_gmm_dact(const void* a, const void* b, const void* pre, void* c, int dtype, const int32_t* bins, int num_groups,
                  int64_t rows, int k, int n, int act, mbx_stream_t stream) {
   return gmm_nt_epilogue(a, b, c, (void*)pre, dtype, bins, num_groups, rows, k, n, act, dma::kEpiDact, stream);
+}
+
+int mbx_gmm_glu(const void* a, const void* b1, const void* b2, void* x1, void* x2, void* h, int dtype, const int32_t* bins,
+                int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream) {
+  if (act != MBX_ACT_SILU && act != MBX_ACT_GELU_TANH) return MBX_EINVAL;
+  return gmm_nt_epilogue(a, b1, x1, h, dtype, bins, num_groups, rows, k, n, act,
+                         act == MBX_ACT_SILU ? dma::kEpiGluSilu : dma::kEpiGluGelu, stream, nullptr, x2, b2);
 }
 
 int mbx_gmm_dglu(const void* a, const void* b, const void* x1, const void* x2, void* d1, void* d2, int dtype,

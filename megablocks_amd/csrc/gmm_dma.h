@@ -457,9 +457,13 @@ __device__ __forceinline__ void mfma16_settle() { asm volatile("s_nop 15\n\ts_no
 // so that every load has at least a K tile and a half of MFMAs before the barrier that waits for it (a B load issued
 // just ahead of the barrier that needs it, as a transcription of the 32 x 32 x 16 schedule had it, stalls every K tile
 // for a memory latency).  The prologue loads tiles 0 .. SB - 1 completely.
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
+// GLU: rows BN / 2 .. BN - 1 of the B tile (the second half of every wave's loads of a K tile) come through g.rsrc_b2,
+// whose base the caller has set BN / 2 rows before the second matrix: the tile is then [w1 rows | v1 rows] of the same
+// BN / 2 output columns, side by side (KC operands only, not with DUAL).
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false>
 __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
   static_assert(T::MF == 16 && T::KS == 2, "two k-steps of 32 per K tile");
+  static_assert(!GLU || (!B_MC && !DUAL && T::LB % 2 == 0), "two matrices side by side in the B tile");
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -484,12 +488,14 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
     return v | (kt < g.nk ? 0u : 0x80000000u);
   };
   __amdgpu_buffer_rsrc_t ra = g.rsrc_a, rb = g.rsrc_b;
+  const __amdgpu_buffer_rsrc_t rb_upper = GLU ? g.rsrc_b2 : g.rsrc_b;
   auto lds_off = [&](bool is_b, int stage, int q) -> uint32_t {
     return (is_b ? B_RING + (uint32_t)stage * T::B_BYTES : (uint32_t)stage * T::A_BYTES) + (uint32_t)(wave + q * T::WAVES) * 1024u;
   };
-  auto issue = [&](bool is_b, uint32_t sc, uint32_t dst, bool odd) {
+  // upper: the load is one of the second half of the wave's B loads of a K tile (GLU only)
+  auto issue = [&](bool is_b, uint32_t sc, uint32_t dst, bool odd, bool upper = false) {
     if (is_b) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? b_lane1 : b_lane) + sc), 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(GLU && upper ? rb_upper : rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? b_lane1 : b_lane) + sc), 0, 0, 0);
     } else {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? a_lane1 : a_lane) + sc), 0, 0, 0);
     }
@@ -498,7 +504,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
     uint32_t sc = scalar_off(is_b, kt, q0), dst = lds_off(is_b, stage, q0);
 #pragma unroll
     for (int i = 0; i < count; ++i) {
-      issue(is_b, sc, dst, ((q0 + i) & 1) != 0);
+      issue(is_b, sc, dst, ((q0 + i) & 1) != 0, is_b && q0 + i >= LB / 2);
       sc += T::WAVES * (is_b ? b_jstep : a_jstep);
       dst += T::WAVES * 1024u;
     }
@@ -588,7 +594,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
       mfma16_acc<DT>(acc[i_][j_], fb[CUR_BUF][j_], fa[CUR_BUF][i_]);                                             \
       MBX_READ_SLOT16(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                            \
       if constexpr (m_ >= (LOAD0) && (m_ - (LOAD0)) % (EVERY) == 0 && (m_ - (LOAD0)) / (EVERY) < (NL))           \
-        issue(IS_B, SC, DST, (((m_ - (LOAD0)) / (EVERY)) & 1) != 0);                                             \
+        issue(IS_B, SC, DST, (((m_ - (LOAD0)) / (EVERY)) & 1) != 0, (IS_B) && (m_ - (LOAD0)) / (EVERY) >= (NL) / 2); \
       if constexpr (m_ > (LOAD0) && (m_ - (LOAD0) - 1) % (EVERY) == 0 && (m_ - (LOAD0) - 1) / (EVERY) < (NL)) {  \
         SC += T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                                           \
         DST += T::WAVES * 1024u;                                                                                 \
@@ -707,10 +713,11 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
 #undef MBX_STEP16
 }
 
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false>
 __device__ __forceinline__ void block_multiply(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds) {
+  static_assert(!GLU || T::MF == 16, "two matrices side by side: 16 x 16 x 32 loop only");
   if constexpr (T::MF == 32) block_multiply32<DT, A_MC, B_MC, T, DUAL>(g, acc, clear, lds);
-  else block_multiply16<DT, A_MC, B_MC, T, DUAL>(g, acc, clear, lds);
+  else block_multiply16<DT, A_MC, B_MC, T, DUAL, GLU>(g, acc, clear, lds);
 }
 
 // ---- activation in the epilogue (tanh-GELU: megablocks/layers/arguments.py:19, megablocks/layers/gelu.py:9-13) ----
@@ -766,8 +773,11 @@ __device__ __forceinline__ void gelu_tanh_bwd8(float (&g)[8], const float (&x)[8
 //   kEpiDgluSilu, kEpiDgluGelu   the tile g is the gradient of act(x1) * x2 (act = SiLU / tanh-GELU) with x1, x2 two
 //                 more inputs of the same shape: stores g * round(act(x1)) and round(g * x2) * act'(x1), two outputs,
 //                 and not g itself.
-enum { kEpiNone = 0, kEpiAct = 1, kEpiDact = 2, kEpiDgluSilu = 3, kEpiDgluGelu = 4 };
+//   kEpiGluSilu, kEpiGluGelu   the tile is [x1 | x2], the same BN / 2 output columns of two products side by side (see
+//                 block_multiply16's GLU): stores x1, x2 and round(round(act(x1)) * x2), three outputs.
+enum { kEpiNone = 0, kEpiAct = 1, kEpiDact = 2, kEpiDgluSilu = 3, kEpiDgluGelu = 4, kEpiGluSilu = 5, kEpiGluGelu = 6 };
 constexpr bool epi_is_dglu(int epi) { return epi == kEpiDgluSilu || epi == kEpiDgluGelu; }
+constexpr bool epi_is_glu(int epi) { return epi == kEpiGluSilu || epi == kEpiGluGelu; }
 
 // the eight 16-bit values of a 16-byte chunk as fp32 and back (rounded)
 template <int DT>
@@ -785,6 +795,33 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
 #pragma unroll
   for (int w = 0; w < 4; ++w) r[w] = pack2<DT>(f[2 * w], f[2 * w + 1]);
   return r;
+}
+// The gated activation on a chunk, round(round(act(x1)) * x2): the two roundings of computing act(x1) and the product
+// separately (glu.py:89,204).
+template <int DT, bool GELU>
+__device__ __forceinline__ u32x4 glu_chunk(const u32x4& x1v, const u32x4& x2v) {
+  float x[8], b[8], s[8], z[8];
+  unpack8<DT>(x1v, x);
+  unpack8<DT>(x2v, b);
+  if (GELU) {
+    sigmoid_2u8(x, z, s);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = -1.44269504f * x[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = __builtin_amdgcn_exp2f(z[i]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = 1.f + z[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] = __builtin_amdgcn_rcpf(z[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = x[i] * s[i];
+  const u32x4 actv = pack8<DT>(z);
+  unpack8<DT>(actv, z);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = z[i] * b[i];
+  return pack8<DT>(z);
 }
 // The backward of the gated activation act(x1) * x2 on a chunk, with the roundings autograd's separate steps make:
 //   d2 = g * round(act(x1)),   d1 = round(g * x2) * act'(x1)
@@ -904,6 +941,57 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
       }
     }
     __syncthreads();
+    if constexpr (epi_is_glu(EPI)) {
+      // The tile is [x1 | x2]: BN / 2 output columns from n_base on.  A lane takes the same 16-byte chunk of both
+      // halves of a row: 16 lanes a row, four rows per instruction; it stores the two chunks (to c and out2) and
+      // their gated activation (to extra).  Batches of four rows per lane: eight LDS reads in flight, twelve stores.
+      static_assert(T::BN == 256, "sixteen chunks per half row");
+      constexpr int RPI = 4, ITERS = T::BM / RPI / T::WAVES, BATCH = 4, ROW_STEP = T::WAVES * RPI;
+      static_assert(ITERS % BATCH == 0, "store batches");
+      const int rl = lane >> 4, ch = lane & 15;
+      const int n = n_base + ch * 8;
+      const uint32_t rd_addr = lds_base + (uint32_t)((wave * RPI + rl) * ROW + ch * 16);
+      int m = m_base + wave * RPI + rl;
+      uint32_t off = ((uint32_t)m * (uint32_t)ldc + (uint32_t)n) * 2u;
+      const uint32_t off_step = (uint32_t)ROW_STEP * (uint32_t)ldc * 2u;
+      char* const cb = (char*)c;
+      char* const hb = (char*)extra;
+      char* const ob = (char*)out2;
+      const bool full_n = n_base + T::BN / 2 <= n_lim;      // uniform
+#pragma unroll 1
+      for (int b = 0; b < ITERS; b += BATCH) {
+        u32x4 v1[BATCH], v2[BATCH], h[BATCH];
+        static_for<BATCH>([&](auto ui) {
+          constexpr int u = decltype(ui)::value;
+          v1[u] = lds_read_b128<u * ROW_STEP * ROW>(rd_addr + (uint32_t)(b * ROW_STEP * ROW));
+          v2[u] = lds_read_b128<u * ROW_STEP * ROW + T::BN>(rd_addr + (uint32_t)(b * ROW_STEP * ROW));
+        });
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v1[0]), "+v"(v1[1]), "+v"(v1[2]), "+v"(v1[3]), "+v"(v2[0]), "+v"(v2[1]), "+v"(v2[2]), "+v"(v2[3]));
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) h[u] = glu_chunk<DT, EPI == kEpiGluGelu>(v1[u], v2[u]);
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          if (m + u * ROW_STEP >= m_lim || n >= n_lim) continue;
+          const uint32_t o = off + (uint32_t)u * off_step;
+          if (full_n || n + 8 <= n_lim) {
+            __builtin_nontemporal_store(v1[u], (u32x4*)(cb + o));
+            __builtin_nontemporal_store(v2[u], (u32x4*)(ob + o));
+            __builtin_nontemporal_store(h[u], (u32x4*)(hb + o));
+          } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+              if (n + t < n_lim) {
+                ((uint16_t*)(cb + o))[t] = (uint16_t)(v1[u][t >> 1] >> ((t & 1) * 16));
+                ((uint16_t*)(ob + o))[t] = (uint16_t)(v2[u][t >> 1] >> ((t & 1) * 16));
+                ((uint16_t*)(hb + o))[t] = (uint16_t)(h[u][t >> 1] >> ((t & 1) * 16));
+              }
+          }
+        }
+        m += BATCH * ROW_STEP;
+        off += BATCH * off_step;
+      }
+      return;
+    }
     constexpr int CHUNKS = T::BN / 8;                 // 16-byte chunks per tile row
     constexpr int ROWS_PER_INSTR = kWave / CHUNKS;    // 2 for 256-wide tiles
     const int rl = lane / CHUNKS, ch = lane % CHUNKS;
@@ -1059,7 +1147,7 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
                                            int n_base, int n_lim, char* lds, uint16_t* __restrict__ extra = nullptr,
                                            const uint16_t* __restrict__ pre2 = nullptr, uint16_t* __restrict__ out2 = nullptr) {
   typename T::Acc acc[T::TM][T::TN];
-  block_multiply<DT, A_MC, B_MC, T, DUAL>(g, acc, true, lds);
+  block_multiply<DT, A_MC, B_MC, T, DUAL, epi_is_glu(EPI)>(g, acc, true, lds);
   block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra, pre2, out2);
 }
 
@@ -1235,7 +1323,8 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
                 uint16_t* __restrict__ out2) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
-  static_assert(!(DUAL && epi_is_dglu(EPI)), "a2 is the second operand pair's a or the epilogue's x2");
+  static_assert(!(DUAL && (epi_is_dglu(EPI) || epi_is_glu(EPI))), "a2 / b2 are the second operand pair, the epilogue's x2 or the second matrix");
+  constexpr int kTileCols = epi_is_glu(EPI) ? T::BN / 2 : T::BN;   // output columns of a tile
   constexpr bool kSplit = T::BM != TS::BM;
   static_assert(!kSplit || T::BM == 2 * TS::BM, "tail tile");
   const int P = gridDim.x, run = P / kXcds;
@@ -1278,11 +1367,13 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     g.rsrc_a2 = DUAL ? make_rsrc(a2 + (int64_t)row0 * k, a_bytes) : g.rsrc_a;
     g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
     g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
-    g.b_r0 = tn * T::BN;
+    // the second matrix of a [w1 | v1] tile: rows BN / 2 .. BN - 1 of the tile are its rows b_r0 .. b_r0 + BN / 2 - 1
+    if (epi_is_glu(EPI)) g.rsrc_b2 = make_rsrc(b2 + ((int64_t)e * n - T::BN / 2) * k, (uint32_t)(((int64_t)n + T::BN / 2) * k * 2));
+    g.b_r0 = tn * kTileCols;
     uint16_t* const c_tile = c + (int64_t)row0 * n;
     uint16_t* const e_tile = EPI != kEpiNone ? extra + (int64_t)row0 * n : nullptr;
     const uint16_t* const p_tile = epi_is_dglu(EPI) ? a2 + (int64_t)row0 * n : nullptr;   // x2 of the gated activation
-    uint16_t* const o_tile = epi_is_dglu(EPI) ? out2 + (int64_t)row0 * n : nullptr;
+    uint16_t* const o_tile = epi_is_dglu(EPI) || epi_is_glu(EPI) ? out2 + (int64_t)row0 * n : nullptr;
     // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
     use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
     if (use_ts) {

@@ -243,6 +243,33 @@ def gmm_dact(a, b, pre, batch_sizes, c=None, fuse=None):
     return c
 
 
+def gmm_glu(a, b1, b2, batch_sizes, act, fuse=None):
+    """(x1, x2, h) with x1 = a[r_e] @ b1[e].T, x2 = a[r_e] @ b2[e].T and h = activation(x1) * x2: the two first
+    products of the GLU experts and their gated activation (glu.py:201-204) in one launch where the library has a
+    kernel for the shape, else as two `gmm` and the element-wise pass.  act: 0 = SiLU, 1 = tanh-GELU."""
+    a, b1, bins = _nt_operands(a, b1, batch_sizes, 'gmm_glu')
+    _lib.require_cuda(b2)
+    if b2.shape != b1.shape or b2.dtype != b1.dtype:
+        raise ValueError('gmm_glu: b2 must be shaped and typed like b1')
+    b2 = b2.contiguous()
+    rows, k, n, groups = a.shape[0], a.shape[1], b1.shape[1], bins.shape[0]
+    rc = _lib.EUNSUPPORTED
+    if _use_epilogue(fuse, a, rows, n):
+        x1, x2, h = (torch.empty((rows, n), dtype=a.dtype, device=a.device) for _ in range(3))
+        with _lib.device_of(a), _lib.record('gmm_nt_glu', rows=rows, k=k, n=2 * n, elem=a.element_size(), groups=groups) as rec:
+            rc = lib.mbx_gmm_glu(_lib.ptr(a), _lib.ptr(b1), _lib.ptr(b2), _lib.ptr(x1), _lib.ptr(x2), _lib.ptr(h),
+                                 _lib.dtype_of(a), _lib.ptr(bins), groups, rows, k, n, act, _lib.stream())
+            if rc == _lib.EUNSUPPORTED:
+                rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        from megablocks_amd.layers.glu import _glu_forward
+        x1 = gmm(a, b1, batch_sizes, trans_b=True)
+        x2 = gmm(a, b2, batch_sizes, trans_b=True)
+        return x1, x2, _glu_forward(x1, x2, act)
+    _lib.check(rc, 'gmm_glu')
+    return x1, x2, h
+
+
 def gmm_dglu(a, b, x1, x2, batch_sizes, act, fuse=None):
     """The gradients (d x1, d x2) of `activation(x1) * x2` where the incoming gradient is g = a[r_e] @ b[e].T: the
     `gmm(ddsd_out, w2, trans_b=True)` of the GLU experts' backward and the backward of their gated activation

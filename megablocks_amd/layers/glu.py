@@ -117,9 +117,7 @@ class GroupedGLUExperts(torch.autograd.Function):
     @torch.amp.custom_fwd(device_type='cuda')
     def forward(ctx, x, w1, v1, w2, batch_sizes, act):
         x = x.contiguous()
-        sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
-        v1_out = gg.backend.gmm(x, v1, batch_sizes, trans_b=True)
-        activation_fn_out = _glu_forward(sdd_out, v1_out, act)
+        sdd_out, v1_out, activation_fn_out = gg.gmm_glu(x, w1, v1, batch_sizes, act)
         ctx.act = act
         ctx.save_for_backward(x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out)
         return gg.backend.gmm(activation_fn_out, w2, batch_sizes)
@@ -161,13 +159,16 @@ class MemoryOptimizedGroupedGLU(torch.autograd.Function):
             x, w1, v1, w2 = x.to(ctx._dtype), w1.to(ctx._dtype), v1.to(ctx._dtype), w2.to(ctx._dtype)
         if not x.is_contiguous() or not w1.is_contiguous() or not v1.is_contiguous() or not w2.is_contiguous():
             raise ValueError("Expected contiguous 'x', 'w1', 'v1' and 'w2'.")
-        sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
-        v1_out = gg.backend.gmm(x, v1, batch_sizes, trans_b=True)
         act = _activation_code(activation_fn)
-        if act is not None and _fusable(sdd_out, v1_out):
-            activation_fn_out = _glu_forward(sdd_out, v1_out, act)
+        if act is not None and _one_node(x, w1, v1, w2, act):
+            sdd_out, v1_out, activation_fn_out = gg.gmm_glu(x, w1, v1, batch_sizes, act)
         else:
-            activation_fn_out = activation_fn(sdd_out) * v1_out
+            sdd_out = gg.backend.gmm(x, w1, batch_sizes, trans_b=True)
+            v1_out = gg.backend.gmm(x, v1, batch_sizes, trans_b=True)
+            if act is not None and _fusable(sdd_out, v1_out):
+                activation_fn_out = _glu_forward(sdd_out, v1_out, act)
+            else:
+                activation_fn_out = activation_fn(sdd_out) * v1_out
         dsd_out = gg.backend.gmm(activation_fn_out, w2, batch_sizes)
         ctx.x_shape = x.shape
         ctx.sdd_out_shape = sdd_out.shape

@@ -629,3 +629,33 @@ def test_gmm_with_gated_activation_backward_epilogue(gg, groups, rows, k, n, dty
     assert torch.equal(u1, t1) and torch.equal(u2, t2)
     with pytest.raises(ValueError):
         gg.gmm_dglu(dy, b, x1[:, :n - 8].contiguous(), x2, sizes, act)
+
+
+@pytest.mark.parametrize('groups,rows,k,n', EPILOGUE + [(6, 2500, 256, 1416), (2, 300, 64, 136)])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('act', [0, 1], ids=['silu', 'gelu_tanh'])
+def test_gmm_with_gated_activation_epilogue(gg, groups, rows, k, n, dtype, act):
+    """gmm_glu: (x @ w1^T, x @ v1^T, round(round(act(x1)) x2)) in one launch (glu.py:201-204): both products must be
+    the plain kernel's bit for bit, the gated activation within a rounding step of the element-wise kernel's and of the
+    fp32 formula on the stored products."""
+    from megablocks_amd.layers.glu import _glu_forward
+    torch.manual_seed(groups * 13 + n + act)
+    sizes = _sizes(groups, rows, seed=rows + k + 2, empty=(1,) if groups > 2 else ())
+    a = torch.randn(rows, k, device='cuda').to(dtype)
+    w1 = (torch.randn(groups, n, k, device='cuda') * (1.5 / k ** 0.5)).to(dtype)
+    v1 = (torch.randn(groups, n, k, device='cuda') * (1.0 / k ** 0.5)).to(dtype)
+    guard = torch.full((3, rows + 16, n), 7.0, device='cuda', dtype=dtype)
+    x1, x2, h = gg.gmm_glu(a, w1, v1, sizes, act, fuse=True)
+    p1, p2 = gg.backend.gmm(a, w1, sizes, trans_b=True), gg.backend.gmm(a, v1, sizes.cuda(), trans_b=True)
+    assert x1.shape == (rows, n) and h.shape == (rows, n) and h.dtype == dtype
+    assert torch.equal(x1, p1) and torch.equal(x2, p2)
+    fn = torch.nn.functional.silu if act == 0 else (lambda t: torch.nn.functional.gelu(t, approximate='tanh'))
+    want = fn(p1.float()).to(dtype).float() * p2.float()
+    step = 1e-6 if dtype == torch.float32 else 4e-3
+    assert rel_err(h.float(), want) < step
+    assert rel_err(h.float(), _glu_forward(p1, p2, act).float()) < step
+    y1, y2, g = gg.gmm_glu(a, w1, v1, sizes, act, fuse=False)
+    assert torch.equal(y1, p1) and torch.equal(y2, p2) and torch.equal(g, _glu_forward(p1, p2, act))
+    assert bool((guard == 7.0).all())
+    with pytest.raises(ValueError):
+        gg.gmm_glu(a, w1, v1[:, :n - 8].contiguous(), sizes, act)
