@@ -161,6 +161,11 @@ def summarize(w, agg, slots_scale):
             nbytes = (pairs * (m['rows'] * slots_scale * kk + m['groups'] * kk * m['n']) + m['rows'] * slots_scale * m['n']) \
                 * m['elem'] if not name.startswith('gmm_tn') else \
                 (m['rows'] * slots_scale * (m['k'] + m['n']) + m['groups'] * m['k'] * m['n']) * m['elem']
+            # [rows, n] tensors the epilogues read or write besides the product: its activation; the saved product; the
+            # gated activation (half as wide as the two products side by side); x1, x2 and a second gradient
+            for suffix, more in (('_act', 1.0), ('_dact', 1.0), ('_glu', 0.5), ('_dglu', 3.0)):
+                if name.endswith(suffix):
+                    nbytes += more * m['rows'] * slots_scale * m['n'] * m['elem']
             gemm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, flops_per_launch=flops,
                               tflops=round(flops / (avg_ms * 1e-3) / 1e12, 1),
                               frac_of_mfma_peak=round(flops / (avg_ms * 1e-3) / MFMA_PEAK[dn], 4),
