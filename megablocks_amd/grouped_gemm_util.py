@@ -166,11 +166,12 @@ ACT_GELU_TANH = 1   # mbx_activation of include/mbx.h
 # False: gmm_act / gmm_dact run the product and the element-wise pass as two launches (what they do anyway for shapes
 # the epilogue kernels do not take); a switch for measurements
 ACTIVATION_EPILOGUES = os.environ.get('MBX_ACTIVATION_EPILOGUES', '1') != '0'
-# The epilogue costs every output tile some 19 k (activation) to 37 k (its gradient) cycles in which the matrix cores
-# idle; the separate pass it replaces costs a trip of the [rows, n] tensor through memory.  Tensors that fit the
-# part's 256 MiB Infinity Cache make that trip cheaply (c2's 128 MiB intermediate: the layer step is 2 % faster with
-# the two passes), so the epilogues are used from this size on (c5's 1.5 GiB: 3.7 % faster with them).
-ACTIVATION_EPILOGUE_MIN_BYTES = 256 << 20
+# The epilogue's arithmetic is exposed (the matrix cores idle meanwhile), the separate pass it replaces costs a launch
+# and a trip of the [rows, n] tensor through memory or, for tensors that fit it, the 256 MiB Infinity Cache.  With the
+# epilogue's inputs fetched ahead the epilogues win at every size measured (c2's 128 MiB intermediate: layer step
+# -1.3 %; c5's 1.5 GiB: -4.5 %; c3 / c4, gated: -2.6 % / -5.9 %), so the threshold is zero; it stays as a switch for
+# measurements.
+ACTIVATION_EPILOGUE_MIN_BYTES = int(os.environ.get('MBX_ACTIVATION_EPILOGUE_MIN_BYTES', 0))
 
 
 def _use_epilogue(fuse, a, rows, n):

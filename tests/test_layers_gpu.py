@@ -116,8 +116,8 @@ def test_dmoe_forward_backward_vs_oracle(syn, tokens, hidden, ffn, experts, top_
 @pytest.mark.parametrize('mlp_impl,memopt', [('grouped', False), ('grouped', True), ('sparse', False), ('sparse', True)])
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 def test_dmoe_mlp_with_activation_epilogues_vs_oracle(syn, monkeypatch, mlp_impl, memopt, dtype):
-    """The GELU expert MLP with the activation and its gradient in the epilogues of the grouped products (taken by
-    itself only for intermediates beyond the Infinity Cache; forced here) against the oracle, forward and backward."""
+    """The GELU expert MLP with the activation and its gradient in the epilogues of the grouped products (a size
+    threshold can switch them off; set to zero here) against the oracle, forward and backward."""
     from megablocks_amd import grouped_gemm_util as gg
     monkeypatch.setattr(gg, 'ACTIVATION_EPILOGUE_MIN_BYTES', 0)
     w = syn.Workload('t', 1500, 256, 768, 8, 2, 'mlp', mlp_impl, dtype, 'logits')
@@ -146,8 +146,8 @@ def test_dmoe_mlp_with_activation_epilogues_vs_oracle(syn, monkeypatch, mlp_impl
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 def test_dmoe_glu_with_the_gate_in_the_epilogues_vs_oracle(syn, monkeypatch, mlp_impl, memopt, dtype):
     """The gated experts with the gated activation in the epilogue of the launch that computes both of its products,
-    and its backward in the epilogue of the product that feeds it (taken by themselves only for intermediates beyond
-    the Infinity Cache; forced here) against the oracle, forward and backward."""
+    and its backward in the epilogue of the product that feeds it (a size threshold can switch them off; set to zero here)
+    against the oracle, forward and backward."""
     from megablocks_amd import grouped_gemm_util as gg
     monkeypatch.setattr(gg, 'ACTIVATION_EPILOGUE_MIN_BYTES', 0)
     w = syn.Workload('t', 1500, 256, 768, 8, 2, 'glu', mlp_impl, dtype, 'logits')
