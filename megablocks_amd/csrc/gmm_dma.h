@@ -1412,6 +1412,13 @@ static inline TnBlocks tn_block_shape(int tiles_m, int tiles_n) {
   TnBlocks best{tiles_m < kTnBlockM ? (tiles_m > 0 ? tiles_m : 1) : kTnBlockM, tiles_n < kTnBlockN ? (tiles_n > 0 ? tiles_n : 1) : kTnBlockN};
   const int64_t raw = (int64_t)tiles_m * tiles_n;
   if (raw >= (int64_t)kXcds * kTnBlockM * kTnBlockN || raw <= kXcds) return best;
+  // the search takes tens of microseconds: the last few answers are kept (per thread; a layer alternates between two
+  // or three shapes)
+  struct Known { int tiles_m, tiles_n; TnBlocks shape; };
+  static thread_local Known known[8];
+  static thread_local int next_slot = 0;
+  for (const Known& kn : known)
+    if (kn.tiles_m == tiles_m && kn.tiles_n == tiles_n) return kn.shape;
   int64_t best_fullest = -1, best_panels = -1;
   for (int bm = 1; bm <= kTnBlockM && bm <= tiles_m; ++bm) {
     for (int bn = 1; bn <= kTnBlockM && bn <= tiles_n; ++bn) {
@@ -1438,6 +1445,8 @@ static inline TnBlocks tn_block_shape(int tiles_m, int tiles_n) {
       }
     }
   }
+  known[next_slot] = Known{tiles_m, tiles_n, best};
+  next_slot = (next_slot + 1) % 8;
   return best;
 }
 static inline int64_t tn_grid(int tiles_m, int tiles_n, TnBlocks shape, int num_groups, int chunk) {
