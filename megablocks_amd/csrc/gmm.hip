@@ -730,8 +730,8 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
   if (layout == MBX_NN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (layout == MBX_TN) fast = fast && k % 8 == 0 && n % 8 == 0;
   if (fast) {
-    // direct-to-LDS kernels: whole K tiles (NN / NT)
-    bool dma_ok = dma_sizes_ok(k, n);
+    // direct-to-LDS kernels: whole K tiles (NN / NT); their epilogue writes 16-byte pieces of the output's rows
+    bool dma_ok = dma_sizes_ok(k, n) && aligned16(c) && n % 8 == 0;
     if (layout != MBX_TN) dma_ok = dma_ok && k % TileDma::BK == 0;
     if (dma_ok) {
       // TN: the half-height tile only when the product has at most 128 rows (it is slower otherwise)
@@ -770,8 +770,8 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
   if (!bins || !c || (k > 0 && (!a || !b || !a2 || !b2))) return MBX_EINVAL;
   if (rows > 0x7fffffff) return MBX_ERANGE;
   // only the direct-to-LDS kernels reduce over two operand pairs: whole K tiles, at least four per pair
-  const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(a2) && aligned16(b2) &&
-                  k % TileDma::BK == 0 && k >= 4 * TileDma::BK && (layout == MBX_NT || n % 8 == 0) && dma_sizes_ok(k, n);
+  const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(a2) && aligned16(b2) && aligned16(c) &&
+                  k % TileDma::BK == 0 && k >= 4 * TileDma::BK && n % 8 == 0 && dma_sizes_ok(k, n);
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   const bool small_m = half_height_only(rows, num_groups, n);

@@ -897,7 +897,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 }
 
 // c[m][n] = acc for m < m_lim, n < n_lim, where m = m_base + (row inside the tile) and
-// n = n_base + (column inside the tile).  Uses the LDS of the operand rings as a staging buffer.
+// n = n_base + (column inside the tile).  Uses the LDS of the operand rings as a staging buffer.  The rows of c must
+// start at multiples of 16 bytes (c 16-byte aligned, ldc a multiple of 8: the launch checks both; outputs that are
+// not go to the kernels of gmm.hip).
 // `extra` (EPI != kEpiNone; laid out like c, same pitch, 16-byte aligned like c): the second output of kEpiAct, the
 // second input of kEpiDact, x1 of kEpiDglu*; `pre2` and `out2` (kEpiDglu* only, laid out alike): x2 and the second
 // output (c gets round(g x2) act'(x1), out2 gets g round(act(x1))).  These take the staged path only (the launch
@@ -918,7 +920,7 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
   constexpr int MF = T::MF, Q = MF == 32 ? 4 : 1;
   const int tile_row = MF == 32 ? (lane & 31) : (lane & 15);
   auto run_col = [&](int q) -> int { return MF == 32 ? q * 8 + (lane >> 5) * 4 : (lane >> 4) * 4; };
-  if ((ldc % 8 == 0) && (((uintptr_t)c & 15u) == 0)) {
+  {
     // Staged through LDS (free by now) so that every global store instruction writes whole rows of the
     // tile: 64 lanes x 16 bytes = two 512-byte row segments, instead of 32 scattered 16-byte pieces.
     __syncthreads();
@@ -1110,33 +1112,6 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
       }
       m += BATCH * ROW_STEP;
       off += BATCH * off_step;
-    }
-  } else {
-    const bool n_vec = (ldc % 4 == 0) && (((uintptr_t)c & 7u) == 0);
-#pragma unroll
-    for (int i = 0; i < T::TM; ++i) {
-      const int m = m_base + wm + i * MF + tile_row;
-      if (m >= m_lim) continue;
-      uint16_t* crow = c + (int64_t)m * ldc;
-#pragma unroll
-      for (int j = 0; j < T::TN; ++j) {
-#pragma unroll
-        for (int q = 0; q < Q; ++q) {
-          const int n = n_base + wn + j * MF + run_col(q);
-          const typename T::Acc& v = acc[i][j];
-          const int o = MF == 32 ? q * 4 : 0;
-          if (n + 3 < n_lim && n_vec) {
-            u32x2 w;
-            w[0] = pack2<DT>(v[o + 0], v[o + 1]);
-            w[1] = pack2<DT>(v[o + 2], v[o + 3]);
-            *(u32x2*)(crow + n) = w;
-          } else {
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-              if (n + t < n_lim) crow[n + t] = (uint16_t)(pack2<DT>(v[o + t], 0.f) & 0xffffu);
-          }
-        }
-      }
     }
   }
 }
