@@ -555,7 +555,7 @@ def test_gmm_on_the_32x32x16_instruction():
 
 EPILOGUE = [  # groups, rows, k, n -- full and half-height tiles, partial last column tile, shapes off the fused path
     (8, 4096, 1024, 4096), (64, 16384, 1024, 1024), (5, 1500, 320, 264), (3, 700, 128, 1408), (1, 37, 64, 8),
-    (4, 1000, 72, 256), (16, 6000, 2048, 520),
+    (4, 1000, 72, 256), (16, 6000, 2048, 520), (72, 5000, 128, 264),
 ]
 
 
