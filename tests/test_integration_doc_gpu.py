@@ -1,6 +1,6 @@
-"""Executes the binding INTEGRATION.md documents: the `megablocks_ops.py` stand-in of section 1 and the `gmm` of
-section 3 are cut out of the document, loaded as a module, and held to the oracle.  What the document shows a
-maintainer therefore cannot drift from include/mbx.h."""
+"""Executes the reference-side binding that the integration guide at the repository root documents: its
+`megablocks_ops.py` stand-in and its `gmm` are cut out of the guide's python blocks, loaded as a module, and held to the
+oracle.  What the guide shows a maintainer of the reference therefore cannot drift from include/mbx.h."""
 import os
 import re
 import types
@@ -13,19 +13,20 @@ import oracle
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GUIDE = 'INTEGRATION.md'
 
 
 @pytest.fixture(scope='module')
 def documented():
     from megablocks_amd import _lib
-    text = open(os.path.join(ROOT, 'INTEGRATION.md')).read()
+    text = open(os.path.join(ROOT, GUIDE)).read()
     blocks = re.findall(r'```python\n(.*?)```', text, flags=re.S)
     ops_src = next(b for b in blocks if b.lstrip().startswith('# megablocks_ops.py'))
     gmm_src = next(b for b in blocks if 'def gmm(' in b)
     assert "ctypes.CDLL('libmbx.so')" in ops_src
     mod = types.ModuleType('megablocks_ops')
-    exec(compile(ops_src.replace("'libmbx.so'", repr(_lib.LIB_PATH)), 'INTEGRATION.md#1', 'exec'), mod.__dict__)
-    exec(compile(gmm_src, 'INTEGRATION.md#3', 'exec'), mod.__dict__)      # uses the helpers of the first block
+    exec(compile(ops_src.replace("'libmbx.so'", repr(_lib.LIB_PATH)), GUIDE + '#ops', 'exec'), mod.__dict__)
+    exec(compile(gmm_src, GUIDE + '#gmm', 'exec'), mod.__dict__)      # uses the helpers of the first block
     return mod
 
 
