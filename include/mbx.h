@@ -259,9 +259,11 @@ int mbx_glu_backward(const void* g, const void* a, const void* b, void* da, void
  *   weights = weights / norm(weights, p = norm_p, dim=-1)   if norm_p > 0        router.py:100-106
  * computed in fp32 and rounded to `dtype` where torch's operations round (scores; the norm; the quotient).
  * Weights come out in descending order; equal scores are taken in ascending expert index.  indices are
- * int64 like torch.topk's.  num_experts up to 512 and top_k up to 64, else MBX_EUNSUPPORTED. */
+ * int64 like torch.topk's; indices32 (NULL: not wanted) receives the same values as int32, which saves the layer the
+ * `top_expert.int()` pass of megablocks/layers/moe.py:160.  num_experts up to 512 and top_k up to 64, else
+ * MBX_EUNSUPPORTED. */
 int mbx_router_forward(const void* logits, int dtype, int64_t tokens, int num_experts, int top_k, float norm_p,
-                       void* scores, void* weights, int64_t* indices, mbx_stream_t stream);
+                       void* scores, void* weights, int64_t* indices, int32_t* indices32, mbx_stream_t stream);
 
 /* Backward of the above as autograd derives it for router.py:98-106: grad_logits from grad_weights
  * [tokens, top_k] (NULL: none) and, optionally, a gradient that reaches `scores` directly (NULL: none;

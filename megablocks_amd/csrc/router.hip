@@ -31,7 +31,8 @@ __device__ __forceinline__ float wave_pnorm(float w, bool live, float p) {
 template <int DT, int R>
 __global__ void __launch_bounds__(kTokenThreads)
 router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_experts, int top_k, float p,
-                      void* __restrict__ scores_, void* __restrict__ weights_, int64_t* __restrict__ indices) {
+                      void* __restrict__ scores_, void* __restrict__ weights_, int64_t* __restrict__ indices,
+                      int32_t* __restrict__ indices32) {
   typedef typename Elem<DT>::type E;
   const E* logits = (const E*)logits_;
   E* scores = (E*)scores_;
@@ -93,6 +94,7 @@ router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_
     if (live) {
       weights[t * top_k + lane] = Elem<DT>::from_f32(my_w);
       indices[t * top_k + lane] = my_i;
+      if (indices32) indices32[t * top_k + lane] = my_i;   // what the routing kernels take, without a cast pass
     }
   }
 }
@@ -195,14 +197,14 @@ using namespace mbx;
 extern "C" {
 
 int mbx_router_forward(const void* logits, int dtype, int64_t tokens, int num_experts, int top_k, float norm_p,
-                       void* scores, void* weights, int64_t* indices, mbx_stream_t stream) {
+                       void* scores, void* weights, int64_t* indices, int32_t* indices32, mbx_stream_t stream) {
   if (tokens < 0 || num_experts <= 0 || top_k <= 0 || top_k > num_experts || !(norm_p >= 0.f)) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
   if (num_experts > kMaxRouterExperts || top_k > kWave) return MBX_EUNSUPPORTED;
   if (tokens == 0) return 0;
   if (!logits || !scores || !weights || !indices) return MBX_EINVAL;
   hipStream_t s = as_stream(stream);
-  MBX_ROUTER_DISPATCH(router_forward_kernel, logits, tokens, num_experts, top_k, norm_p, scores, weights, indices);
+  MBX_ROUTER_DISPATCH(router_forward_kernel, logits, tokens, num_experts, top_k, norm_p, scores, weights, indices, indices32);
   return launch_status();
 }
 

@@ -149,5 +149,5 @@ class MoE(torch.nn.Module):
 
     def forward(self, x: torch.Tensor):
         x = common.cast_if_autocast_enabled(x)
-        scores, expert_weights, top_experts = self.router(x)
-        return self.experts(x, scores, expert_weights, top_experts)
+        scores, expert_weights, top_experts, top_experts32 = self.router.route(x)
+        return self.experts(x, scores, expert_weights, top_experts if top_experts32 is None else top_experts32)

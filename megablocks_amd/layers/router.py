@@ -99,7 +99,8 @@ class _RouterLinear(torch.autograd.Function):
 
 class _SoftmaxTopK(torch.autograd.Function):
     """softmax -> top-k -> optional p-norm renormalisation (router.py:87-106) as one kernel each way.
-    Returns (scores, expert_weights, expert_indices) with torch's shapes and dtypes (int64 indices)."""
+    Returns (scores, expert_weights, expert_indices, expert_indices as int32) with torch's shapes and dtypes (int64
+    indices); the int32 copy, written by the same kernel, is what the layer's routing takes (moe.py:160 casts)."""
 
     @staticmethod
     def supported(logits: torch.Tensor, top_k: int) -> bool:
@@ -113,17 +114,18 @@ class _SoftmaxTopK(torch.autograd.Function):
         scores = torch.empty_like(logits)
         weights = torch.empty((tokens, top_k), dtype=logits.dtype, device=logits.device)
         indices = torch.empty((tokens, top_k), dtype=torch.int64, device=logits.device)
+        indices32 = torch.empty((tokens, top_k), dtype=torch.int32, device=logits.device)
         with _lib.device_of(logits):
             _lib.check(_lib.lib.mbx_router_forward(_lib.ptr(logits), _lib.dtype_of(logits), tokens, experts, top_k,
                                                    float(norm_p), _lib.ptr(scores), _lib.ptr(weights), _lib.ptr(indices),
-                                                   _lib.stream()), 'router_forward')
+                                                   _lib.ptr(indices32), _lib.stream()), 'router_forward')
         ctx.save_for_backward(scores, indices)
         ctx.top_k, ctx.norm_p = top_k, float(norm_p)
-        ctx.mark_non_differentiable(indices)
-        return scores, weights, indices
+        ctx.mark_non_differentiable(indices, indices32)
+        return scores, weights, indices, indices32
 
     @staticmethod
-    def backward(ctx: Any, grad_scores, grad_weights, _grad_indices):
+    def backward(ctx: Any, grad_scores, grad_weights, _grad_indices, _grad_indices32):
         scores, indices = ctx.saved_tensors
         tokens, experts = scores.shape
         grad_logits = torch.empty_like(scores)
@@ -157,6 +159,11 @@ class LearnedRouter(torch.nn.Module):
         return torch.topk(scores, self.args.moe_top_k, dim=-1)
 
     def forward(self, x: torch.Tensor):
+        return self.route(x)[:3]
+
+    def route(self, x: torch.Tensor):
+        """forward's (scores, expert_weights, expert_indices) and, where the router kernel wrote them, the indices as
+        int32 (else None): the layer routes with those and skips the cast of moe.py:160."""
         if self.training and self.args.moe_jitter_eps is not None:
             x = x * self.jitter(x)
         x2d = x.view(-1, x.shape[-1])
@@ -168,8 +175,9 @@ class LearnedRouter(torch.nn.Module):
         if logits.is_cuda and logits.dtype != torch.float32 and torch.is_autocast_enabled():
             # autocast runs softmax in fp32 (router.py:98 under torch.autocast): scores and weights come out in fp32
             logits = logits.float()
+        expert_indices32 = None
         if FUSED_SOFTMAX_TOPK and _SoftmaxTopK.supported(logits, self.args.moe_top_k):
-            scores, expert_weights, expert_indices = _SoftmaxTopK.apply(
+            scores, expert_weights, expert_indices, expert_indices32 = _SoftmaxTopK.apply(
                 logits, self.args.moe_top_k, self.args.moe_normalize_expert_weights or 0)
         else:
             scores = logits.softmax(dim=-1)
@@ -179,4 +187,5 @@ class LearnedRouter(torch.nn.Module):
                     expert_weights, p=self.args.moe_normalize_expert_weights, dim=-1, keepdim=True)
         if self.args.uniform_expert_assignment:
             expert_indices = _UniformExpertAssignment.apply(expert_indices, self.args.moe_num_experts)
-        return scores, expert_weights, expert_indices
+            expert_indices32 = None
+        return scores, expert_weights, expert_indices, expert_indices32

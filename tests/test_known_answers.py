@@ -145,4 +145,4 @@ def test_library_permute():
 @pytest.mark.gpu
 def test_library_router():
     from megablocks_amd.layers.router import _SoftmaxTopK
-    _check_router(lambda logits, k, p: _SoftmaxTopK.apply(logits, k, p), True, True)
+    _check_router(lambda logits, k, p: _SoftmaxTopK.apply(logits, k, p)[:3], True, True)

@@ -221,7 +221,8 @@ def test_router_softmax_topk_fp32_matches_oracle(tokens, experts, top_k, norm_p)
     torch.manual_seed(tokens + experts)
     logits = torch.randn(tokens, experts) * 3
     want_s, want_w, want_i = oracle.router_forward(logits, torch.eye(experts), top_k, norm_p or None)
-    s, w, i = _SoftmaxTopK.apply(logits.cuda(), top_k, norm_p)
+    s, w, i, i32 = _SoftmaxTopK.apply(logits.cuda(), top_k, norm_p)
+    assert i32.dtype == torch.int32 and torch.equal(i32.long(), i)
     assert s.dtype == torch.float32 and w.shape == (tokens, top_k) and i.dtype == torch.int64
     assert torch.allclose(s.cpu(), want_s, rtol=1e-5, atol=1e-7)
     assert torch.equal(i.cpu(), want_i)                      # fp32 scores of random logits have no ties
@@ -237,7 +238,7 @@ def test_router_softmax_topk_16bit(dtype, tokens, experts, top_k, norm_p):
     from megablocks_amd.layers.router import _SoftmaxTopK
     torch.manual_seed(experts)
     logits = (torch.randn(tokens, experts, device='cuda') * 2).to(dtype)
-    s, w, i = _SoftmaxTopK.apply(logits, top_k, norm_p)
+    s, w, i, _ = _SoftmaxTopK.apply(logits, top_k, norm_p)
     ref_s, _, _ = _softmax_topk_reference(logits, top_k, norm_p)
     ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     assert ((s.float() - ref_s.float()).abs() <= ulp * ref_s.float().abs() + 1e-30).all()   # at most one rounding step apart
@@ -259,7 +260,7 @@ def test_router_softmax_topk_backward(dtype, experts, top_k, norm_p, with_score_
     gw = torch.randn(tokens, top_k, device='cuda').to(dtype)
     gs = torch.randn(tokens, experts, device='cuda').to(dtype) if with_score_grad else None
     x = logits.clone().requires_grad_(True)
-    s, w, i = _SoftmaxTopK.apply(x, top_k, norm_p)
+    s, w, i, _ = _SoftmaxTopK.apply(x, top_k, norm_p)
     loss = (w.float() * gw.float()).sum() + ((s.float() * gs.float()).sum() if with_score_grad else 0)
     loss.backward()
     # reference: autograd through torch's operations in fp32, with the kernel's selection
@@ -287,7 +288,8 @@ def test_router_softmax_topk_with_nan_and_inf_logits(dtype):
     bad[3, 5] = float('nan')
     bad[10, 0] = float('inf')
     bad[20, :] = float('nan')
-    s, w, i = _SoftmaxTopK.apply(bad, top_k, 1)
+    s, w, i, i32 = _SoftmaxTopK.apply(bad, top_k, 1)
+    assert torch.equal(i32.long(), i)
     assert int(i.min()) >= 0 and int(i.max()) < experts
     assert bool((i[:, 0] != i[:, 1]).all())
     ref_s = bad.float().softmax(-1)
