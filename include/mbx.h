@@ -55,6 +55,22 @@ size_t mbx_sort_scratch_bytes(int64_t n, int itype, int end_bit);
 int mbx_sort(const void* x, int itype, int64_t n, int end_bit, void* keys_out,
              void* perm_out, void* scratch, size_t scratch_bytes, mbx_stream_t stream);
 
+/* The routing bookkeeping of one layer step, megablocks/layers/moe.py:152-183 (`indices_and_bins`) and
+ * megablocks/layers/dmoe.py:131-154 (`indices_and_padded_bins`), in three launches instead of the seven of
+ * sort + histogram + the cumsums + mbx_slot_rows.  For int32 expert ids [n] in [0, num_experts):
+ *   bin_ids, indices      = sort(expert_ids, end_bit)                      (csrc/sort.h:59)
+ *   tokens_per_expert     = histogram(expert_ids, num_experts)             (csrc/histogram.h:61)
+ *   bins                  = inclusive_cumsum(tokens_per_expert)            (csrc/cumsum.h:131)
+ *   padded_bins           = inclusive_cumsum(round_up(tokens_per_expert, pad))   if pad > 0 (else not written; may be NULL)
+ *   slot_rows (or NULL)   = what mbx_slot_rows builds from these (with padded_bins if pad > 0)
+ * bit for bit what the separate entry points give.  An id outside [0, num_experts) is a caller's error here: it is
+ * sorted by its low end_bit bits like mbx_sort does, but counted where mbx_histogram would drop it.
+ * scratch: mbx_sort_scratch_bytes(n, MBX_I32, end_bit) bytes.  MBX_EUNSUPPORTED (use the separate entry points):
+ * end_bit above 8 or num_experts above 2^end_bit. */
+int mbx_route(const int32_t* expert_ids, int64_t n, int num_experts, int end_bit, int pad, int32_t* indices,
+              int32_t* bin_ids, int32_t* tokens_per_expert, int32_t* bins, int32_t* padded_bins,
+              int32_t* slot_rows, void* scratch, size_t scratch_bytes, mbx_stream_t stream);
+
 /* csrc/cumsum.h:104-156 `inclusive_cumsum / exclusive_cumsum(x, dim=1, out)`: scan of
  * every row of x [rows, n]. */
 int mbx_cumsum(const void* x, int itype, int64_t rows, int64_t n, int exclusive, void* out,

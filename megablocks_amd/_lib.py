@@ -27,6 +27,7 @@ _SIGNATURES = {
     'mbx_histogram': (_i, [_vp, _i, _i64, _i64, _i, _vp, _vp]),
     'mbx_sort_scratch_bytes': (_sz, [_i64, _i, _i]),
     'mbx_sort': (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _sz, _vp]),
+    'mbx_route': (_i, [_vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     'mbx_cumsum': (_i, [_vp, _i, _i64, _i64, _i, _vp, _vp]),
     'mbx_topology': (_i, [_vp, _i, _i, _i, _i, _vp, _vp]),
     'mbx_replicate_forward': (_i, [_vp, _i, _i64, _i, _vp, _vp, _i64, _vp]),

@@ -41,6 +41,22 @@ def _scratch(n_slots, device):
     return torch.empty(max(n_slots, 1), dtype=torch.int32, device=device)
 
 
+def _slot_rows_key(indices, bins, padded_bins):
+    return (indices._version, bins.data_ptr(), bins._version,
+            None if padded_bins is None else (padded_bins.data_ptr(), padded_bins._version))
+
+
+def remember_slot_rows(indices, bins, padded_bins, rows):
+    """Leaves a slot -> row map that was built together with `indices` (ops.route) where _slot_rows looks for it.
+    Not under stream capture, where nothing is kept (see _slot_rows)."""
+    if torch.cuda.is_current_stream_capturing():
+        return
+    try:
+        indices._mbx_slot_rows = (_slot_rows_key(indices, bins, padded_bins), rows, bins, padded_bins)
+    except AttributeError:
+        pass
+
+
 def _slot_rows(indices, bin_ids, bins, padded_bins):
     """int32 [n_slots]: the row of the expert-major (optionally padded) buffer that holds each slot.  One map
     serves all gathers and scatters of a routing decision, forward and backward, so it is kept on the `indices`
@@ -50,8 +66,7 @@ def _slot_rows(indices, bin_ids, bins, padded_bins):
     call gets a new map for every call.  Under stream capture nothing is reused or kept: a captured graph has to
     contain the kernels that build its map."""
     capturing = torch.cuda.is_current_stream_capturing()
-    key = (indices._version, bins.data_ptr(), bins._version,
-           None if padded_bins is None else (padded_bins.data_ptr(), padded_bins._version))
+    key = _slot_rows_key(indices, bins, padded_bins)
     cached = getattr(indices, '_mbx_slot_rows', None)
     if not capturing and cached is not None and cached[0] == key:
         return cached[1]

@@ -152,8 +152,8 @@ radix_count_kernel(const T* __restrict__ keys, int64_t n, int shift, uint32_t ma
   counts[(int64_t)threadIdx.x * nblocks + blockIdx.x] = hist[threadIdx.x];
 }
 
-// Pass step 2: exclusive scan, in place, of the digit-major count table (one block).
-__global__ void __launch_bounds__(1024) exclusive_scan_i32_kernel(int32_t* __restrict__ data, int64_t n) {
+// Pass step 2: exclusive scan, in place, of the digit-major count table (one block of 1024 threads).
+__device__ __forceinline__ void block_exclusive_scan_i32(int32_t* __restrict__ data, int64_t n) {
   __shared__ int32_t wave_tot[16];
   __shared__ int32_t carry_s;
   if (threadIdx.x == 0) carry_s = 0;
@@ -174,14 +174,54 @@ __global__ void __launch_bounds__(1024) exclusive_scan_i32_kernel(int32_t* __res
     __syncthreads();
   }
 }
+__global__ void __launch_bounds__(1024) exclusive_scan_i32_kernel(int32_t* __restrict__ data, int64_t n) {
+  block_exclusive_scan_i32(data, n);
+}
+
+// The same scan for the one-pass sort of expert ids, which then also knows what histogram and the cumsums of the
+// routing step would compute (megablocks/layers/moe.py:167-176, dmoe.py:137-153): after the scan, entry [d][0] of the
+// table is the number of ids with a digit below d, so
+//   tokens_per_expert[e] = table[e + 1][0] - table[e][0],   bins[e] = table[e + 1][0]        (table[ndigits][0] := n)
+// for ids inside [0, num_experts), and padded_bins = cumsum(round_up(tokens_per_expert, pad)) when pad > 0.
+__global__ void __launch_bounds__(1024)
+route_scan_kernel(int32_t* __restrict__ table, int ndigits, int nblocks, int32_t n, int num_experts, int pad,
+                  int32_t* __restrict__ tokens_per_expert, int32_t* __restrict__ bins, int32_t* __restrict__ padded_bins) {
+  __shared__ int32_t padded[1024];
+  block_exclusive_scan_i32(table, (int64_t)ndigits * nblocks);
+  __syncthreads();
+  const int e = threadIdx.x;
+  int32_t count = 0;
+  if (e < num_experts) {
+    const int32_t start = e < ndigits ? table[(int64_t)e * nblocks] : n;
+    const int32_t next = e + 1 < ndigits ? table[(int64_t)(e + 1) * nblocks] : n;
+    count = next - start;
+    tokens_per_expert[e] = count;
+    bins[e] = next;
+  }
+  if (pad > 0 && padded_bins != nullptr) {
+    padded[e] = e < num_experts ? (count + pad - 1) / pad * pad : 0;
+    __syncthreads();
+    if (e < num_experts) {
+      int32_t run = 0;
+      for (int j = 0; j <= e; ++j) run += padded[j];
+      padded_bins[e] = run;
+    }
+  }
+}
 
 // Pass step 3: stable scatter.  Wave w of a block owns kSortItems consecutive rounds of 64
 // consecutive keys, so "earlier key" means earlier wave, then earlier round, then lower lane.
+// slot_rows (with IOTA, i.e. on the first pass, whose values are the key's positions in the input; NULL: not wanted):
+// also writes, for the key at input position i that lands at sorted position p, the row of the expert-major buffer
+// that holds it: p itself, or with padded_bins the row p - bins[e - 1] + padded_bins[e - 1] of expert e's padded
+// block (-1 for an expert id outside [0, num_bins)) -- the map inverse_map_kernel of the permutation kernels builds.
 template <typename T, bool IOTA>
 __global__ void __launch_bounds__(kSortThreads)
 radix_scatter_kernel(const T* __restrict__ keys_in, const T* __restrict__ vals_in, int64_t n,
                      int shift, uint32_t mask, int nbits, const int32_t* __restrict__ offsets,
-                     int nblocks, T* __restrict__ keys_out, T* __restrict__ vals_out) {
+                     int nblocks, T* __restrict__ keys_out, T* __restrict__ vals_out,
+                     int32_t* __restrict__ slot_rows = nullptr, const int32_t* __restrict__ bins = nullptr,
+                     const int32_t* __restrict__ padded_bins = nullptr, int num_bins = 0) {
   __shared__ int32_t wave_hist[kSortWaves][kRadix];
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   for (int w = 0; w < kSortWaves; ++w) wave_hist[w][threadIdx.x] = 0;
@@ -225,6 +265,15 @@ radix_scatter_kernel(const T* __restrict__ keys_in, const T* __restrict__ vals_i
     if (valid) {
       keys_out[pos] = key[it];
       vals_out[pos] = IOTA ? (T)i : vals_in[i];
+      if (IOTA && slot_rows != nullptr) {
+        int32_t row = pos;
+        if (padded_bins != nullptr) {
+          const int64_t e = (int64_t)key[it];
+          if (e < 0 || e >= num_bins) row = -1;
+          else if (e > 0) row = pos - bins[e - 1] + padded_bins[e - 1];
+        }
+        slot_rows[i] = row;
+      }
     }
   }
 }
@@ -421,6 +470,32 @@ int mbx_sort(const void* x, int itype, int64_t n, int end_bit, void* keys_out, v
     case MBX_I64: return sort_impl<int64_t>((const int64_t*)x, n, end_bit, (int64_t*)keys_out, (int64_t*)perm_out, scratch, scratch_bytes, s);
   }
   return MBX_EINVAL;
+}
+
+int mbx_route(const int32_t* expert_ids, int64_t n, int num_experts, int end_bit, int pad, int32_t* indices,
+              int32_t* bin_ids, int32_t* tokens_per_expert, int32_t* bins, int32_t* padded_bins, int32_t* slot_rows,
+              void* scratch, size_t scratch_bytes, mbx_stream_t stream) {
+  if (n < 0 || num_experts <= 0 || end_bit <= 0 || pad < 0) return MBX_EINVAL;
+  // one 8-bit pass whose digits are the expert ids themselves
+  if (end_bit > kRadixBits || num_experts > (1 << end_bit)) return MBX_EUNSUPPORTED;
+  if (!tokens_per_expert || !bins || (pad > 0 && !padded_bins)) return MBX_EINVAL;
+  if (n > 0 && (!expert_ids || !indices || !bin_ids)) return MBX_EINVAL;
+  if (n > 0x7fffffff - kSortTile) return MBX_ERANGE;
+  hipStream_t s = as_stream(stream);
+  const int nblocks = n > 0 ? (int)ceil_div(n, kSortTile) : 1;
+  if (scratch_bytes < (size_t)kRadix * nblocks * sizeof(int32_t) || scratch == nullptr) return MBX_ESCRATCH;
+  int32_t* counts = (int32_t*)scratch;
+  const uint32_t mask = (1u << end_bit) - 1u;
+  const int ndigits = 1 << end_bit;
+  // (n = 0: a table of zeros makes every count and bound zero)
+  radix_count_kernel<int32_t><<<nblocks, kSortThreads, 0, s>>>(expert_ids, n, 0, mask, end_bit, counts, nblocks);
+  route_scan_kernel<<<1, 1024, 0, s>>>(counts, ndigits, nblocks, (int32_t)n, num_experts, pad, tokens_per_expert, bins,
+                                       pad > 0 ? padded_bins : nullptr);
+  if (n > 0)
+    radix_scatter_kernel<int32_t, true><<<nblocks, kSortThreads, 0, s>>>(expert_ids, nullptr, n, 0, mask, end_bit, counts, nblocks,
+                                                                        bin_ids, indices, slot_rows, bins,
+                                                                        pad > 0 ? padded_bins : nullptr, num_experts);
+  return launch_status();
 }
 
 int mbx_cumsum(const void* x, int itype, int64_t rows, int64_t n, int exclusive, void* out, mbx_stream_t stream) {

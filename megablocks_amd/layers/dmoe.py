@@ -8,6 +8,7 @@ import numpy as np
 import torch
 
 import megablocks_amd.ops as ops
+from megablocks_amd.ops import routing as ops_routing
 from megablocks_amd import grouped_gemm_util as gg
 from megablocks_amd.layers import common, dmlp_registry, moe, mpu
 from megablocks_amd.layers.arguments import Arguments
@@ -76,6 +77,10 @@ class ParallelDroplessMLP(moe.ParallelMLP):
     def indices_and_padded_bins(self, top_experts):
         """dmoe.py:131-154."""
         top_experts = top_experts.int()
+        if ops_routing.route_supported(top_experts, self.num_experts, self.sort_end_bit):
+            indices, bin_ids, tokens_per_expert, bins, padded_bins = ops_routing.route(
+                top_experts, self.num_experts, self.sort_end_bit, self.blocking)
+            return indices, bin_ids, bins, padded_bins, tokens_per_expert
         bin_ids, indices = ops.sort(top_experts, self.sort_end_bit)
         tokens_per_expert = ops.histogram(top_experts, self.num_experts)
         padded_tokens_per_expert = ops.round_up(tokens_per_expert, self.blocking)

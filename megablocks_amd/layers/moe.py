@@ -6,6 +6,7 @@ import numpy as np
 import torch
 
 import megablocks_amd.ops as ops
+from megablocks_amd.ops import routing as ops_routing
 from megablocks_amd import grouped_gemm_util as gg
 from megablocks_amd.layers import common, mlp, router
 from megablocks_amd.layers.arguments import Arguments
@@ -92,10 +93,13 @@ class ParallelMLP(torch.nn.Module):
     def indices_and_bins(self, top_expert: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
         """moe.py:152-183 -> (indices, bin_ids, bins, tokens_per_expert), all int32 on the device."""
         top_expert = top_expert.int()
-        bin_ids, indices = ops.sort(top_expert, self.sort_end_bit)
-        tokens_per_expert = ops.histogram(top_expert, self.num_experts)
-        bins = ops.inclusive_cumsum(tokens_per_expert, 0)
-        bins = bins.view(1) if not len(bins.size()) else bins
+        if ops_routing.route_supported(top_expert, self.num_experts, self.sort_end_bit):
+            indices, bin_ids, tokens_per_expert, bins, _ = ops_routing.route(top_expert, self.num_experts, self.sort_end_bit)
+        else:
+            bin_ids, indices = ops.sort(top_expert, self.sort_end_bit)
+            tokens_per_expert = ops.histogram(top_expert, self.num_experts)
+            bins = ops.inclusive_cumsum(tokens_per_expert, 0)
+            bins = bins.view(1) if not len(bins.size()) else bins
         gg.note_bins(tokens_per_expert, bins)     # the grouped products of this step take these row bins
         return indices, bin_ids, bins, tokens_per_expert
 

@@ -75,6 +75,37 @@ class SortOp(torch.autograd.Function):
 sort = SortOp.apply
 
 
+def route_supported(expert_ids: torch.Tensor, num_experts: int, end_bit: int) -> bool:
+    """Whether `route` takes these ids: int32 on the GPU, one 8-bit sort pass whose digits are the expert ids."""
+    return (expert_ids.is_cuda and expert_ids.dtype == torch.int32 and expert_ids.ndim == 1 and
+            0 < end_bit <= 8 and 0 < num_experts <= (1 << end_bit))
+
+
+def route(expert_ids: torch.Tensor, num_experts: int, end_bit: int, blocking: int = 0):
+    """The routing bookkeeping of a layer step (moe.py:152-183, dmoe.py:131-154) in three launches:
+    (indices, bin_ids, tokens_per_expert, bins, padded_bins) with the values `sort`, `histogram`, `inclusive_cumsum`
+    and `round_up` give for ids inside [0, num_experts); padded_bins is None without `blocking`.  The slot -> row map
+    of the permutation kernels comes out of the same launches and is left where they look for it."""
+    from megablocks_amd.backend import kernels
+    n = expert_ids.shape[0]
+    expert_ids = expert_ids.contiguous()
+    dev = expert_ids.device
+    indices = torch.empty(n, dtype=torch.int32, device=dev)
+    bin_ids = torch.empty(n, dtype=torch.int32, device=dev)
+    tokens_per_expert = torch.empty(num_experts, dtype=torch.int32, device=dev)
+    bins = torch.empty(num_experts, dtype=torch.int32, device=dev)
+    padded_bins = torch.empty(num_experts, dtype=torch.int32, device=dev) if blocking else None
+    slot_rows = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
+    with _lib.device_of(expert_ids):
+        nbytes = max(lib.mbx_sort_scratch_bytes(max(n, 1), _lib.I32, end_bit), 1)
+        scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _lib.check(lib.mbx_route(_lib.ptr(expert_ids), n, num_experts, end_bit, int(blocking), _lib.ptr(indices),
+                                 _lib.ptr(bin_ids), _lib.ptr(tokens_per_expert), _lib.ptr(bins), _lib.ptr(padded_bins),
+                                 _lib.ptr(slot_rows), _lib.ptr(scratch), nbytes, _lib.stream()), 'route')
+    kernels.remember_slot_rows(indices, bins, padded_bins, slot_rows)
+    return indices, bin_ids, tokens_per_expert, bins, padded_bins
+
+
 def _cumsum(x, dim, exclusive):
     _lib.require_cuda(x)
     it = _lib.itype_of(x)

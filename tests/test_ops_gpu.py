@@ -460,3 +460,49 @@ def test_routing_chain_matches_the_c_restatement(ops, tokens, experts, top_k):
     pbins = ops.inclusive_cumsum(ops.round_up(tpe, 128), 0).view(-1)
     for got, want in ((indices, want_idx), (bin_ids, want_ids), (tpe, want_tpe), (bins, want_bins), (pbins, want_pbins)):
         assert got.dtype == torch.int32 and torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize('n', [0, 1, 100, 2048, 2049, 16384, 100003])
+@pytest.mark.parametrize('experts', [1, 2, 8, 17, 64, 200, 256])
+@pytest.mark.parametrize('blocking', [0, 128])
+def test_route_equals_the_separate_routing_ops(n, experts, blocking):
+    """ops.route (sort + histogram + cumsums + the slot -> row map in three launches) against the oracle's
+    indices_and_bins / indices_and_padded_bins chain (moe.py:152-183, dmoe.py:131-154) and against the library's own
+    separate entry points, bit for bit."""
+    from megablocks_amd import _lib, ops
+    from megablocks_amd.backend import kernels
+    from megablocks_amd.ops import routing
+    g = torch.Generator().manual_seed(n * 7 + experts)
+    top = torch.randint(0, experts, (n,), generator=g, dtype=torch.int32)
+    if experts > 4:
+        top[top == 3] = 1                                           # an expert without tokens
+    end_bit = max(int(np.ceil(np.log2(experts))), 1)
+    ids = top.cuda()
+    assert routing.route_supported(ids, experts, end_bit)
+    indices, bin_ids, tpe, bins, pbins = routing.route(ids, experts, end_bit, blocking)
+    if blocking:
+        wi, wb, wbins, wpbins, wtpe = oracle.indices_and_padded_bins(top.long(), experts, blocking)
+        assert torch.equal(pbins.cpu(), wpbins.int())
+    else:
+        wi, wb, wbins, wtpe = oracle.indices_and_bins(top.long(), experts)
+        assert pbins is None
+    assert torch.equal(indices.cpu(), wi.int()) and torch.equal(bin_ids.cpu(), wb.int())
+    assert torch.equal(bins.cpu(), wbins.int()) and torch.equal(tpe.cpu(), wtpe.int())
+    assert indices.dtype == torch.int32 and tpe.dtype == torch.int32 and bins.shape == (experts,)
+    # the separate entry points
+    s_bin_ids, s_indices = ops.sort(ids, end_bit)
+    assert torch.equal(s_bin_ids, bin_ids) and torch.equal(s_indices, indices)
+    assert torch.equal(ops.histogram(ids, experts), tpe)
+    # the slot -> row map that came out of the same launches, against mbx_slot_rows
+    if n:
+        kept = indices._mbx_slot_rows[1]
+        del indices._mbx_slot_rows
+        built = kernels._slot_rows(indices, bin_ids, bins, pbins)
+        assert torch.equal(kept[:n], built[:n])
+
+
+def test_route_falls_back_where_it_does_not_apply():
+    from megablocks_amd.ops import routing
+    ids = torch.zeros(8, dtype=torch.int32, device='cuda')
+    assert not routing.route_supported(ids.long(), 8, 3) and not routing.route_supported(ids, 512, 9)
+    assert not routing.route_supported(ids, 9, 3) and not routing.route_supported(ids.cpu(), 8, 3)
