@@ -535,6 +535,18 @@ for dtype in (torch.bfloat16, torch.float16):
         worst = max(worst, rel(gg.backend.gmm(a, bn, sizes), want_nn), rel(gg.backend.gmm(a, bt, sizes, trans_b=True), want_nn),
                     rel(gg.backend.gmm(a, g, sizes, trans_a=True), want_tn), rel(gg.gmm_dual(a, bn, a2, bn2, sizes), want_dual))
         assert int(torch.count_nonzero(gg.backend.gmm(a, g, sizes, trans_a=True)[1])) == 0 or groups <= 2
+        # the epilogue forms: this main loop has the GELU ones; the gated ones fall back to their separate passes
+        x2 = torch.randn(rows, n, device='cuda').to(dtype)
+        p1, act = gg.gmm_act(a, bt, sizes, fuse=True)
+        q1, act2 = gg.gmm_act(a, bt, sizes, fuse=False)
+        assert torch.equal(p1, q1)
+        worst = max(worst, rel(act.float(), act2.float()))
+        x1, xx2, h = gg.gmm_glu(a, bt, bt, sizes, 0, fuse=True)
+        y1, yy2, h2 = gg.gmm_glu(a, bt, bt, sizes, 0, fuse=False)
+        assert torch.equal(x1, y1) and torch.equal(h, h2)
+        d1, d2 = gg.gmm_dglu(a, bt, p1, x2, sizes, 0, fuse=True)
+        e1, e2 = gg.gmm_dglu(a, bt, p1, x2, sizes, 0, fuse=False)
+        assert torch.equal(d1, e1) and torch.equal(d2, e2)
 print('worst', worst)
 assert worst < 1e-2, worst
 '''
@@ -542,7 +554,8 @@ assert worst < 1e-2, worst
 
 def test_gmm_on_the_32x32x16_instruction():
     """MBX_MFMA=32 selects the main loop built on v_mfma_f32_32x32x16 instead of the default 16x16x32 one (read once
-    per process, hence the child process): the three layouts and the two-pair product against fp32 torch."""
+    per process, hence the child process): the three layouts and the two-pair product against fp32 torch, and the
+    epilogue forms against their two-step formulations (the gated ones are two-step under this main loop)."""
     import os
     import subprocess
     import sys
