@@ -506,3 +506,23 @@ def test_route_falls_back_where_it_does_not_apply():
     ids = torch.zeros(8, dtype=torch.int32, device='cuda')
     assert not routing.route_supported(ids.long(), 8, 3) and not routing.route_supported(ids, 512, 9)
     assert not routing.route_supported(ids, 9, 3) and not routing.route_supported(ids.cpu(), 8, 3)
+
+
+@pytest.mark.parametrize('blocking', [0, 128])
+def test_route_with_ids_outside_the_experts_stays_in_range(blocking):
+    """Ids outside [0, num_experts) are a caller's error for ops.route; like ops.sort it orders them by their low bits,
+    and no index it writes may leave its range: positions inside [0, n), rows inside the padded buffer or -1."""
+    from megablocks_amd import ops
+    from megablocks_amd.ops import routing
+    experts, end_bit, n = 12, 4, 5000
+    g = torch.Generator().manual_seed(3)
+    top = torch.randint(-3, experts + 4, (n,), generator=g, dtype=torch.int32)
+    ids = top.cuda()
+    indices, bin_ids, tpe, bins, pbins = routing.route(ids, experts, end_bit, blocking)
+    s_bin_ids, s_indices = ops.sort(ids, end_bit)
+    assert torch.equal(s_bin_ids, bin_ids) and torch.equal(s_indices, indices)
+    assert torch.equal(torch.sort(indices.cpu().long())[0], torch.arange(n))
+    assert int(tpe.min()) >= 0 and int(bins[-1]) <= n and bool((bins[1:] >= bins[:-1]).all())
+    rows = indices._mbx_slot_rows[1][:n].cpu()
+    limit = int(pbins[-1]) if blocking else n
+    assert int(rows.min()) >= -1 and int(rows.max()) < max(limit, n)
