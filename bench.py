@@ -51,6 +51,8 @@ def parse():
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
     ap.add_argument('--graph', action='store_true',
                     help='capture the step (forward + backward) in a HIP graph after the warm-up and time replays of it')
+    ap.add_argument('--forward-only', action='store_true',
+                    help='time the forward pass alone, without gradients (not the headline metric; no CPU baseline)')
     ap.add_argument('--cpu-tokens', type=int, default=None)
     ap.add_argument('--library-gemm', action='store_true',
                     help='also time the three grouped products as per-expert torch.matmul loops (the vendor GEMM library)')
@@ -92,6 +94,14 @@ def gpu_leg(args, w, inp):
         for p in layer.parameters():
             p.grad = None
         synthetic.layer_step(layer, w, x, grad, routing)
+
+    if args.forward_only:
+        if args.graph:
+            sys.exit('bench.py: --graph captures the training step; not with --forward-only')
+
+        def step():
+            with torch.no_grad():
+                return layer(x) if routing is None else layer.experts(x, *routing)
 
     for _ in range(args.warmup):
         step()
@@ -467,10 +477,13 @@ def main():
         roofline = dict(bound='hbm', kernel=dom_name, achieved=dom['gbps'], peak=HBM_PEAK / 1e9, unit='GB/s',
                         frac=dom['frac_of_hbm_peak'], traffic=traffic, traffic_source=traffic_source,
                         bytes_per_launch=dom['bytes_per_launch'], avg_launch_ms=dom['avg_ms'])
-    all_gemm_tflops = w.gemm_flops() / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None
+    step_flops = w.gemm_flops()
+    if args.forward_only:
+        step_flops = sum(g['flops_per_launch'] * g['launches'] for g in gemm.values()) / args.steps
+    all_gemm_tflops = step_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None
 
     out = {
-        'metric': 'dmoe_layer_fwd_bwd_tokens_per_s',
+        'metric': 'dmoe_layer_fwd_tokens_per_s' if args.forward_only else 'dmoe_layer_fwd_bwd_tokens_per_s',
         'value': round(w.tokens / (ms_per_step * 1e-3), 1),
         'unit': 'tokens/s',
         'n_gpus': 1,
@@ -497,7 +510,7 @@ def main():
         out['operand_patterns'] = operand_pattern_leg(w, inp)
     if args.mfma_ceiling:
         out['mfma_ceiling'] = mfma_ceiling_leg()
-    if not args.no_cpu:
+    if not args.no_cpu and not args.forward_only:
         del layer
         torch.cuda.empty_cache()
         out['cpu_baseline'] = cpu_leg(args, w, inp)

@@ -240,6 +240,24 @@ int mbx_gmm_dact(const void* a, const void* b, const void* pre, void* c, int dty
 int mbx_gmm_glu(const void* a, const void* b1, const void* b2, void* x1, void* x2, void* h, int dtype,
                 const int32_t* bins, int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
 
+/* The token gather and the experts' first product(s) in one launch: megablocks/layers/dmoe.py:219 / :273
+ * (`x = ops.padded_gather(x, indices, bin_ids, bins, padded_bins, top_k)` / `ops.gather(...)`) followed by
+ * megablocks/layers/mlp.py:521 (`gmm(x, w1, trans_b=True)`, then the activation) or glu.py:201-204.  The rows of the
+ * product's first operand are read from the ungathered x through the row map, so the gathered copy is never written:
+ *   A[first(e) + r] = x[indices[x_first(e) + r] / top_k]  for r < x_bins[e] - x_first(e),   zeros for the other rows of e
+ * (first(e) = bins[e - 1], x_first(e) = x_bins[e - 1], 0 for e = 0: `bins` are the row bins of the products, `x_bins`
+ * the bins of the sorted assignments `indices` -- padded_bins and bins of dmoe.py:131-154; x_bins NULL = `bins`), then
+ *   b2 == NULL, h == NULL:  c = A[r_e] @ b1[e]^T
+ *   b2 == NULL, h != NULL:  the same and h = act(c) as mbx_gmm_act writes it (act: MBX_ACT_GELU_TANH)
+ *   b2 != NULL:             c, c2, h = x1, x2, h of mbx_gmm_glu (act: MBX_ACT_SILU or MBX_ACT_GELU_TANH)
+ * x: [x_rows, k]; b1, b2: [E, n, k]; c, c2, h: [rows, n].  The results are bit-identical to mbx_gather / mbx_padded_gather
+ * followed by mbx_gmm / mbx_gmm_act / mbx_gmm_glu.  An assignment outside [0, x_rows * top_k) reads as a row of zeros.
+ * MBX_EUNSUPPORTED (the caller gathers and multiplies in two steps): what mbx_gmm_act / mbx_gmm_glu do not take, x of
+ * 2 GiB or more, x_rows * top_k above INT32_MAX, the library running with MBX_MFMA=32. */
+int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int top_k, const int32_t* x_bins,
+                   const void* b1, const void* b2, void* c, void* c2, void* h, int dtype, const int32_t* bins,
+                   int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
+
 /* The backward of the GLU experts' gated activation on the product that feeds it, megablocks/layers/glu.py:135-153
  * (`gmm(ddsd_out, w2, trans_b=True, c=dactivation_fn_out)`, then autograd's gradient of
  * `activation_fn(sdd_out) * v1_out`, glu.py:120-124), in one launch:

@@ -47,6 +47,7 @@ _SIGNATURES = {
     'mbx_gmm_dact': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_glu': (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_dglu': (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
+    'mbx_gmm_gather': (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gelu_backward_inplace': (_i, [_vp, _vp, _i, _i64, _vp]),
     'mbx_glu_forward': (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp]),
     'mbx_glu_backward': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _vp]),

@@ -580,10 +580,16 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
 // TS is the tile the tail of an NN / NT launch is cut into (TS = T: never cut).
 // a2 / b2 non-null (NN / NT only): c = a @ b[e] + a2 @ b2[e], the second pair shaped like the first.
 // epi / extra (NT, one operand pair only): dma::kEpiAct with the second output, dma::kEpiDact with the second input.
+// Rows of `a` gathered on the fly (NT; no epilogue, kEpiAct or kEpiGlu*; 16 x 16 x 32 tiles only): see GatherRows.
+struct GatherRows {
+  const int32_t* slots = nullptr;      // non-null: a is [src_rows, k], read through the row map
+  const int32_t* src_bins = nullptr;
+  int top_k = 1, src_rows = 0;
+};
 template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
             int layout, hipStream_t s, const void* a2 = nullptr, const void* b2 = nullptr, int epi = dma::kEpiNone,
-            void* extra = nullptr, void* out2 = nullptr) {
+            void* extra = nullptr, void* out2 = nullptr, GatherRows gather = GatherRows()) {
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
   const uint16_t* ap2 = (const uint16_t*)a2;
@@ -623,13 +629,30 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
   if (tiles > 0x7fffffff) return MBX_ERANGE;
   const unsigned grid = (unsigned)persistent_grid(tiles);
-#define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI)                                                              \
+#define MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, GATHER)                                                    \
   do {                                                                                                \
-    auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL, EPI>;                                     \
+    auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL, EPI, GATHER>;                             \
     int rc = allow_lds(kern, lds);                                                                    \
     if (rc) return rc;                                                                                \
-    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2);  \
+    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2,  \
+                                       gather.slots, gather.src_bins, gather.top_k, gather.src_rows);  \
   } while (0)
+#define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI) MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, false)
+  if (gather.slots) {
+    if (layout != MBX_NT || a2 || !gather.src_bins || gather.top_k <= 0) return MBX_EINVAL;
+    if constexpr (T::MF == 16) {
+      switch (epi) {
+        case dma::kEpiNone: MBX_LAUNCH_ROWS_G(false, false, dma::kEpiNone, true); break;
+        case dma::kEpiAct: if (!extra) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiAct, true); break;
+        case dma::kEpiGluSilu: if (!extra || !b2 || !out2) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiGluSilu, true); break;
+        case dma::kEpiGluGelu: if (!extra || !b2 || !out2) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiGluGelu, true); break;
+        default: return MBX_EINVAL;
+      }
+      return launch_status();
+    } else {
+      return MBX_EUNSUPPORTED;
+    }
+  }
   if (dma::epi_is_glu(epi)) {
     // b2 is the second matrix of the [w1 | v1] tiles (not a second operand pair); 16 x 16 x 32 tiles only
     if (layout != MBX_NT || !extra || !b2 || !out2 || a2) return MBX_EINVAL;
@@ -661,6 +684,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (dual) MBX_LAUNCH_ROWS(true, true, dma::kEpiNone); else MBX_LAUNCH_ROWS(true, false, dma::kEpiNone);
   }
 #undef MBX_LAUNCH_ROWS
+#undef MBX_LAUNCH_ROWS_G
   return launch_status();
 }
 
@@ -795,15 +819,18 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
 // kernels take; anything else is MBX_EUNSUPPORTED and the caller runs the product and the element-wise pass.
 // (kEpiDglu*: pre2 = x2, out2 = the second output; 16 x 16 x 32 main loop only.)
 // (kEpiGlu*: b2 = the second matrix, extra = the gated activation, out2 = the second product.)
+// gather.slots non-null: `a` is read through the row map (no epilogue, kEpiAct and kEpiGlu* only; `extra` may then be
+// null for no epilogue).
 static int gmm_nt_epilogue(const void* a, const void* b, void* c, void* extra, int dtype, const int32_t* bins, int num_groups,
                            int64_t rows, int k, int n, int act, int epi, mbx_stream_t stream, const void* pre2 = nullptr,
-                           void* out2 = nullptr, const void* b2 = nullptr) {
+                           void* out2 = nullptr, const void* b2 = nullptr, GatherRows gather = GatherRows()) {
   if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
   const bool dglu = dma::epi_is_dglu(epi), glu = dma::epi_is_glu(epi);
-  if (!dglu && !glu && act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
+  const bool plain = epi == dma::kEpiNone;   // gathered rows only
+  if (!dglu && !glu && !plain && act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
   if (num_groups == 0 || rows == 0 || n == 0) return 0;
-  if (!bins || !c || !extra || (k > 0 && (!a || !b)) || (dglu && (!pre2 || !out2)) || (glu && (!out2 || (k > 0 && !b2)))) return MBX_EINVAL;
+  if (!bins || !c || (!extra && !plain) || (k > 0 && (!a || !b)) || (dglu && (!pre2 || !out2)) || (glu && (!out2 || (k > 0 && !b2)))) return MBX_EINVAL;
   if (rows > 0x7fffffff) return MBX_ERANGE;
   bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(extra) && k > 0 &&
             k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n) && (!dglu || (aligned16(pre2) && aligned16(out2)));
@@ -813,13 +840,13 @@ static int gmm_nt_epilogue(const void* a, const void* b, void* c, void* extra, i
   hipStream_t s = as_stream(stream);
   if (use_mfma16()) {
     if (half_height_only(rows, num_groups, n)) {
-      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
-      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
+      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
     }
-    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
-    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2);
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
+    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
   }
-  if (dglu || glu) return MBX_EUNSUPPORTED;
+  if (dglu || glu || gather.slots) return MBX_EUNSUPPORTED;
   if (half_height_only(rows, num_groups, n)) {
     if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
     return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
@@ -843,6 +870,25 @@ int mbx_gmm_glu(const void* a, const void* b1, const void* b2, void* x1, void* x
   if (act != MBX_ACT_SILU && act != MBX_ACT_GELU_TANH) return MBX_EINVAL;
   return gmm_nt_epilogue(a, b1, x1, h, dtype, bins, num_groups, rows, k, n, act,
                          act == MBX_ACT_SILU ? dma::kEpiGluSilu : dma::kEpiGluGelu, stream, nullptr, x2, b2);
+}
+
+int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int top_k, const int32_t* x_bins, const void* b1,
+                   const void* b2, void* c, void* c2, void* h, int dtype, const int32_t* bins, int num_groups, int64_t rows,
+                   int k, int n, int act, mbx_stream_t stream) {
+  if (x_rows < 0 || top_k <= 0 || k < 0) return MBX_EINVAL;
+  if (b2 ? (act != MBX_ACT_SILU && act != MBX_ACT_GELU_TANH) || !c2 || !h : c2 != nullptr) return MBX_EINVAL;
+  if (h && !b2 && act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
+  if (num_groups > 0 && rows > 0 && n > 0 && (!indices || (k > 0 && !x && x_rows > 0))) return MBX_EINVAL;
+  // the row map is indexed with 32 bits and the rows of x are addressed with 31 (bit 31 marks a row of zeros)
+  if (x_rows * top_k > 0x7fffffff || x_rows * (int64_t)k * 2 >= ((int64_t)1 << 31)) return MBX_EUNSUPPORTED;
+  if (x_rows == 0 && rows > 0) x = b1;   // no row is read; the buffer descriptor still wants an address
+  GatherRows gather;
+  gather.slots = indices;
+  gather.src_bins = x_bins ? x_bins : bins;
+  gather.top_k = top_k;
+  gather.src_rows = (int)x_rows;
+  const int epi = b2 ? (act == MBX_ACT_SILU ? dma::kEpiGluSilu : dma::kEpiGluGelu) : h ? dma::kEpiAct : dma::kEpiNone;
+  return gmm_nt_epilogue(x, b1, c, h, dtype, bins, num_groups, rows, k, n, act, epi, stream, nullptr, c2, b2, gather);
 }
 
 int mbx_gmm_dglu(const void* a, const void* b, const void* x1, const void* x2, void* d1, void* d2, int dtype,

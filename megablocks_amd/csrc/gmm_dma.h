@@ -216,6 +216,10 @@ struct Args {
   // from the second pair.  Used only by the DUAL instantiations.
   __amdgpu_buffer_rsrc_t rsrc_a2, rsrc_b2;
   int nk1;
+  // GATHER instantiations: row r of the A tile is row slots[j0 + r] / top_k of the matrix behind rsrc_a (a_r0 = 0),
+  // zeros when j0 + r >= j1, the slot is negative or the row is not below src_rows.
+  const int32_t* gather_slots;
+  int gather_j0, gather_j1, gather_top_k, gather_src_rows;
 };
 
 // acc = (clear ? 0 : acc) + A_tile * B_tile over all K tiles.  On return no load is in flight and no LDS
@@ -460,10 +464,14 @@ __device__ __forceinline__ void mfma16_settle() { asm volatile("s_nop 15\n\ts_no
 // GLU: rows BN / 2 .. BN - 1 of the B tile (the second half of every wave's loads of a K tile) come through g.rsrc_b2,
 // whose base the caller has set BN / 2 rows before the second matrix: the tile is then [w1 rows | v1 rows] of the same
 // BN / 2 output columns, side by side (KC operands only, not with DUAL).
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false>
+// GATHER: the rows of the A tile (KC operand) are gathered rows of a matrix: each of a lane's LA loads of a K tile gets
+// a byte offset of its own (its row's, worked out once per tile from the row map), where the plain tile adds a
+// multiple of the row pitch to one lane offset.  The loads are the same 16-byte pieces of 128-byte row segments.
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false>
 __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
   static_assert(T::MF == 16 && T::KS == 2, "two k-steps of 32 per K tile");
   static_assert(!GLU || (!B_MC && !DUAL && T::LB % 2 == 0), "two matrices side by side in the B tile");
+  static_assert(!GATHER || (!A_MC && !DUAL && T::BK == 64), "gathered rows: a KC operand, one operand pair");
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -481,30 +489,48 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
   const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
   const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
   constexpr uint32_t A_ROWS = (uint32_t)(1024 / ((A_MC ? T::BM : BK) * 2)), B_ROWS = (uint32_t)(1024 / ((B_MC ? T::BN : BK) * 2));
-  const uint32_t a_jstep = A_ROWS * g.a_ld_bytes, b_jstep = B_ROWS * g.b_ld_bytes;
+  const uint32_t a_jstep = GATHER ? 0u : A_ROWS * g.a_ld_bytes, b_jstep = B_ROWS * g.b_ld_bytes;
   auto scalar_off = [&](bool is_b, int kt, int q) -> uint32_t {
     const uint32_t j = (uint32_t)(wave + q * T::WAVES);
     const uint32_t v = is_b ? (uint32_t)kt * b_step + j * b_jstep : (uint32_t)kt * a_step + j * a_jstep;
     return v | (kt < g.nk ? 0u : 0x80000000u);
   };
+  // byte offset of the q-th A load's row and 16-byte piece (bit 31: no such row, the load brings zeros)
+  uint32_t a_row[GATHER ? LA : 1];
+  if constexpr (GATHER) {
+    const uint32_t piece = load_lane_offset<false, BK, T::BM, 16>(wave, 0, 0u, false);   // pitch 0: the piece inside the row
+    const int lane_row = lane_id() >> 3;
+    int slot[LA];
+#pragma unroll
+    for (int q = 0; q < LA; ++q) {
+      const int j = g.gather_j0 + (int)A_ROWS * (wave + q * T::WAVES) + lane_row;
+      slot[q] = j < g.gather_j1 ? g.gather_slots[j] : -1;
+    }
+#pragma unroll
+    for (int q = 0; q < LA; ++q) {
+      const uint32_t row = (uint32_t)slot[q] / (uint32_t)g.gather_top_k;
+      a_row[q] = slot[q] >= 0 && row < (uint32_t)g.gather_src_rows ? row * g.a_ld_bytes + piece : 0x80000000u;
+    }
+  }
   __amdgpu_buffer_rsrc_t ra = g.rsrc_a, rb = g.rsrc_b;
   const __amdgpu_buffer_rsrc_t rb_upper = GLU ? g.rsrc_b2 : g.rsrc_b;
   auto lds_off = [&](bool is_b, int stage, int q) -> uint32_t {
     return (is_b ? B_RING + (uint32_t)stage * T::B_BYTES : (uint32_t)stage * T::A_BYTES) + (uint32_t)(wave + q * T::WAVES) * 1024u;
   };
   // upper: the load is one of the second half of the wave's B loads of a K tile (GLU only)
-  auto issue = [&](bool is_b, uint32_t sc, uint32_t dst, bool odd, bool upper = false) {
+  // q: the load's index among the wave's loads of the tile (GATHER, A loads: which row offset)
+  auto issue = [&](bool is_b, uint32_t sc, uint32_t dst, bool odd, bool upper, int q) {
     if (is_b) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(GLU && upper ? rb_upper : rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? b_lane1 : b_lane) + sc), 0, 0, 0);
     } else {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? a_lane1 : a_lane) + sc), 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((GATHER ? a_row[GATHER ? q : 0] : odd ? a_lane1 : a_lane) + sc), 0, 0, 0);
     }
   };
   auto issue_group = [&](bool is_b, int kt, int stage, int q0, int count) {   // prologue
     uint32_t sc = scalar_off(is_b, kt, q0), dst = lds_off(is_b, stage, q0);
 #pragma unroll
     for (int i = 0; i < count; ++i) {
-      issue(is_b, sc, dst, ((q0 + i) & 1) != 0, is_b && q0 + i >= LB / 2);
+      issue(is_b, sc, dst, ((q0 + i) & 1) != 0, is_b && q0 + i >= LB / 2, q0 + i);
       sc += T::WAVES * (is_b ? b_jstep : a_jstep);
       dst += T::WAVES * 1024u;
     }
@@ -594,7 +620,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
       mfma16_acc<DT>(acc[i_][j_], fb[CUR_BUF][j_], fa[CUR_BUF][i_]);                                             \
       MBX_READ_SLOT16(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                            \
       if constexpr (m_ >= (LOAD0) && (m_ - (LOAD0)) % (EVERY) == 0 && (m_ - (LOAD0)) / (EVERY) < (NL))           \
-        issue(IS_B, SC, DST, (((m_ - (LOAD0)) / (EVERY)) & 1) != 0, (IS_B) && (m_ - (LOAD0)) / (EVERY) >= (NL) / 2); \
+        issue(IS_B, SC, DST, (((m_ - (LOAD0)) / (EVERY)) & 1) != 0, (IS_B) && (m_ - (LOAD0)) / (EVERY) >= (NL) / 2, (m_ - (LOAD0)) / (EVERY)); \
       if constexpr (m_ > (LOAD0) && (m_ - (LOAD0) - 1) % (EVERY) == 0 && (m_ - (LOAD0) - 1) / (EVERY) < (NL)) {  \
         SC += T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                                           \
         DST += T::WAVES * 1024u;                                                                                 \
@@ -713,11 +739,11 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
 #undef MBX_STEP16
 }
 
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false>
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false>
 __device__ __forceinline__ void block_multiply(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds) {
-  static_assert(!GLU || T::MF == 16, "two matrices side by side: 16 x 16 x 32 loop only");
+  static_assert((!GLU && !GATHER) || T::MF == 16, "two matrices side by side, gathered rows: 16 x 16 x 32 loop only");
   if constexpr (T::MF == 32) block_multiply32<DT, A_MC, B_MC, T, DUAL>(g, acc, clear, lds);
-  else block_multiply16<DT, A_MC, B_MC, T, DUAL, GLU>(g, acc, clear, lds);
+  else block_multiply16<DT, A_MC, B_MC, T, DUAL, GLU, GATHER>(g, acc, clear, lds);
 }
 
 // ---- activation in the epilogue (tanh-GELU: megablocks/layers/arguments.py:19, megablocks/layers/gelu.py:9-13) ----
@@ -1117,12 +1143,12 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
 }
 
 // c = A_tile * B_tile over all K tiles (the whole product of one output tile)
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, int EPI = kEpiNone>
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, int EPI = kEpiNone, bool GATHER = false>
 __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
                                            int n_base, int n_lim, char* lds, uint16_t* __restrict__ extra = nullptr,
                                            const uint16_t* __restrict__ pre2 = nullptr, uint16_t* __restrict__ out2 = nullptr) {
   typename T::Acc acc[T::TM][T::TN];
-  block_multiply<DT, A_MC, B_MC, T, DUAL, epi_is_glu(EPI)>(g, acc, true, lds);
+  block_multiply<DT, A_MC, B_MC, T, DUAL, epi_is_glu(EPI), GATHER>(g, acc, true, lds);
   block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra, pre2, out2);
 }
 
@@ -1290,12 +1316,16 @@ struct RowTiles {
 // (SB + 1) K tiles), as one reduction over 2 k.
 // EPI: see block_store; `extra` is its second output / input, [rows, n] like c; kEpiDglu*: `a2` is x2 and `out2` the
 // second output, both [rows, n].
-template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false, int EPI = kEpiNone>
+// GATHER: `a` is [src_rows, k] and row r of expert e's rows is a[slots[src_start(e) + r] / top_k] while
+// src_start(e) + r < src_bins[e], zeros after that (src_start(e) = src_bins[e - 1], 0 for the first expert): the
+// product of the rows that megablocks/ops/gather.py:20-38 / padded_gather.py:20-55 would have copied out first.
+template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false, int EPI = kEpiNone, bool GATHER = false>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra,
-                uint16_t* __restrict__ out2) {
+                uint16_t* __restrict__ out2, const int32_t* __restrict__ slots, const int32_t* __restrict__ src_bins,
+                int top_k, int src_rows) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
   static_assert(!(DUAL && (epi_is_dglu(EPI) || epi_is_glu(EPI))), "a2 / b2 are the second operand pair, the epilogue's x2 or the second matrix");
@@ -1316,6 +1346,11 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   g.nk1 = k / T::BK;
   g.nk = DUAL ? 2 * g.nk1 : g.nk1;
   g.a_r0 = 0;   // the buffers of a and c start at the tile's first row: byte offsets stay small whatever the row count
+  if constexpr (GATHER) {
+    g.gather_slots = slots;
+    g.gather_top_k = top_k;
+    g.gather_src_rows = src_rows;
+  }
   // Work items of this workgroup: one tile per round, then (if the tail is split) one half tile.
   const int items = big_rounds + ((kSplit && split) ? 1 : 0);
   for (int r = 0; r < items; ++r) {
@@ -1338,7 +1373,16 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     const int row0 = start + tm * T::BM + half * TS::BM;
     if (row0 >= end) break;               // the second half of a tile whose rows end in the first (a last item)
     const uint32_t a_bytes = clip_bytes((rows - row0) * k * 2);   // rows past the tile's are fetched, never stored
-    g.rsrc_a = make_rsrc(a + (int64_t)row0 * k, a_bytes);
+    if constexpr (GATHER) {
+      // the whole source matrix (below 2 GiB: bit 31 of an offset marks a load that must bring zeros)
+      g.rsrc_a = make_rsrc(a, clip_bytes((int64_t)src_rows * k * 2));
+      const int64_t slots_end = (int64_t)src_rows * top_k;
+      const int src_start = e > 0 ? src_bins[e - 1] : 0, src_end = src_bins[e];
+      g.gather_j0 = (src_start < 0 ? 0 : src_start) + (row0 - start);
+      g.gather_j1 = (int)(src_end < slots_end ? src_end : slots_end);
+    } else {
+      g.rsrc_a = make_rsrc(a + (int64_t)row0 * k, a_bytes);
+    }
     g.rsrc_a2 = DUAL ? make_rsrc(a2 + (int64_t)row0 * k, a_bytes) : g.rsrc_a;
     g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
     g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
@@ -1352,9 +1396,9 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
     use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
     if (use_ts) {
-      block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
+      block_gemm<DT, false, B_MC, TS, DUAL, EPI, GATHER>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
     } else {
-      block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
+      block_gemm<DT, false, B_MC, T, DUAL, EPI, GATHER>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
     }
     tile_done();
   }

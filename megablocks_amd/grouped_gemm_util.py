@@ -271,6 +271,80 @@ def gmm_glu(a, b1, b2, batch_sizes, act, fuse=None):
     return x1, x2, h
 
 
+# Whether the dMoE layer hands the experts the ungathered tokens (`gmm_gather`) instead of calling ops.gather /
+# ops.padded_gather first: 'auto' = where no gradient is recorded (the forward then never writes the gathered copy;
+# with gradients the weight gradients need that copy anyway, so fusing only moves the gather into the backward),
+# '1' = always (the copy then exists only during the backward), '0' = never.
+FUSED_GATHER = os.environ.get('MBX_FUSED_GATHER', 'auto')
+
+
+class GatheredRows:
+    """The matrix ops.gather / ops.padded_gather (dmoe.py:219 / :273) would make of `x`, as a description: the rows of
+    x in the order of the sorted assignments `indices`, each expert's rows padded with zero rows up to its padded bin
+    when `padded_bins` is given.  `rows` is the row count of that matrix."""
+
+    def __init__(self, x, indices, bin_ids, bins, padded_bins, top_k, rows):
+        self.x, self.indices, self.bin_ids, self.bins, self.padded_bins = x, indices, bin_ids, bins, padded_bins
+        self.top_k, self.rows = int(top_k), int(rows)
+
+    def materialize(self):
+        from megablocks_amd.backend import kernels
+        if self.padded_bins is None:
+            return kernels.gather(self.x, self.indices, self.bin_ids, None, self.bins, self.top_k)
+        return kernels.padded_gather(self.x, self.indices, self.bin_ids, None, self.bins, self.padded_bins, self.top_k)
+
+    def scatter_grad(self, grad):
+        """The gradient of x from the gradient of the gathered matrix (gather.py:28-35, padded_gather.py:36-52)."""
+        from megablocks_amd.backend import kernels
+        if self.padded_bins is None:
+            return kernels.scatter(grad, self.indices, self.bin_ids, None, self.bins, self.top_k)
+        return kernels.padded_scatter(grad, self.indices, self.bin_ids, None, self.bins, self.padded_bins, self.top_k)
+
+
+def gmm_gather(src: GatheredRows, b1, batch_sizes, b2=None, act=None):
+    """The first product(s) of the experts on the rows `src` describes, read from the ungathered tokens (one launch,
+    `mbx_gmm_gather`): bit-identical to `src.materialize()` followed by
+        b2 None, act None:  (gmm(a, b1, trans_b=True),)
+        b2 None, act ACT_GELU_TANH:  gmm_act(a, b1)  -> (c, gelu_tanh(c))
+        b2 given:  gmm_glu(a, b1, b2, act)  -> (x1, x2, h)
+    Returns None where the library has no kernel for the operands: the caller then gathers and multiplies."""
+    x = src.x
+    if not (x.is_cuda and x.ndim == 2 and x.dtype in (torch.bfloat16, torch.float16) and b1.ndim == 3 and
+            b1.dtype == x.dtype and b1.shape[2] == x.shape[1] and src.indices.dtype == torch.int32 and
+            src.bins.dtype == torch.int32 and ACTIVATION_EPILOGUES):
+        return None
+    if b2 is not None and (b2.shape != b1.shape or b2.dtype != b1.dtype or act is None):
+        return None
+    if src.padded_bins is not None and src.padded_bins.dtype != torch.int32:
+        return None
+    if src.indices.ndim != 1 or src.indices.shape[0] != x.shape[0] * src.top_k:
+        raise ValueError('gmm_gather: one assignment per token and top_k choice')
+    _lib.require_cuda(b1, b2, src.indices, src.bins, src.padded_bins)
+    x, b1 = x.contiguous(), b1.contiguous()
+    b2 = None if b2 is None else b2.contiguous()
+    rows, k, n = src.rows, x.shape[1], b1.shape[1]
+    bins = _device_bins(batch_sizes, x.device, rows)
+    groups = bins.shape[0]
+    if b1.shape[0] != groups or src.bins.numel() != groups:
+        return None
+    x_bins = None if src.padded_bins is None else src.bins.contiguous()
+    c = torch.empty((rows, n), dtype=x.dtype, device=x.device)
+    c2 = None if b2 is None else torch.empty_like(c)
+    h = None if act is None else torch.empty_like(c)
+    name = 'gmm_nt_glu' if b2 is not None else 'gmm_nt_act' if act is not None else 'gmm_nt'
+    with _lib.device_of(x), _lib.record(name, rows=rows, k=k, n=n * (2 if b2 is not None else 1), elem=x.element_size(),
+                                        groups=groups) as rec:
+        rc = lib.mbx_gmm_gather(_lib.ptr(x), x.shape[0], _lib.ptr(src.indices.contiguous()), src.top_k, _lib.ptr(x_bins),
+                                _lib.ptr(b1), _lib.ptr(b2), _lib.ptr(c), _lib.ptr(c2), _lib.ptr(h), _lib.dtype_of(x),
+                                _lib.ptr(bins), groups, rows, k, n, 0 if act is None else act, _lib.stream())
+        if rc == _lib.EUNSUPPORTED:
+            rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        return None
+    _lib.check(rc, 'gmm_gather')
+    return (c,) if act is None else (c, h) if b2 is None else (c, c2, h)
+
+
 def gmm_dglu(a, b, x1, x2, batch_sizes, act, fuse=None):
     """The gradients (d x1, d x2) of `activation(x1) * x2` where the incoming gradient is g = a[r_e] @ b[e].T: the
     `gmm(ddsd_out, w2, trans_b=True)` of the GLU experts' backward and the backward of their gated activation

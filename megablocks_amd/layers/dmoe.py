@@ -88,6 +88,30 @@ class ParallelDroplessMLP(moe.ParallelMLP):
         bins = promote_scalar(ops.inclusive_cumsum(tokens_per_expert, 0))
         return indices, bin_ids, bins, padded_bins, tokens_per_expert
 
+    def _fuse_gather(self, x):
+        """Whether the experts get the ungathered tokens (gg.FUSED_GATHER): the built-in experts on the GPU only."""
+        if gg.FUSED_GATHER == '0' or not x.is_cuda or not hasattr(self.mlp, 'forward_tokens'):
+            return False
+        if gg.FUSED_GATHER == 'auto':
+            return not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.mlp.parameters())))
+        return True
+
+    def _sparse_experts(self, x, indices, bin_ids, bins, padded_bins, top_k):
+        """dmoe.py:219-226: padded gather, topology, experts.  Where the experts take the ungathered tokens the gather
+        is part of their first product."""
+        if self._fuse_gather(x):
+            padded_rows = int(padded_bins[-1].item()) if padded_bins.numel() else 0   # as ops.padded_gather reads it
+            with torch.no_grad():
+                topo = self.topology(x.new_empty((padded_rows, 0)), padded_bins)
+            src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, top_k, padded_rows)
+            out = self.mlp.forward_tokens(src, topo.padded_tokens_per_expert)
+            if out is not None:
+                return out
+        x = ops.padded_gather(x, indices, bin_ids, bins, padded_bins, top_k)
+        with torch.no_grad():
+            topo = self.topology(x, padded_bins)
+        return self.mlp(x, topo)
+
     def sparse_forward_once(self, x, expert_weights, top_experts):
         """dmoe.py:156-193."""
         expert_weights = expert_weights.flatten()
@@ -95,10 +119,7 @@ class ParallelDroplessMLP(moe.ParallelMLP):
         with torch.no_grad():
             indices, bin_ids, bins, padded_bins, tokens_per_expert = self.indices_and_padded_bins(top_experts)
         x = x.view(-1, x.shape[-1])
-        x = ops.padded_gather(x, indices, bin_ids, bins, padded_bins, self.top_k)
-        with torch.no_grad():
-            topo = self.topology(x, padded_bins)
-        x = self.mlp(x, topo)
+        x = self._sparse_experts(x, indices, bin_ids, bins, padded_bins, self.top_k)
         x = ops.padded_scatter(x, indices, bin_ids, expert_weights, bins, padded_bins, self.top_k)
         return x, tokens_per_expert
 
@@ -108,10 +129,7 @@ class ParallelDroplessMLP(moe.ParallelMLP):
         padded_tokens_per_expert = ops.round_up(tokens_per_expert, self.blocking)
         padded_bins = promote_scalar(ops.inclusive_cumsum(padded_tokens_per_expert, 0))
         x = x.view(-1, x.shape[-1])
-        x = ops.padded_gather(x, indices, bin_ids, bins, padded_bins, top_k)
-        with torch.no_grad():
-            topo = self.topology(x, padded_bins)
-        x = self.mlp(x, topo)
+        x = self._sparse_experts(x, indices, bin_ids, bins, padded_bins, top_k)
         return ops.padded_scatter(x, indices, bin_ids, expert_weights, bins, padded_bins, top_k)
 
     def grouped_forward_once(self, x, expert_weights, top_experts):
@@ -128,9 +146,14 @@ class ParallelDroplessMLP(moe.ParallelMLP):
                                     expert_capactiy, top_k):
         """dmoe.py:260-280."""
         x = x.view(-1, x.shape[-1])
-        x = ops.gather(x, indices, bin_ids, bins, top_k)
-        x = self.mlp(x, tokens_per_expert)
-        return ops.scatter(x, indices, bin_ids, expert_weights, bins, top_k)
+        out = None
+        if self._fuse_gather(x):
+            src = gg.GatheredRows(x, indices, bin_ids, bins, None, top_k, indices.shape[0])
+            out = self.mlp.forward_tokens(src, tokens_per_expert)
+        if out is None:
+            x = ops.gather(x, indices, bin_ids, bins, top_k)
+            out = self.mlp(x, tokens_per_expert)
+        return ops.scatter(out, indices, bin_ids, expert_weights, bins, top_k)
 
     def forward_once(self, x, expert_weights, top_experts):
         if self.args.mlp_impl == 'sparse':

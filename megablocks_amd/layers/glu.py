@@ -126,19 +126,61 @@ class GroupedGLUExperts(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type='cuda')
     def backward(ctx, ddsd_out):
         x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out = ctx.saved_tensors
-        ddsd_out = ddsd_out.contiguous()
-        dx = dw1 = dv1 = dw2 = None
-        if ctx.needs_input_grad[3]:
-            dw2 = gg.backend.gmm(activation_fn_out, ddsd_out, batch_sizes, trans_a=True)
-        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            dsdd_out, dv1_out = gg.gmm_dglu(ddsd_out, w2, sdd_out, v1_out, batch_sizes, ctx.act)
-            if ctx.needs_input_grad[1]:
-                dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
-            if ctx.needs_input_grad[2]:
-                dv1 = gg.backend.gmm(dv1_out, x, batch_sizes, trans_a=True)
-            if ctx.needs_input_grad[0]:
-                dx = gg.gmm_dual(dsdd_out, w1, dv1_out, v1, batch_sizes)
-        return dx, dw1, dv1, dw2, None, None
+        return (*_glu_experts_backward(ctx.needs_input_grad, x, w1, v1, w2, batch_sizes, sdd_out, v1_out,
+                                       activation_fn_out, ddsd_out, ctx.act), None, None)
+
+
+def _glu_experts_backward(needs, x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, ddsd_out, act):
+    """(dx, dw1, dv1, dw2) of GroupedGLUExperts from what its forward saved; needs = which of (x, w1, v1, w2) want a
+    gradient."""
+    ddsd_out = ddsd_out.contiguous()
+    dx = dw1 = dv1 = dw2 = None
+    if needs[3]:
+        dw2 = gg.backend.gmm(activation_fn_out, ddsd_out, batch_sizes, trans_a=True)
+    if needs[0] or needs[1] or needs[2]:
+        dsdd_out, dv1_out = gg.gmm_dglu(ddsd_out, w2, sdd_out, v1_out, batch_sizes, act)
+        if needs[1]:
+            dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
+        if needs[2]:
+            dv1 = gg.backend.gmm(dv1_out, x, batch_sizes, trans_a=True)
+        if needs[0]:
+            dx = gg.gmm_dual(dsdd_out, w1, dv1_out, v1, batch_sizes)
+    return dx, dw1, dv1, dw2
+
+
+class GatheredGLUExperts(torch.autograd.Function):
+    """GroupedGLUExperts on the rows ops.gather / ops.padded_gather would copy out of the tokens `x` (dmoe.py:219 / :273
+    followed by glu.py:201-205), without that copy in the forward: the launch that computes both first products and
+    the gated activation reads its rows from `x` through the sorted assignments (`gg.gmm_gather`).  The weight
+    gradients of w1 and v1 need the gathered rows as an operand, so the backward makes the copy then, and returns the
+    gradient of the tokens (the backward of the gather).  Same values as the two separate nodes."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
+    def forward(ctx, x, w1, v1, w2, batch_sizes, act, indices, bin_ids, bins, padded_bins, top_k, rows):
+        x = x.contiguous()
+        src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, top_k, rows)
+        out = gg.gmm_gather(src, w1, batch_sizes, b2=v1, act=act)
+        if out is None:
+            out = gg.gmm_glu(src.materialize(), w1, v1, batch_sizes, act)
+        sdd_out, v1_out, activation_fn_out = out
+        ctx.act, ctx.top_k, ctx.rows = act, top_k, rows
+        ctx.save_for_backward(x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, indices, bin_ids, bins,
+                              padded_bins)
+        return gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
+    def backward(ctx, ddsd_out):
+        (x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, indices, bin_ids, bins,
+         padded_bins) = ctx.saved_tensors
+        src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, ctx.top_k, ctx.rows)
+        rows_of_x = src.materialize() if ctx.needs_input_grad[1] or ctx.needs_input_grad[2] else None
+        dx, dw1, dv1, dw2 = _glu_experts_backward(ctx.needs_input_grad, rows_of_x, w1, v1, w2, batch_sizes, sdd_out,
+                                                  v1_out, activation_fn_out, ddsd_out, ctx.act)
+        if dx is not None:
+            dx = src.scatter_grad(dx)
+        return dx, dw1, dv1, dw2, None, None, None, None, None, None, None, None
 
 
 def _one_node(x, w1, v1, w2, act):
@@ -243,6 +285,19 @@ class SparseGLU(SparseMLP):
 
     def forward(self, x, topo: Topology):
         return self._compute(x, topo.padded_tokens_per_expert, allow_memory_optimized=False)   # glu.py:47-50
+
+    def forward_tokens(self, src, batch_sizes):
+        """forward on the rows of the tokens that `src` (a `gg.GatheredRows`) describes, which are then never copied
+        out in the forward; None where that is not built (the caller gathers and calls forward)."""
+        if self.args.memory_optimized_mlp:
+            return None
+        act = _activation_code(self.args.activation_fn)
+        w1, v1, w2 = self._expert_views(self.w1, self.v1, self.w2)
+        x, w1, v1, w2 = gg.autocast_operands(src.x, w1, v1, w2)
+        if not _one_node(x, w1, v1, w2, act):
+            return None
+        return GatheredGLUExperts.apply(x, w1, v1, w2, batch_sizes, act, src.indices, src.bin_ids, src.bins,
+                                        src.padded_bins, src.top_k, src.rows)
 
 
 class GroupedGLU(SparseGLU):

@@ -161,17 +161,58 @@ class GroupedGeluMLP(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type='cuda')
     def backward(ctx: Any, ddsd_out: torch.Tensor):
         w1, w2, batch_sizes, x, sdd_out, activation_fn_out = ctx.saved_tensors
-        ddsd_out = ddsd_out.contiguous()
-        dx = dw1 = dw2 = None
-        if ctx.needs_input_grad[2]:
-            dw2 = gg.backend.gmm(activation_fn_out, ddsd_out, batch_sizes, trans_a=True)
-        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-            dsdd_out = gg.gmm_dact(ddsd_out, w2, sdd_out, batch_sizes)
-            if ctx.needs_input_grad[1]:
-                dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
-            if ctx.needs_input_grad[0]:
-                dx = gg.backend.gmm(dsdd_out, w1, batch_sizes)
-        return dx, dw1, dw2, None
+        return (*_gelu_mlp_backward(ctx.needs_input_grad, x, w1, w2, batch_sizes, sdd_out, activation_fn_out, ddsd_out),
+                None)
+
+
+def _gelu_mlp_backward(needs, x, w1, w2, batch_sizes, sdd_out, activation_fn_out, ddsd_out):
+    """(dx, dw1, dw2) of GroupedGeluMLP from what its forward saved; needs = which of (x, w1, w2) want a gradient."""
+    ddsd_out = ddsd_out.contiguous()
+    dx = dw1 = dw2 = None
+    if needs[2]:
+        dw2 = gg.backend.gmm(activation_fn_out, ddsd_out, batch_sizes, trans_a=True)
+    if needs[0] or needs[1]:
+        dsdd_out = gg.gmm_dact(ddsd_out, w2, sdd_out, batch_sizes)
+        if needs[1]:
+            dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
+        if needs[0]:
+            dx = gg.backend.gmm(dsdd_out, w1, batch_sizes)
+    return dx, dw1, dw2
+
+
+class GatheredGeluMLP(torch.autograd.Function):
+    """GroupedGeluMLP on the rows ops.gather / ops.padded_gather would copy out of the tokens `x` (dmoe.py:219 / :273
+    followed by mlp.py:499-523), without that copy in the forward: the first product reads its rows from `x` through
+    the sorted assignments (`gg.gmm_gather`).  The weight gradient of w1 needs the gathered rows as an operand, so the
+    backward makes the copy then, and returns the gradient of the tokens (the sum over each token's rows, which is
+    the backward of the gather).  Same values as the two separate nodes."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type='cuda')
+    def forward(ctx, x, w1, w2, batch_sizes, indices, bin_ids, bins, padded_bins, top_k, rows):
+        if ctx._fwd_used_autocast:
+            x, w1, w2 = x.to(ctx._dtype), w1.to(ctx._dtype), w2.to(ctx._dtype)
+        x, w1, w2 = x.contiguous(), w1.contiguous(), w2.contiguous()
+        src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, top_k, rows)
+        out = gg.gmm_gather(src, w1, batch_sizes, act=gg.ACT_GELU_TANH)
+        if out is None:
+            out = gg.gmm_act(src.materialize(), w1, batch_sizes)
+        sdd_out, activation_fn_out = out
+        ctx.top_k, ctx.rows = top_k, rows
+        ctx.save_for_backward(w1, w2, batch_sizes, x, sdd_out, activation_fn_out, indices, bin_ids, bins, padded_bins)
+        return gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type='cuda')
+    def backward(ctx: Any, ddsd_out: torch.Tensor):
+        w1, w2, batch_sizes, x, sdd_out, activation_fn_out, indices, bin_ids, bins, padded_bins = ctx.saved_tensors
+        src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, ctx.top_k, ctx.rows)
+        rows_of_x = src.materialize() if ctx.needs_input_grad[1] else None
+        dx, dw1, dw2 = _gelu_mlp_backward(ctx.needs_input_grad, rows_of_x, w1, w2, batch_sizes, sdd_out,
+                                          activation_fn_out, ddsd_out)
+        if dx is not None:
+            dx = src.scatter_grad(dx)
+        return dx, dw1, dw2, None, None, None, None, None, None, None
 
 
 grouped_gelu_mlp = GroupedGeluMLP.apply
@@ -283,6 +324,15 @@ class SparseMLP(torch.nn.Module):
 
     def forward(self, x, topo: Topology):
         return self._compute(x, topo.padded_tokens_per_expert)
+
+    def forward_tokens(self, src, batch_sizes):
+        """forward on the rows of the tokens that `src` (a `gg.GatheredRows`) describes, which are then never copied
+        out in the forward; None where that is not built (the caller gathers and calls forward)."""
+        if self.args.memory_optimized_mlp or self.args.activation_fn is not DEFAULT_ACTIVATION_FN or not src.x.is_cuda:
+            return None
+        w1, w2 = self._expert_views(self.w1, self.w2)
+        return GatheredGeluMLP.apply(src.x, w1, w2, batch_sizes, src.indices, src.bin_ids, src.bins, src.padded_bins,
+                                     src.top_k, src.rows)
 
 
 class GroupedMLP(SparseMLP):

@@ -1,6 +1,8 @@
 """GPU parity tests of the grouped GEMM: against the CPU oracle at small sizes and against an
 fp32 torch formulation on the GPU at the benchmark shapes.  Tolerance: relative Frobenius
 error <= 1e-2 (bf16/f16 inputs, fp32 accumulation)."""
+import math
+
 import pytest
 import torch
 
@@ -672,3 +674,79 @@ def test_gmm_with_gated_activation_epilogue(gg, groups, rows, k, n, dtype, act):
     assert bool((guard == 7.0).all())
     with pytest.raises(ValueError):
         gg.gmm_glu(a, w1, v1[:, :n - 8].contiguous(), sizes, act)
+
+
+def _routing(tokens, experts, top_k, seed, blocking=0):
+    """(indices, bin_ids, bins, padded_bins or None, tokens_per_expert) of a random assignment, from the library's ops."""
+    from megablocks_amd import ops
+    g = torch.Generator().manual_seed(seed)
+    top = torch.randint(0, experts, (tokens * top_k,), generator=g, dtype=torch.int32)
+    if experts > 2:
+        top[top == 1] = 0                                   # an expert without tokens
+    top = top.cuda()
+    end_bit = max(int(math.ceil(math.log2(experts))), 1)
+    bin_ids, indices = ops.sort(top, end_bit)
+    tpe = ops.histogram(top, experts)
+    bins = ops.inclusive_cumsum(tpe, 0).view(-1)
+    padded_bins = None
+    if blocking:
+        padded_bins = ops.inclusive_cumsum(ops.round_up(tpe, blocking), 0).view(-1)
+    return indices, bin_ids, bins, padded_bins, tpe
+
+
+GATHERED = [  # tokens, experts, top_k, k, n, blocking
+    (4096, 8, 2, 1024, 512, 0), (3000, 5, 1, 320, 264, 0), (700, 3, 4, 128, 1408, 0), (37, 1, 1, 64, 8, 0),
+    (2048, 16, 4, 256, 384, 128), (1000, 72, 2, 128, 264, 128), (5000, 64, 1, 1024, 1024, 0), (9, 4, 2, 64, 136, 128),
+]
+
+
+@pytest.mark.parametrize('tokens,experts,top_k,k,n,blocking', GATHERED)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_gmm_on_rows_gathered_on_the_fly(gg, tokens, experts, top_k, k, n, blocking, dtype):
+    """gmm_gather: the first product(s) of the experts reading their rows from the ungathered tokens must equal, bit
+    for bit, ops.gather / ops.padded_gather (dmoe.py:219 / :273) followed by gmm, gmm_act and gmm_glu: the same
+    products over the same operand values in the same order, only fetched from other addresses."""
+    torch.manual_seed(tokens + n)
+    indices, bin_ids, bins, padded_bins, tpe = _routing(tokens, experts, top_k, seed=tokens + k, blocking=blocking)
+    x = torch.randn(tokens, k, device='cuda').to(dtype)
+    w1 = (torch.randn(experts, n, k, device='cuda') * (1.5 / k ** 0.5)).to(dtype)
+    v1 = (torch.randn(experts, n, k, device='cuda') * (1.0 / k ** 0.5)).to(dtype)
+    rows = tokens * top_k if padded_bins is None else int(padded_bins[-1])
+    sizes = tpe if padded_bins is None else torch.diff(padded_bins, prepend=padded_bins.new_zeros(1))
+    src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, top_k, rows)
+    a = src.materialize()
+    assert a.shape == (rows, k)
+    guard = torch.full((3, rows + 16, n), 7.0, device='cuda', dtype=dtype)
+    (c,) = gg.gmm_gather(src, w1, sizes)
+    assert torch.equal(c, gg.backend.gmm(a, w1, sizes, trans_b=True))
+    c, h = gg.gmm_gather(src, w1, sizes, act=gg.ACT_GELU_TANH)
+    want_c, want_h = gg.gmm_act(a, w1, sizes, fuse=True)
+    assert torch.equal(c, want_c) and torch.equal(h, want_h)
+    for act in (0, 1):
+        x1, x2, h = gg.gmm_gather(src, w1, sizes, b2=v1, act=act)
+        w_x1, w_x2, w_h = gg.gmm_glu(a, w1, v1, sizes, act, fuse=True)
+        assert torch.equal(x1, w_x1) and torch.equal(x2, w_x2) and torch.equal(h, w_h)
+    assert bool((guard == 7.0).all())
+
+
+def test_gmm_on_gathered_rows_with_assignments_out_of_range(gg):
+    """An assignment outside [0, tokens * top_k) reads as a row of zeros (nothing outside x is fetched), and what the
+    library has no kernel for comes back as None (the caller gathers first)."""
+    tokens, experts, top_k, k, n = 600, 4, 2, 128, 256
+    indices, bin_ids, bins, _, tpe = _routing(tokens, experts, top_k, seed=5)
+    x = torch.randn(tokens, k, device='cuda').to(torch.bfloat16)
+    w1 = (torch.randn(experts, n, k, device='cuda') / k ** 0.5).to(torch.bfloat16)
+    bad = indices.clone()
+    bad[::7] = -1
+    bad[3::11] = tokens * top_k + 5
+    src = gg.GatheredRows(x, bad, bin_ids, bins, None, top_k, tokens * top_k)
+    (c,) = gg.gmm_gather(src, w1, tpe)
+    a = x[(indices.long() // top_k)].clone()
+    a[::7] = 0
+    a[3::11] = 0
+    assert torch.equal(c, gg.backend.gmm(a, w1, tpe, trans_b=True))
+    # fp32, a reduction that is not whole K tiles, 64-bit assignments: no kernel
+    assert gg.gmm_gather(gg.GatheredRows(x.float(), indices, bin_ids, bins, None, top_k, tokens * top_k), w1.float(), tpe) is None
+    assert gg.gmm_gather(gg.GatheredRows(x[:, :72].contiguous(), indices, bin_ids, bins, None, top_k, tokens * top_k),
+                         w1[:, :, :72].contiguous(), tpe) is None
+    assert gg.gmm_gather(gg.GatheredRows(x, indices.long(), bin_ids, bins, None, top_k, tokens * top_k), w1, tpe) is None

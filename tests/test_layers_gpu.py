@@ -836,3 +836,53 @@ def test_memory_optimized_requires_all_grads():
     x = torch.randn(4, 4, 128, device='cuda').bfloat16()     # x does not need grad
     with pytest.raises(ValueError):
         layer(x).sum().backward()
+
+
+@pytest.mark.parametrize('mlp_type,mlp_impl', [('glu', 'grouped'), ('mlp', 'grouped'), ('glu', 'sparse'), ('mlp', 'sparse')])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, mlp_impl, dtype):
+    """The layer with the token gather of dmoe.py:219 / :273 done by the experts' first product (gg.FUSED_GATHER): without
+    gradients that is the default; with gradients it is opt-in and the backward gathers for the weight gradients.
+    Output and every gradient must be the unfused layer's bit for bit (the same kernels on the same values), and the
+    gather kernel must be gone from the forward."""
+    from megablocks_amd import _lib
+    from megablocks_amd import grouped_gemm_util as gg
+    w = syn.Workload('t', 1500, 256, 768, 8, 2, mlp_type, mlp_impl, dtype, 'logits')
+    inp = syn.make_inputs(w, seed=9)
+    layer = syn.build_layer(w, inp)
+    routing = lambda ew: (inp['scores'].to(dtype).cuda(), ew, inp['top_experts'].cuda())
+    grad = inp['grad'].to(dtype).cuda()
+
+    def step(mode, with_grad):
+        monkeypatch.setattr(gg, 'FUSED_GATHER', mode)
+        layer.zero_grad(set_to_none=True)
+        x = inp['x'].to(dtype).cuda().requires_grad_(with_grad)
+        ew = inp['expert_weights'].to(dtype).cuda().requires_grad_(with_grad)
+        _lib.profile_hook = []
+        try:
+            if with_grad:
+                out = syn.layer_step(layer, w, x, grad, routing(ew))
+            else:
+                with torch.no_grad():
+                    out = layer.experts(x, *routing(ew))
+            torch.cuda.synchronize()
+            launched = [name for name, *_ in _lib.profile_hook]
+        finally:
+            _lib.profile_hook = None
+        mlp = layer.experts.mlp
+        grads = [x.grad, ew.grad] + [getattr(mlp, n).grad for n in ('w1', 'v1', 'w2') if hasattr(mlp, n)] if with_grad else []
+        return out.detach().clone(), [g.clone() for g in grads], launched
+
+    first = 'gmm_nt_glu' if mlp_type == 'glu' else 'gmm_nt_act'
+    want, _, launched = step('0', False)
+    assert 'gather' in launched
+    got, _, launched = step('auto', False)
+    assert torch.equal(got, want) and 'gather' not in launched
+    want, want_grads, launched = step('auto', True)                           # gradients recorded: not fused by default
+    assert launched.count('gather') == 1 and launched.index('gather') < launched.index(first)
+    got, got_grads, launched = step('1', True)
+    assert torch.equal(got, want)
+    assert launched.count('gather') == 1 and launched.index('gather') > launched.index(first)   # now in the backward
+    assert len(got_grads) == len(want_grads) >= 4
+    for g, wg in zip(got_grads, want_grads):
+        assert torch.equal(g, wg)
