@@ -294,17 +294,21 @@ int mbx_glu_backward(const void* g, const void* a, const void* b, void* da, void
  * computed in fp32 and rounded to `dtype` where torch's operations round (scores; the norm; the quotient).
  * Weights come out in descending order; equal scores are taken in ascending expert index.  indices are
  * int64 like torch.topk's; indices32 (NULL: not wanted) receives the same values as int32, which saves the layer the
- * `top_expert.int()` pass of megablocks/layers/moe.py:160.  num_experts up to 512 and top_k up to 64, else
- * MBX_EUNSUPPORTED. */
+ * `top_expert.int()` pass of megablocks/layers/moe.py:160.  lse (NULL: not wanted) receives logsumexp(logits, dim=1) in
+ * fp32, [tokens]: the term of the router z-loss, megablocks/layers/router.py:37, which the softmax has at hand.
+ * num_experts up to 512 and top_k up to 64, else MBX_EUNSUPPORTED. */
 int mbx_router_forward(const void* logits, int dtype, int64_t tokens, int num_experts, int top_k, float norm_p,
-                       void* scores, void* weights, int64_t* indices, int32_t* indices32, mbx_stream_t stream);
+                       void* scores, void* weights, int64_t* indices, int32_t* indices32, float* lse,
+                       mbx_stream_t stream);
 
 /* Backward of the above as autograd derives it for router.py:98-106: grad_logits from grad_weights
  * [tokens, top_k] (NULL: none) and, optionally, a gradient that reaches `scores` directly (NULL: none;
- * e.g. from the load-balancing loss, moe.py:32-89), given the forward's scores and indices. */
+ * e.g. from the load-balancing loss, moe.py:32-89), given the forward's scores and indices.  grad_lse (NULL: none): a
+ * gradient that reaches the forward's `lse` ([tokens], fp32; from the z-loss, router.py:25-42); it adds
+ * grad_lse[t] * scores[t, :] to the row. */
 int mbx_router_backward(const void* grad_weights, const void* grad_scores, const void* scores, const int64_t* indices,
                         int dtype, int64_t tokens, int num_experts, int top_k, float norm_p, void* grad_logits,
-                        mbx_stream_t stream);
+                        const float* grad_lse, mbx_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -51,8 +51,8 @@ _SIGNATURES = {
     'mbx_gelu_backward_inplace': (_i, [_vp, _vp, _i, _i64, _vp]),
     'mbx_glu_forward': (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp]),
     'mbx_glu_backward': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _vp]),
-    'mbx_router_forward': (_i, [_vp, _i, _i64, _i, _i, ctypes.c_float, _vp, _vp, _vp, _vp, _vp]),
-    'mbx_router_backward': (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i, _i, ctypes.c_float, _vp, _vp]),
+    'mbx_router_forward': (_i, [_vp, _i, _i64, _i, _i, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp]),
+    'mbx_router_backward': (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i, _i, ctypes.c_float, _vp, _vp, _vp]),
 }
 
 

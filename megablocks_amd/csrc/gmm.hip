@@ -875,10 +875,11 @@ int mbx_gmm_glu(const void* a, const void* b1, const void* b2, void* x1, void* x
 int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int top_k, const int32_t* x_bins, const void* b1,
                    const void* b2, void* c, void* c2, void* h, int dtype, const int32_t* bins, int num_groups, int64_t rows,
                    int k, int n, int act, mbx_stream_t stream) {
-  if (x_rows < 0 || top_k <= 0 || k < 0) return MBX_EINVAL;
+  if (x_rows < 0 || top_k <= 0 || k < 0 || num_groups < 0 || rows < 0 || n < 0) return MBX_EINVAL;
+  if (num_groups == 0 || rows == 0 || n == 0) return 0;   // nothing to write (empty outputs may come as NULL)
   if (b2 ? (act != MBX_ACT_SILU && act != MBX_ACT_GELU_TANH) || !c2 || !h : c2 != nullptr) return MBX_EINVAL;
   if (h && !b2 && act != MBX_ACT_GELU_TANH) return MBX_EUNSUPPORTED;
-  if (num_groups > 0 && rows > 0 && n > 0 && (!indices || (k > 0 && !x && x_rows > 0))) return MBX_EINVAL;
+  if (!indices || (k > 0 && !x && x_rows > 0)) return MBX_EINVAL;
   // the row map is indexed with 32 bits and the rows of x are addressed with 31 (bit 31 marks a row of zeros)
   if (x_rows * top_k > 0x7fffffff || x_rows * (int64_t)k * 2 >= ((int64_t)1 << 31)) return MBX_EUNSUPPORTED;
   if (x_rows == 0 && rows > 0) x = b1;   // no row is read; the buffer descriptor still wants an address

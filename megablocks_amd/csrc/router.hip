@@ -32,7 +32,7 @@ template <int DT, int R>
 __global__ void __launch_bounds__(kTokenThreads)
 router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_experts, int top_k, float p,
                       void* __restrict__ scores_, void* __restrict__ weights_, int64_t* __restrict__ indices,
-                      int32_t* __restrict__ indices32) {
+                      int32_t* __restrict__ indices32, float* __restrict__ lse) {
   typedef typename Elem<DT>::type E;
   const E* logits = (const E*)logits_;
   E* scores = (E*)scores_;
@@ -56,6 +56,8 @@ router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_
       sum += x[r];
     }
     sum = wave_sum(sum);
+    // logsumexp of the row, the term of the router z-loss (router.py:37): an infinite maximum is the result itself
+    if (lse && lane == 0) lse[t] = (m == INFINITY || m == -INFINITY) ? m : m + logf(sum);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int e = lane + r * kWave;
@@ -101,12 +103,14 @@ router_forward_kernel(const void* __restrict__ logits_, int64_t tokens, int num_
 
 // grad_logits = d(loss)/d(logits) given d/d(weights) (and optionally d/d(scores) from other users of the
 // scores, e.g. a load-balancing loss): through the p-norm division, the selection (a scatter to the chosen
-// experts) and the softmax, in fp32 from the rounded forward values.
+// experts) and the softmax, in fp32 from the rounded forward values.  grad_lse (optional): d/d(logsumexp of the
+// row), whose gradient with respect to the logits is the softmax itself.
 template <int DT, int R>
 __global__ void __launch_bounds__(kTokenThreads)
 router_backward_kernel(const void* __restrict__ grad_weights_, const void* __restrict__ grad_scores_,
                        const void* __restrict__ scores_, const int64_t* __restrict__ indices, int64_t tokens,
-                       int num_experts, int top_k, float p, void* __restrict__ grad_logits_) {
+                       int num_experts, int top_k, float p, void* __restrict__ grad_logits_,
+                       const float* __restrict__ grad_lse) {
   typedef typename Elem<DT>::type E;
   const E* grad_weights = (const E*)grad_weights_;
   const E* grad_scores = (const E*)grad_scores_;
@@ -147,10 +151,11 @@ router_backward_kernel(const void* __restrict__ grad_weights_, const void* __res
 #pragma unroll
     for (int r = 0; r < R; ++r) dot += ds[r] * s[r];
     dot = wave_sum(dot);
+    const float gl = grad_lse ? grad_lse[t] : 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int e = lane + r * kWave;
-      if (e < num_experts) grad_logits[t * num_experts + e] = Elem<DT>::from_f32(s[r] * (ds[r] - dot));
+      if (e < num_experts) grad_logits[t * num_experts + e] = Elem<DT>::from_f32(s[r] * (ds[r] - dot + gl));
     }
   }
 }
@@ -197,20 +202,21 @@ using namespace mbx;
 extern "C" {
 
 int mbx_router_forward(const void* logits, int dtype, int64_t tokens, int num_experts, int top_k, float norm_p,
-                       void* scores, void* weights, int64_t* indices, int32_t* indices32, mbx_stream_t stream) {
+                       void* scores, void* weights, int64_t* indices, int32_t* indices32, float* lse,
+                       mbx_stream_t stream) {
   if (tokens < 0 || num_experts <= 0 || top_k <= 0 || top_k > num_experts || !(norm_p >= 0.f)) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
   if (num_experts > kMaxRouterExperts || top_k > kWave) return MBX_EUNSUPPORTED;
   if (tokens == 0) return 0;
   if (!logits || !scores || !weights || !indices) return MBX_EINVAL;
   hipStream_t s = as_stream(stream);
-  MBX_ROUTER_DISPATCH(router_forward_kernel, logits, tokens, num_experts, top_k, norm_p, scores, weights, indices, indices32);
+  MBX_ROUTER_DISPATCH(router_forward_kernel, logits, tokens, num_experts, top_k, norm_p, scores, weights, indices, indices32, lse);
   return launch_status();
 }
 
 int mbx_router_backward(const void* grad_weights, const void* grad_scores, const void* scores, const int64_t* indices,
                         int dtype, int64_t tokens, int num_experts, int top_k, float norm_p, void* grad_logits,
-                        mbx_stream_t stream) {
+                        const float* grad_lse, mbx_stream_t stream) {
   if (tokens < 0 || num_experts <= 0 || top_k <= 0 || top_k > num_experts || !(norm_p >= 0.f)) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
   if (num_experts > kMaxRouterExperts || top_k > kWave) return MBX_EUNSUPPORTED;
@@ -218,7 +224,7 @@ int mbx_router_backward(const void* grad_weights, const void* grad_scores, const
   if (!scores || !grad_logits || (grad_weights && !indices)) return MBX_EINVAL;
   hipStream_t s = as_stream(stream);
   MBX_ROUTER_DISPATCH(router_backward_kernel, grad_weights, grad_scores, scores, indices, tokens, num_experts, top_k,
-                      norm_p, grad_logits);
+                      norm_p, grad_logits, grad_lse);
   return launch_status();
 }
 

@@ -16,10 +16,12 @@ _ROUTER_LOGITS = []
 FUSED_SOFTMAX_TOPK = True
 
 
-def _save_router_logits(logits: torch.Tensor, args: Arguments):
+def _save_router_logits(logits: torch.Tensor, args: Arguments, lse=None):
+    """router.py:17-22.  lse: logsumexp(logits, dim=1) in fp32 where the router kernel has written it (differentiable
+    through that kernel's backward), else None."""
     if args.moe_zloss_weight == 0:
         return
-    _ROUTER_LOGITS.append(logits)
+    _ROUTER_LOGITS.append((logits, lse))
 
 
 def clear_router_zloss():
@@ -32,11 +34,14 @@ def batched_router_zloss(args: Arguments):
         import warnings
         warnings.warn('Call to batched_router_zloss, but moe_zloss_weight=0')
         return 0
-    logits_per_router = _ROUTER_LOGITS
-    if args.moe_zloss_in_fp32:
-        logits_per_router = [logits.float() for logits in logits_per_router]
-    unscaled = torch.stack([torch.logsumexp(logits, dim=1).square().mean() for logits in logits_per_router])
-    return args.moe_zloss_weight * unscaled
+    terms = []
+    for logits, lse in _ROUTER_LOGITS:
+        if lse is None:
+            lse = torch.logsumexp(logits.float() if args.moe_zloss_in_fp32 else logits, dim=1)
+        elif not args.moe_zloss_in_fp32:
+            lse = lse.to(logits.dtype)     # what torch.logsumexp returns for 16-bit logits: computed in fp32, rounded
+        terms.append(lse.square().mean())
+    return args.moe_zloss_weight * torch.stack(terms)
 
 
 class _UniformExpertAssignment(torch.autograd.Function):
@@ -99,8 +104,10 @@ class _RouterLinear(torch.autograd.Function):
 
 class _SoftmaxTopK(torch.autograd.Function):
     """softmax -> top-k -> optional p-norm renormalisation (router.py:87-106) as one kernel each way.
-    Returns (scores, expert_weights, expert_indices, expert_indices as int32) with torch's shapes and dtypes (int64
-    indices); the int32 copy, written by the same kernel, is what the layer's routing takes (moe.py:160 casts)."""
+    Returns (scores, expert_weights, expert_indices, expert_indices as int32, lse) with torch's shapes and dtypes (int64
+    indices); the int32 copy, written by the same kernel, is what the layer's routing takes (moe.py:160 casts); lse
+    (`want_lse`, else None) is logsumexp(logits, dim=1) in fp32, the term of the z-loss (router.py:37), which the
+    backward kernel differentiates along with the rest."""
 
     @staticmethod
     def supported(logits: torch.Tensor, top_k: int) -> bool:
@@ -108,34 +115,36 @@ class _SoftmaxTopK(torch.autograd.Function):
                 and 0 < top_k <= min(64, logits.shape[1]))
 
     @staticmethod
-    def forward(ctx: Any, logits: torch.Tensor, top_k: int, norm_p: float):
+    def forward(ctx: Any, logits: torch.Tensor, top_k: int, norm_p: float, want_lse: bool = False):
         logits = logits.contiguous()
         tokens, experts = logits.shape
         scores = torch.empty_like(logits)
         weights = torch.empty((tokens, top_k), dtype=logits.dtype, device=logits.device)
         indices = torch.empty((tokens, top_k), dtype=torch.int64, device=logits.device)
         indices32 = torch.empty((tokens, top_k), dtype=torch.int32, device=logits.device)
+        lse = torch.empty((tokens,), dtype=torch.float32, device=logits.device) if want_lse else None
         with _lib.device_of(logits):
             _lib.check(_lib.lib.mbx_router_forward(_lib.ptr(logits), _lib.dtype_of(logits), tokens, experts, top_k,
                                                    float(norm_p), _lib.ptr(scores), _lib.ptr(weights), _lib.ptr(indices),
-                                                   _lib.ptr(indices32), _lib.stream()), 'router_forward')
+                                                   _lib.ptr(indices32), _lib.ptr(lse), _lib.stream()), 'router_forward')
         ctx.save_for_backward(scores, indices)
         ctx.top_k, ctx.norm_p = top_k, float(norm_p)
         ctx.mark_non_differentiable(indices, indices32)
-        return scores, weights, indices, indices32
+        return scores, weights, indices, indices32, lse
 
     @staticmethod
-    def backward(ctx: Any, grad_scores, grad_weights, _grad_indices, _grad_indices32):
+    def backward(ctx: Any, grad_scores, grad_weights, _grad_indices, _grad_indices32, grad_lse):
         scores, indices = ctx.saved_tensors
         tokens, experts = scores.shape
         grad_logits = torch.empty_like(scores)
         gs = None if grad_scores is None else grad_scores.to(scores.dtype).contiguous()
         gw = None if grad_weights is None else grad_weights.to(scores.dtype).contiguous()
+        gl = None if grad_lse is None else grad_lse.float().contiguous()
         with _lib.device_of(scores):
             _lib.check(_lib.lib.mbx_router_backward(_lib.ptr(gw), _lib.ptr(gs), _lib.ptr(scores), _lib.ptr(indices),
                                                     _lib.dtype_of(scores), tokens, experts, ctx.top_k, ctx.norm_p,
-                                                    _lib.ptr(grad_logits), _lib.stream()), 'router_backward')
-        return grad_logits, None, None
+                                                    _lib.ptr(grad_logits), _lib.ptr(gl), _lib.stream()), 'router_backward')
+        return grad_logits, None, None, None
 
 
 class LearnedRouter(torch.nn.Module):
@@ -171,20 +180,22 @@ class LearnedRouter(torch.nn.Module):
             logits = _RouterLinear.apply(x2d, self.layer.weight)
         else:
             logits = self.layer(x2d)
-        _save_router_logits(logits, self.args)
+        saved_logits, lse = logits, None
         if logits.is_cuda and logits.dtype != torch.float32 and torch.is_autocast_enabled():
             # autocast runs softmax in fp32 (router.py:98 under torch.autocast): scores and weights come out in fp32
             logits = logits.float()
         expert_indices32 = None
         if FUSED_SOFTMAX_TOPK and _SoftmaxTopK.supported(logits, self.args.moe_top_k):
-            scores, expert_weights, expert_indices, expert_indices32 = _SoftmaxTopK.apply(
-                logits, self.args.moe_top_k, self.args.moe_normalize_expert_weights or 0)
+            scores, expert_weights, expert_indices, expert_indices32, lse = _SoftmaxTopK.apply(
+                logits, self.args.moe_top_k, self.args.moe_normalize_expert_weights or 0,
+                self.args.moe_zloss_weight != 0)
         else:
             scores = logits.softmax(dim=-1)
             expert_weights, expert_indices = self._top_k(scores)
             if self.args.moe_normalize_expert_weights:
                 expert_weights = expert_weights / torch.norm(
                     expert_weights, p=self.args.moe_normalize_expert_weights, dim=-1, keepdim=True)
+        _save_router_logits(saved_logits, self.args, lse)
         if self.args.uniform_expert_assignment:
             expert_indices = _UniformExpertAssignment.apply(expert_indices, self.args.moe_num_experts)
             expert_indices32 = None

@@ -2,6 +2,7 @@
 manner of the reference's tests/layers/{dmoe,glu,moe}_test.py.  Tolerance: relative Frobenius
 error <= 1e-2 for bf16/f16 (north-star bar), 1e-4 for fp32."""
 import dataclasses
+import math
 from functools import partial
 
 import pytest
@@ -221,7 +222,7 @@ def test_router_softmax_topk_fp32_matches_oracle(tokens, experts, top_k, norm_p)
     torch.manual_seed(tokens + experts)
     logits = torch.randn(tokens, experts) * 3
     want_s, want_w, want_i = oracle.router_forward(logits, torch.eye(experts), top_k, norm_p or None)
-    s, w, i, i32 = _SoftmaxTopK.apply(logits.cuda(), top_k, norm_p)
+    s, w, i, i32, _ = _SoftmaxTopK.apply(logits.cuda(), top_k, norm_p)
     assert i32.dtype == torch.int32 and torch.equal(i32.long(), i)
     assert s.dtype == torch.float32 and w.shape == (tokens, top_k) and i.dtype == torch.int64
     assert torch.allclose(s.cpu(), want_s, rtol=1e-5, atol=1e-7)
@@ -238,7 +239,7 @@ def test_router_softmax_topk_16bit(dtype, tokens, experts, top_k, norm_p):
     from megablocks_amd.layers.router import _SoftmaxTopK
     torch.manual_seed(experts)
     logits = (torch.randn(tokens, experts, device='cuda') * 2).to(dtype)
-    s, w, i, _ = _SoftmaxTopK.apply(logits, top_k, norm_p)
+    s, w, i, _, _ = _SoftmaxTopK.apply(logits, top_k, norm_p)
     ref_s, _, _ = _softmax_topk_reference(logits, top_k, norm_p)
     ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     assert ((s.float() - ref_s.float()).abs() <= ulp * ref_s.float().abs() + 1e-30).all()   # at most one rounding step apart
@@ -260,7 +261,7 @@ def test_router_softmax_topk_backward(dtype, experts, top_k, norm_p, with_score_
     gw = torch.randn(tokens, top_k, device='cuda').to(dtype)
     gs = torch.randn(tokens, experts, device='cuda').to(dtype) if with_score_grad else None
     x = logits.clone().requires_grad_(True)
-    s, w, i, _ = _SoftmaxTopK.apply(x, top_k, norm_p)
+    s, w, i, _, _ = _SoftmaxTopK.apply(x, top_k, norm_p)
     loss = (w.float() * gw.float()).sum() + ((s.float() * gs.float()).sum() if with_score_grad else 0)
     loss.backward()
     # reference: autograd through torch's operations in fp32, with the kernel's selection
@@ -272,6 +273,33 @@ def test_router_softmax_topk_backward(dtype, experts, top_k, norm_p, with_score_
     ((wr * gw.float()).sum() + ((sr * gs.float()).sum() if with_score_grad else 0)).backward()
     assert x.grad.dtype == dtype
     assert rel_err(x.grad, xr.grad) < (1e-5 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('tokens,experts,top_k', [(777, 8, 2), (300, 64, 1), (100, 200, 4), (5, 1, 1)])
+def test_router_logsumexp_for_the_zloss(dtype, tokens, experts, top_k):
+    """The router kernel's optional fifth output: logsumexp(logits, dim=1) in fp32 (the term of router.py:37), against
+    torch.logsumexp on the same logits in fp32, and its gradient through the kernel's backward together with a gradient
+    of the weights, against autograd through torch's operations."""
+    from megablocks_amd.layers.router import _SoftmaxTopK
+    torch.manual_seed(tokens + experts)
+    logits = (torch.randn(tokens, experts, device='cuda') * 4).to(dtype)
+    logits[0] = 50.0 if dtype != torch.float16 else 9.0      # large equal logits: lse = value + log(experts)
+    x = logits.clone().requires_grad_(True)
+    s, w, i, _, lse = _SoftmaxTopK.apply(x, top_k, 0, True)
+    assert lse.dtype == torch.float32 and lse.shape == (tokens,)
+    want = torch.logsumexp(logits.float(), dim=1)
+    assert torch.allclose(lse, want, rtol=1e-6, atol=1e-6)
+    assert abs(float(lse[0].detach()) - (float(logits[0, 0]) + math.log(experts))) < 1e-4
+    assert _SoftmaxTopK.apply(logits, top_k, 0)[4] is None
+    gw = torch.randn(tokens, top_k, device='cuda')
+    (lse.square().mean() * 3.0 + (w.float() * gw).sum()).backward()
+    xr = logits.float().clone().requires_grad_(True)
+    (torch.logsumexp(xr, dim=1).square().mean() * 3.0 + (xr.softmax(-1).gather(1, i) * gw).sum()).backward()
+    assert rel_err(x.grad, xr.grad) < (1e-5 if dtype == torch.float32 else 1e-2)
+    # -inf everywhere: -inf, as torch gives it
+    dead = torch.full((2, experts), float('-inf'), device='cuda', dtype=dtype)
+    assert bool((_SoftmaxTopK.apply(dead, top_k, 0, True)[4] == float('-inf')).all())
 
 
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
@@ -288,7 +316,7 @@ def test_router_softmax_topk_with_nan_and_inf_logits(dtype):
     bad[3, 5] = float('nan')
     bad[10, 0] = float('inf')
     bad[20, :] = float('nan')
-    s, w, i, i32 = _SoftmaxTopK.apply(bad, top_k, 1)
+    s, w, i, i32, _ = _SoftmaxTopK.apply(bad, top_k, 1)
     assert torch.equal(i32.long(), i)
     assert int(i.min()) >= 0 and int(i.max()) < experts
     assert bool((i[:, 0] != i[:, 1]).all())
@@ -886,3 +914,51 @@ def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, m
     assert len(got_grads) == len(want_grads) >= 4
     for g, wg in zip(got_grads, want_grads):
         assert torch.equal(g, wg)
+
+
+@pytest.mark.parametrize('mlp_type,tokens,hs,ffn,ne,top_k', [('mlp', 2048, 1024, 1024, 64, 1), ('glu', 1024, 512, 1408, 8, 2)])
+def test_dmoe_forward_replays_from_a_captured_graph(monkeypatch, mlp_type, tokens, hs, ffn, ne, top_k):
+    """The forward pass without gradients, where the first product of the experts reads the ungathered tokens: captured
+    once and replayed with new inputs and eager work in between, every replay gives bit for bit what the eager pass gives,
+    fused or not."""
+    from megablocks_amd import grouped_gemm_util as gg
+    from megablocks_amd.layers.dmoe import dMoE
+    torch.manual_seed(tokens + 1)
+    layer = dMoE(_args(hidden_size=hs, ffn_hidden_size=ffn, moe_num_experts=ne, moe_top_k=top_k, mlp_type=mlp_type,
+                       moe_normalize_expert_weights=1 if top_k > 1 else None))
+    xs = [torch.randn(tokens, 1, hs, device='cuda').bfloat16() for _ in range(3)]
+    with torch.no_grad():
+        monkeypatch.setattr(gg, 'FUSED_GATHER', '0')
+        want = [layer(x).clone() for x in xs]
+        monkeypatch.setattr(gg, 'FUSED_GATHER', 'auto')
+        for x, w in zip(xs, want):
+            assert torch.equal(layer(x), w)
+        static_x = xs[0].clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = layer(static_x)
+        for i in (1, 2, 0, 1, 2, 0):
+            static_x.copy_(xs[i])
+            static_out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_out, want[i])
+            layer(xs[(i + 1) % 3])                                      # eager work between the replays
+
+
+@pytest.mark.parametrize('mlp_type,mlp_impl', [('mlp', 'grouped'), ('glu', 'grouped'), ('mlp', 'sparse'), ('glu', 'sparse')])
+@pytest.mark.parametrize('tokens', [0, 1, 3])
+def test_dmoe_forward_without_gradients_on_no_tokens_and_on_a_few(monkeypatch, mlp_type, mlp_impl, tokens):
+    """Empty and nearly empty batches through the forward whose first product gathers its own rows: most experts (all
+    of them for an empty batch) have no rows, and the result is the unfused layer's."""
+    from megablocks_amd import grouped_gemm_util as gg
+    from megablocks_amd.layers.dmoe import dMoE
+    torch.manual_seed(tokens)
+    layer = dMoE(_args(moe_num_experts=4, moe_top_k=2, mlp_type=mlp_type, mlp_impl=mlp_impl))
+    x = torch.randn(tokens, 1, 128, device='cuda').bfloat16()
+    with torch.no_grad():
+        monkeypatch.setattr(gg, 'FUSED_GATHER', '0')
+        want = layer(x).clone()
+        monkeypatch.setattr(gg, 'FUSED_GATHER', 'auto')
+        got = layer(x)
+    assert got.shape == x.shape and torch.equal(got, want)
