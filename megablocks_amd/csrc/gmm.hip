@@ -629,13 +629,16 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
   if (tiles > 0x7fffffff) return MBX_ERANGE;
   const unsigned grid = (unsigned)persistent_grid(tiles);
+  uint32_t gather_magic = 0;
+  int gather_shift = 0;
+  if (gather.slots) dma::gather_divisor(gather.top_k, gather_magic, gather_shift);
 #define MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, GATHER)                                                    \
   do {                                                                                                \
     auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL, EPI, GATHER>;                             \
     int rc = allow_lds(kern, lds);                                                                    \
     if (rc) return rc;                                                                                \
     kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2,  \
-                                       gather.slots, gather.src_bins, gather.top_k, gather.src_rows);  \
+                                       gather.slots, gather.src_bins, gather.top_k, gather.src_rows, gather_magic, gather_shift);  \
   } while (0)
 #define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI) MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, false)
   if (gather.slots) {

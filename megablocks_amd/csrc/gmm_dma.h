@@ -216,10 +216,10 @@ struct Args {
   // from the second pair.  Used only by the DUAL instantiations.
   __amdgpu_buffer_rsrc_t rsrc_a2, rsrc_b2;
   int nk1;
-  // GATHER instantiations: row r of the A tile is row slots[j0 + r] / top_k of the matrix behind rsrc_a (a_r0 = 0),
-  // zeros when j0 + r >= j1, the slot is negative or the row is not below src_rows.
-  const int32_t* gather_slots;
-  int gather_j0, gather_j1, gather_top_k, gather_src_rows;
+  // GATHER instantiations: the rows of the A tile are rows of the matrix behind rsrc_a picked by a row map.  Load q of
+  // a lane's LA loads of a K tile fetches the 16 bytes at gather_row[q] (+ the K tile's offset); bit 31 set: the row
+  // is a row of zeros.
+  uint32_t gather_row[8];
 };
 
 // acc = (clear ? 0 : acc) + A_tile * B_tile over all K tiles.  On return no load is in flight and no LDS
@@ -496,21 +496,11 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
     return v | (kt < g.nk ? 0u : 0x80000000u);
   };
   // byte offset of the q-th A load's row and 16-byte piece (bit 31: no such row, the load brings zeros)
+  static_assert(!GATHER || LA <= 8, "Args::gather_row");
   uint32_t a_row[GATHER ? LA : 1];
   if constexpr (GATHER) {
-    const uint32_t piece = load_lane_offset<false, BK, T::BM, 16>(wave, 0, 0u, false);   // pitch 0: the piece inside the row
-    const int lane_row = lane_id() >> 3;
-    int slot[LA];
 #pragma unroll
-    for (int q = 0; q < LA; ++q) {
-      const int j = g.gather_j0 + (int)A_ROWS * (wave + q * T::WAVES) + lane_row;
-      slot[q] = j < g.gather_j1 ? g.gather_slots[j] : -1;
-    }
-#pragma unroll
-    for (int q = 0; q < LA; ++q) {
-      const uint32_t row = (uint32_t)slot[q] / (uint32_t)g.gather_top_k;
-      a_row[q] = slot[q] >= 0 && row < (uint32_t)g.gather_src_rows ? row * g.a_ld_bytes + piece : 0x80000000u;
-    }
+    for (int q = 0; q < LA; ++q) a_row[q] = g.gather_row[q];
   }
   __amdgpu_buffer_rsrc_t ra = g.rsrc_a, rb = g.rsrc_b;
   const __amdgpu_buffer_rsrc_t rb_upper = GLU ? g.rsrc_b2 : g.rsrc_b;
@@ -1319,13 +1309,15 @@ struct RowTiles {
 // GATHER: `a` is [src_rows, k] and row r of expert e's rows is a[slots[src_start(e) + r] / top_k] while
 // src_start(e) + r < src_bins[e], zeros after that (src_start(e) = src_bins[e - 1], 0 for the first expert): the
 // product of the rows that megablocks/ops/gather.py:20-38 / padded_gather.py:20-55 would have copied out first.
+// slot / top_k is computed as (slot * top_k_magic) >> (32 + top_k_shift) (see gather_divisor(); top_k = 1: magic 0),
+// a division per row and tile being a few hundred dependent instructions on a wave that has its SIMD to itself.
 template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false, int EPI = kEpiNone, bool GATHER = false>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra,
                 uint16_t* __restrict__ out2, const int32_t* __restrict__ slots, const int32_t* __restrict__ src_bins,
-                int top_k, int src_rows) {
+                int top_k, int src_rows, uint32_t top_k_magic, int top_k_shift) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
   static_assert(!(DUAL && (epi_is_dglu(EPI) || epi_is_glu(EPI))), "a2 / b2 are the second operand pair, the epilogue's x2 or the second matrix");
@@ -1346,43 +1338,12 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   g.nk1 = k / T::BK;
   g.nk = DUAL ? 2 * g.nk1 : g.nk1;
   g.a_r0 = 0;   // the buffers of a and c start at the tile's first row: byte offsets stay small whatever the row count
-  if constexpr (GATHER) {
-    g.gather_slots = slots;
-    g.gather_top_k = top_k;
-    g.gather_src_rows = src_rows;
-  }
   // Work items of this workgroup: one tile per round, then (if the tail is split) one half tile.
   const int items = big_rounds + ((kSplit && split) ? 1 : 0);
-  for (int r = 0; r < items; ++r) {
-    int id, half = 0;
-    bool use_ts = false;
-    if (r < big_rounds) {
-      // Rotated by one member per round: where full and half-height tiles alternate along the list, a
-      // workgroup would otherwise be dealt the same kind in every round.
-      id = (r * kXcds + xcd) * run + (member + r) % run;
-      if (id >= total) break;
-    } else {
-      const int j = xcd * run + member;   // half tile j: tile j / 2 of the tail, rows half j % 2
-      if (j >= 2 * rest) break;
-      id = full_rounds * P + j / 2;
-      half = j & 1;
-      use_ts = true;
-    }
-    int e, start, end, tm, tn;
-    tiles.find(id, e, start, end, tm, tn);
-    const int row0 = start + tm * T::BM + half * TS::BM;
-    if (row0 >= end) break;               // the second half of a tile whose rows end in the first (a last item)
+  // the tile with first row row0 of expert e (rows start .. end - 1), column tile tn
+  auto compute_tile = [&](int e, int end, int tn, int row0, bool use_ts) {
     const uint32_t a_bytes = clip_bytes((rows - row0) * k * 2);   // rows past the tile's are fetched, never stored
-    if constexpr (GATHER) {
-      // the whole source matrix (below 2 GiB: bit 31 of an offset marks a load that must bring zeros)
-      g.rsrc_a = make_rsrc(a, clip_bytes((int64_t)src_rows * k * 2));
-      const int64_t slots_end = (int64_t)src_rows * top_k;
-      const int src_start = e > 0 ? src_bins[e - 1] : 0, src_end = src_bins[e];
-      g.gather_j0 = (src_start < 0 ? 0 : src_start) + (row0 - start);
-      g.gather_j1 = (int)(src_end < slots_end ? src_end : slots_end);
-    } else {
-      g.rsrc_a = make_rsrc(a + (int64_t)row0 * k, a_bytes);
-    }
+    if constexpr (!GATHER) g.rsrc_a = make_rsrc(a + (int64_t)row0 * k, a_bytes);
     g.rsrc_a2 = DUAL ? make_rsrc(a2 + (int64_t)row0 * k, a_bytes) : g.rsrc_a;
     g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
     g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
@@ -1401,7 +1362,118 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
       block_gemm<DT, false, B_MC, T, DUAL, EPI, GATHER>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
     }
     tile_done();
+  };
+  // item r -> expert, its row range, the column tile, the tile's first row, whether it is a half tile of the split
+  // tail; false when the workgroup has no such item (then it has none after it either)
+  auto locate = [&](int r, int& e, int& start, int& end, int& tn, int& row0, bool& tail_half) -> bool {
+    int id, half = 0;
+    tail_half = false;
+    if (r < big_rounds) {
+      // Rotated by one member per round: where full and half-height tiles alternate along the list, a
+      // workgroup would otherwise be dealt the same kind in every round.
+      id = (r * kXcds + xcd) * run + (member + r) % run;
+      if (id >= total) return false;
+    } else {
+      const int j = xcd * run + member;   // half tile j: tile j / 2 of the tail, rows half j % 2
+      if (j >= 2 * rest) return false;
+      id = full_rounds * P + j / 2;
+      half = j & 1;
+      tail_half = true;
+    }
+    int tm;
+    tiles.find(id, e, start, end, tm, tn);
+    row0 = start + tm * T::BM + half * TS::BM;
+    return row0 < end;                    // false: the second half of a tile whose rows end in the first (a last item)
+  };
+  if constexpr (!GATHER) {
+    for (int r = 0; r < items; ++r) {
+      int id, half = 0;
+      bool use_ts = false;
+      if (r < big_rounds) {
+        id = (r * kXcds + xcd) * run + (member + r) % run;   // as in locate()
+        if (id >= total) break;
+      } else {
+        const int j = xcd * run + member;
+        if (j >= 2 * rest) break;
+        id = full_rounds * P + j / 2;
+        half = j & 1;
+        use_ts = true;
+      }
+      int e, start, end, tm, tn;
+      tiles.find(id, e, start, end, tm, tn);
+      const int row0 = start + tm * T::BM + half * TS::BM;
+      if (row0 >= end) break;
+      const uint32_t a_bytes = clip_bytes((rows - row0) * k * 2);   // rows past the tile's are fetched, never stored
+      g.rsrc_a = make_rsrc(a + (int64_t)row0 * k, a_bytes);
+      g.rsrc_a2 = DUAL ? make_rsrc(a2 + (int64_t)row0 * k, a_bytes) : g.rsrc_a;
+      g.rsrc_b = make_rsrc(b + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2));
+      g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
+      // the second matrix of a [w1 | v1] tile: rows BN / 2 .. BN - 1 of the tile are its rows b_r0 .. b_r0 + BN / 2 - 1
+      if (epi_is_glu(EPI)) g.rsrc_b2 = make_rsrc(b2 + ((int64_t)e * n - T::BN / 2) * k, (uint32_t)(((int64_t)n + T::BN / 2) * k * 2));
+      g.b_r0 = tn * kTileCols;
+      uint16_t* const c_tile = c + (int64_t)row0 * n;
+      uint16_t* const e_tile = EPI != kEpiNone ? extra + (int64_t)row0 * n : nullptr;
+      const uint16_t* const p_tile = epi_is_dglu(EPI) ? a2 + (int64_t)row0 * n : nullptr;   // x2 of the gated activation
+      uint16_t* const o_tile = epi_is_dglu(EPI) || epi_is_glu(EPI) ? out2 + (int64_t)row0 * n : nullptr;
+      // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
+      use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
+      if (use_ts) {
+        block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
+      } else {
+        block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
+      }
+      tile_done();
+    }
+  } else {
+    // The assignments of a tile's rows are fetched while the tile before it is computed (the tile's loads cannot start
+    // without them).  Lane l of wave w issues load w + 4 q of the tile, which holds rows 8 (w + 4 q) + l / 8.
+    static_assert(!GATHER || (T::LA >= TS::LA && T::LA <= 8 && T::BK == 64 && T::WAVES == TS::WAVES), "the row map is fetched for the taller tile");
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane_row = lane_id() >> 3;
+    const uint32_t piece = load_lane_offset<false, T::BK, T::BM, 16>(wave, 0, 0u, false);   // pitch 0: the piece inside the row
+    const int64_t slots_end = (int64_t)src_rows * top_k;
+    int next_slot[T::LA];
+    auto fetch_slots = [&](int e, int start, int row0) {
+      const int src_start = e > 0 ? src_bins[e - 1] : 0, src_end = src_bins[e];
+      const int j0 = (src_start < 0 ? 0 : src_start) + (row0 - start);
+      const int j1 = (int)(src_end < slots_end ? src_end : slots_end);
+#pragma unroll
+      for (int q = 0; q < T::LA; ++q) {
+        const int j = j0 + 8 * (wave + q * T::WAVES) + lane_row;
+        next_slot[q] = j < j1 ? slots[j] : -1;
+      }
+    };
+    g.rsrc_a = make_rsrc(a, clip_bytes((int64_t)src_rows * k * 2));   // the whole source matrix, below 2 GiB
+    int e_next, start_next, end_next, tn_next, row0_next;
+    bool use_ts_next;
+    bool have_next = items > 0 && locate(0, e_next, start_next, end_next, tn_next, row0_next, use_ts_next);
+    if (have_next) fetch_slots(e_next, start_next, row0_next);
+    for (int r = 0; have_next; ++r) {
+      const int e = e_next, end = end_next, tn = tn_next, row0 = row0_next;
+      const bool use_ts = use_ts_next;
+      // byte offset of the row and 16-byte piece each of this lane's loads of a K tile fetches (bit 31: a row of zeros)
+#pragma unroll
+      for (int q = 0; q < T::LA; ++q) {
+        const uint32_t row = top_k_magic ? __umulhi((uint32_t)next_slot[q], top_k_magic) >> top_k_shift : (uint32_t)next_slot[q];
+        g.gather_row[q] = next_slot[q] >= 0 && row < (uint32_t)src_rows ? row * g.a_ld_bytes + piece : 0x80000000u;
+      }
+      have_next = r + 1 < items && locate(r + 1, e_next, start_next, end_next, tn_next, row0_next, use_ts_next);
+      if (have_next) fetch_slots(e_next, start_next, row0_next);
+      compute_tile(e, end, tn, row0, use_ts);
+    }
   }
+}
+
+// n / d for 0 <= n < 2^31 as (n * magic) >> (32 + shift): magic = ceil(2^(31 + l) / d) with l = ceil(log2 d) (at least
+// 1) fits 32 bits and gives the exact quotient for every such n; d = 1: magic 0, meaning "no division".
+static inline void gather_divisor(int d, uint32_t& magic, int& shift) {
+  magic = 0;
+  shift = 0;
+  if (d <= 1) return;
+  int l = 1;
+  while ((1 << l) < d) ++l;
+  const uint64_t two = (uint64_t)1 << (31 + l);
+  magic = (uint32_t)((two + (uint64_t)d - 1) / (uint64_t)d);
+  shift = l - 1;
 }
 
 // ---- TN ----

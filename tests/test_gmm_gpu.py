@@ -697,6 +697,7 @@ def _routing(tokens, experts, top_k, seed, blocking=0):
 GATHERED = [  # tokens, experts, top_k, k, n, blocking
     (4096, 8, 2, 1024, 512, 0), (3000, 5, 1, 320, 264, 0), (700, 3, 4, 128, 1408, 0), (37, 1, 1, 64, 8, 0),
     (2048, 16, 4, 256, 384, 128), (1000, 72, 2, 128, 264, 128), (5000, 64, 1, 1024, 1024, 0), (9, 4, 2, 64, 136, 128),
+    (3000, 12, 3, 128, 256, 0), (4000, 64, 6, 192, 1408, 0), (1111, 9, 7, 64, 128, 128), (500, 40, 33, 64, 64, 0),
 ]
 
 
