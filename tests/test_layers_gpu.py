@@ -347,7 +347,7 @@ def test_router_falls_back_to_torch_for_many_experts():
 
 
 @pytest.mark.parametrize('name', ['c2', 'c3', 'c4', 'c5'])
-def test_full_size_layer_properties(syn, name):
+def test_full_size_layer_properties(syn, monkeypatch, name):
     """The benchmark workloads at full size, through properties that do not need an oracle of that size:
     the backward is linear in the upstream gradient (doubling it doubles every gradient exactly: a power
     of two commutes with every rounding on the way), and sampled output rows equal the per-token definition
@@ -376,6 +376,18 @@ def test_full_size_layer_properties(syn, name):
     assert torch.equal(out, out_again)                                   # same kernels, same order: deterministic
     for a, b in zip(g1, g2):
         assert torch.isfinite(a).all() and torch.equal(a * 2, b)
+
+    # the token gather as the operand load of the first product: the forward without gradients (where it is the
+    # default) and the step with it switched on give the same bits
+    from megablocks_amd import grouped_gemm_util as gg
+    with torch.no_grad():
+        assert torch.equal(layer(x) if routing_t is None else layer.experts(x, *routing_t), out)
+    monkeypatch.setattr(gg, 'FUSED_GATHER', '1')
+    out_fused, g_fused = grads(grad)
+    monkeypatch.setattr(gg, 'FUSED_GATHER', 'auto')
+    assert torch.equal(out_fused, out)
+    for a, b in zip(g1, g_fused):
+        assert torch.equal(a, b)
 
     # sampled rows against the definition
     with torch.no_grad():
