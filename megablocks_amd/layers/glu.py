@@ -289,7 +289,9 @@ class SparseGLU(SparseMLP):
     def forward_tokens(self, src, batch_sizes):
         """forward on the rows of the tokens that `src` (a `gg.GatheredRows`) describes, which are then never copied
         out in the forward; None where that is not built (the caller gathers and calls forward)."""
-        if self.args.memory_optimized_mlp:
+        if self.args.memory_optimized_mlp and (torch.is_grad_enabled() or not isinstance(self, GroupedGLU)):
+            # the memory-optimised schedule is a matter of what the backward keeps (without one, the same forward);
+            # with the block-sparse experts it raises (glu.py:47-50), which is left to forward()
             return None
         act = _activation_code(self.args.activation_fn)
         w1, v1, w2 = self._expert_views(self.w1, self.v1, self.w2)

@@ -328,8 +328,10 @@ class SparseMLP(torch.nn.Module):
     def forward_tokens(self, src, batch_sizes):
         """forward on the rows of the tokens that `src` (a `gg.GatheredRows`) describes, which are then never copied
         out in the forward; None where that is not built (the caller gathers and calls forward)."""
-        if self.args.memory_optimized_mlp or self.args.activation_fn is not DEFAULT_ACTIVATION_FN or not src.x.is_cuda:
+        if self.args.activation_fn is not DEFAULT_ACTIVATION_FN or not src.x.is_cuda:
             return None
+        if self.args.memory_optimized_mlp and torch.is_grad_enabled():
+            return None   # the memory-optimised schedule is a matter of what the backward keeps: without one, the same forward
         w1, w2 = self._expert_views(self.w1, self.w2)
         return GatheredGeluMLP.apply(src.x, w1, w2, batch_sizes, src.indices, src.bin_ids, src.bins, src.padded_bins,
                                      src.top_k, src.rows)

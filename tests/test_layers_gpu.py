@@ -974,3 +974,26 @@ def test_dmoe_forward_without_gradients_on_no_tokens_and_on_a_few(monkeypatch, m
         monkeypatch.setattr(gg, 'FUSED_GATHER', 'auto')
         got = layer(x)
     assert got.shape == x.shape and torch.equal(got, want)
+
+
+@pytest.mark.parametrize('mlp_type', ['mlp', 'glu'])
+def test_memory_optimized_dmoe_forward_without_gradients_gathers_in_the_first_product(syn, monkeypatch, mlp_type):
+    """memory_optimized_mlp only changes what the backward keeps: without gradients the layer takes the same forward
+    as the plain one, first product on the ungathered tokens included."""
+    from megablocks_amd import _lib
+    from megablocks_amd import grouped_gemm_util as gg
+    w = syn.Workload('t', 1200, 256, 512, 8, 2, mlp_type, 'grouped', torch.bfloat16, 'logits')
+    inp = syn.make_inputs(w, seed=4)
+    plain, memopt = syn.build_layer(w, inp), syn.build_layer(w, inp, memory_optimized=True)
+    x = inp['x'].bfloat16().cuda()
+    routing = (inp['scores'].bfloat16().cuda(), inp['expert_weights'].bfloat16().cuda(), inp['top_experts'].cuda())
+    with torch.no_grad():
+        want = plain.experts(x, *routing)
+        _lib.profile_hook = []
+        try:
+            got = memopt.experts(x, *routing)
+            torch.cuda.synchronize()
+            launched = [name for name, *_ in _lib.profile_hook]
+        finally:
+            _lib.profile_hook = None
+    assert torch.equal(got, want) and 'gather' not in launched
