@@ -56,6 +56,12 @@ def test_argument_errors_are_reported_without_touching_the_gpu():
     assert lib.mbx_gmm(None, None, None, 0, None, 0, 0, 8, 8, 0, None) == 0     # no groups: nothing to do
     assert lib.mbx_sort(None, 1, 0, 32, None, None, None, 0, None) == 0         # empty input early-out
     assert lib.mbx_cumsum(None, 1, -1, 4, 0, None, None) == -1
+    # mbx_gmm_gather(x, x_rows, indices, top_k, x_bins, b1, b2, c, c2, h, dtype, bins, groups, rows, k, n, act, stream)
+    assert lib.mbx_gmm_gather(None, 8, None, 0, None, None, None, None, None, None, 0, None, 2, 16, 64, 8, 0, None) == -1  # top_k
+    assert lib.mbx_gmm_gather(None, 8, None, 2, None, None, None, None, None, None, 0, None, 2, 0, 64, 8, 0, None) == 0    # no rows
+    assert lib.mbx_gmm_gather(None, 8, None, 2, None, None, None, None, None, None, 0, None, 2, 16, 64, 8, 0, None) == -1  # null map
+    # more tokens than 31 bits of byte offsets address: the caller gathers first
+    assert lib.mbx_gmm_gather(1, 1 << 22, 1, 2, None, 1, None, 1, None, None, 0, 1, 2, 16, 4096, 8, 0, None) == -4
 
 
 def test_host_wrappers_validate_like_the_reference():
