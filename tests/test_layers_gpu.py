@@ -696,6 +696,24 @@ def test_autocast_with_fp32_parameters_equals_the_bf16_layer(mlp_type, mlp_impl,
     assert x32.grad.dtype == torch.float32 and rel_err(x32.grad, x16.grad) < 1e-2
     for (name, p32), p16 in zip(master.named_parameters(), half.parameters()):
         assert p32.grad.dtype == torch.float32 and rel_err(p32.grad, p16.grad) < (2e-2 if 'router' in name else 1e-2), name
+    # the forward without gradients (first product on the ungathered tokens, cast inside) and the step with the gather
+    # fused: what the autocast step above gave
+    from megablocks_amd import grouped_gemm_util as gg
+    with torch.no_grad(), torch.autocast('cuda', dtype=torch.bfloat16):
+        assert torch.equal(master(x32), out)
+    grads = [x32.grad.clone()] + [p.grad.clone() for p in master.parameters()]
+    x32.grad = None
+    master.zero_grad(set_to_none=True)
+    mode, gg.FUSED_GATHER = gg.FUSED_GATHER, '1'
+    try:
+        with torch.autocast('cuda', dtype=torch.bfloat16):
+            fused = master(x32)
+        fused.backward(grad)
+    finally:
+        gg.FUSED_GATHER = mode
+    assert torch.equal(fused, out)
+    for got, ref in zip([x32.grad] + [p.grad for p in master.parameters()], grads):
+        assert got.dtype == ref.dtype and torch.equal(got, ref)
 
 
 def test_parameter_names_and_shapes_are_the_reference_checkpoint_layout():
