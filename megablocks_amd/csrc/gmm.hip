@@ -629,6 +629,17 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   const int64_t tiles = (ceil_div(rows, T::BM) + num_groups) * tiles_n;   // the row counts are only known on the device
   if (tiles > 0x7fffffff) return MBX_ERANGE;
   const unsigned grid = (unsigned)persistent_grid(tiles);
+  // An expert's last row tile, when at most half full, is computed with the half-height tile -- unless a row of tiles is
+  // longer than the run of tiles an XCD's workgroups take per round: the half-height tiles of such a row fill whole
+  // rounds of some XCDs, those finish early, and from then on the XCD's workgroups are no longer within the few K tiles
+  // of each other that the L2 holds (c3's NT launches, 112 and 56 column tiles against runs of 32: L2 misses 5.8 ->
+  // 3.3 GB; the launches themselves take 1 % longer for the padding they multiply, the step is 0.7 % shorter, the
+  // launches after them running at a higher clock).  With shorter rows of tiles the half-height tile wins (every
+  // launch of c2, c4 and c5: 0.7 - 2.8 % per step).  MBX_FULL_SHORT_FROM=N overrides the column-tile count from which
+  // the full tile is used (measurements).
+  static const int full_short_from = [] { const char* v = getenv("MBX_FULL_SHORT_FROM"); return v ? atoi(v) : -1; }();
+  const int run_tiles = (int)grid / kXcds;
+  const int half_limit = tiles_n >= (full_short_from >= 0 ? full_short_from : run_tiles + 1) ? 0 : TS::BM;
   uint32_t gather_magic = 0;
   int gather_shift = 0;
   if (gather.slots) dma::gather_divisor(gather.top_k, gather_magic, gather_shift);
@@ -638,7 +649,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     int rc = allow_lds(kern, lds);                                                                    \
     if (rc) return rc;                                                                                \
     kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2,  \
-                                       gather.slots, gather.src_bins, gather.top_k, gather.src_rows, gather_magic, gather_shift);  \
+                                       gather.slots, gather.src_bins, gather.top_k, gather.src_rows, gather_magic, gather_shift, half_limit);  \
   } while (0)
 #define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI) MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, false)
   if (gather.slots) {

@@ -1309,6 +1309,8 @@ struct RowTiles {
 // GATHER: `a` is [src_rows, k] and row r of expert e's rows is a[slots[src_start(e) + r] / top_k] while
 // src_start(e) + r < src_bins[e], zeros after that (src_start(e) = src_bins[e - 1], 0 for the first expert): the
 // product of the rows that megablocks/ops/gather.py:20-38 / padded_gather.py:20-55 would have copied out first.
+// half_limit: an expert's last row tile with at most this many rows is computed as a TS tile (TS::BM, or 0: never; the
+// launch decides).
 // slot / top_k is computed as (slot * top_k_magic) >> (32 + top_k_shift) (see gather_divisor(); top_k = 1: magic 0),
 // a division per row and tile being a few hundred dependent instructions on a wave that has its SIMD to itself.
 template <int DT, bool B_MC, typename T, typename TS, bool DUAL = false, int EPI = kEpiNone, bool GATHER = false>
@@ -1317,7 +1319,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra,
                 uint16_t* __restrict__ out2, const int32_t* __restrict__ slots, const int32_t* __restrict__ src_bins,
-                int top_k, int src_rows, uint32_t top_k_magic, int top_k_shift) {
+                int top_k, int src_rows, uint32_t top_k_magic, int top_k_shift, int half_limit) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
   static_assert(!(DUAL && (epi_is_dglu(EPI) || epi_is_glu(EPI))), "a2 / b2 are the second operand pair, the epilogue's x2 or the second matrix");
@@ -1355,7 +1357,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     const uint16_t* const p_tile = epi_is_dglu(EPI) ? a2 + (int64_t)row0 * n : nullptr;   // x2 of the gated activation
     uint16_t* const o_tile = epi_is_dglu(EPI) || epi_is_glu(EPI) ? out2 + (int64_t)row0 * n : nullptr;
     // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
-    use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
+    use_ts = kSplit && (use_ts || end - row0 <= half_limit);
     if (use_ts) {
       block_gemm<DT, false, B_MC, TS, DUAL, EPI, GATHER>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
     } else {
@@ -1416,7 +1418,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
       const uint16_t* const p_tile = epi_is_dglu(EPI) ? a2 + (int64_t)row0 * n : nullptr;   // x2 of the gated activation
       uint16_t* const o_tile = epi_is_dglu(EPI) || epi_is_glu(EPI) ? out2 + (int64_t)row0 * n : nullptr;
       // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
-      use_ts = kSplit && (use_ts || end - row0 <= TS::BM);
+      use_ts = kSplit && (use_ts || end - row0 <= half_limit);
       if (use_ts) {
         block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
       } else {
