@@ -98,7 +98,7 @@ class _RouterLinear(torch.autograd.Function):
             sizes = _RouterLinear.piece_sizes(x.shape[0])
             pieces = sizes.shape[0]
             parts = gg.gmm(grad.contiguous(), x.contiguous(), sizes, trans_a=True, _record_as='router_wgrad')   # [pieces, E, h]
-            dw = (parts[0] if pieces == 1 else parts.float().sum(0)).to(ctx.weight_dtype)
+            dw = (parts[0] if pieces == 1 else parts.sum(0, dtype=torch.float32)).to(ctx.weight_dtype)
         return dx, dw
 
 
@@ -130,6 +130,9 @@ class _SoftmaxTopK(torch.autograd.Function):
         ctx.save_for_backward(scores, indices)
         ctx.top_k, ctx.norm_p = top_k, float(norm_p)
         ctx.mark_non_differentiable(indices, indices32)
+        # an output nobody differentiates (the scores without a load-balancing loss, lse without a z-loss, the indices)
+        # arrives in backward as None instead of a zero-filled tensor: three fill launches less per step
+        ctx.set_materialize_grads(False)
         return scores, weights, indices, indices32, lse
 
     @staticmethod
