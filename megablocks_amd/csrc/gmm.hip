@@ -635,11 +635,14 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   // of each other that the L2 holds (c3's NT launches, 112 and 56 column tiles against runs of 32: L2 misses 5.8 ->
   // 3.3 GB; the launches themselves take 1 % longer for the padding they multiply, the step is 0.7 % shorter, the
   // launches after them running at a higher clock).  With shorter rows of tiles the half-height tile wins (every
-  // launch of c2, c4 and c5: 0.7 - 2.8 % per step).  MBX_FULL_SHORT_FROM=N overrides the column-tile count from which
+  // launch of c2, c4 and c5: 0.7 - 2.8 % per step), and with few row tiles per expert the padding would be a large
+  // part of the work.  MBX_FULL_SHORT_FROM=N overrides the column-tile count from which
   // the full tile is used (measurements).
   static const int full_short_from = [] { const char* v = getenv("MBX_FULL_SHORT_FROM"); return v ? atoi(v) : -1; }();
   const int run_tiles = (int)grid / kXcds;
-  const int half_limit = tiles_n >= (full_short_from >= 0 ? full_short_from : run_tiles + 1) ? 0 : TS::BM;
+  // ... and only for experts of eight row tiles and more on average, where the padding is a few percent of the work
+  const bool long_experts = rows >= (int64_t)num_groups * 8 * T::BM;
+  const int half_limit = (full_short_from >= 0 ? tiles_n >= full_short_from : tiles_n > run_tiles && long_experts) ? 0 : TS::BM;
   uint32_t gather_magic = 0;
   int gather_shift = 0;
   if (gather.slots) dma::gather_divisor(gather.top_k, gather_magic, gather_shift);
