@@ -34,11 +34,17 @@ enum mbx_activation { MBX_ACT_SILU = 0, MBX_ACT_GELU_TANH = 1 };
 #define MBX_ESCRATCH (-2) /* scratch buffer too small */
 #define MBX_ERANGE (-3)   /* size beyond what the kernels index with 32 bits */
 #define MBX_EUNSUPPORTED (-4) /* this entry point does not handle the shape / type; use the general form */
+#define MBX_ECAPTURE (-5) /* the call needs a one-time set-up that cannot run under stream capture: mbx_init() first */
 
 /* Human-readable text for a return code (static storage). */
 const char* mbx_error_string(int code);
 /* ABI version of the loaded library. */
 int mbx_version(void);
+/* One-time set-up for the current device (hipSetDevice first), outside stream capture: looks up the addresses of the
+ * device memory that is part of the library image (the buffer of mbx_scatter_static).  Optional -- the entry points
+ * that need it do it on their first call on a device -- except ahead of a first call under stream capture, which
+ * returns MBX_ECAPTURE instead.  Idempotent, thread-safe.  No counterpart in the reference. */
+int mbx_init(void);
 
 /* ------------------------------------------------------------------ routing ops */
 
@@ -63,8 +69,10 @@ int mbx_sort(const void* x, int itype, int64_t n, int end_bit, void* keys_out,
  *   bins                  = inclusive_cumsum(tokens_per_expert)            (csrc/cumsum.h:131)
  *   padded_bins           = inclusive_cumsum(round_up(tokens_per_expert, pad))   if pad > 0 (else not written; may be NULL)
  *   slot_rows (or NULL)   = what mbx_slot_rows builds from these (with padded_bins if pad > 0)
- * bit for bit what the separate entry points give.  An id outside [0, num_experts) is a caller's error here: it is
- * sorted by its low end_bit bits like mbx_sort does, but counted where mbx_histogram would drop it.
+ * bit for bit what the separate entry points give.  An id outside [0, num_experts) is a caller's error here; it is
+ * taken by its low end_bit bits throughout (the order, the counts and the row map agree): one more row of the expert
+ * those bits name, or, if they name none, sorted behind the last bin with row -1 -- where mbx_histogram would drop it
+ * and leave the bins short of the sorted order.  No row inside a bin is left without a slot or padding.
  * scratch: mbx_sort_scratch_bytes(n, MBX_I32, end_bit) bytes.  MBX_EUNSUPPORTED (use the separate entry points):
  * end_bit above 8 or num_experts above 2^end_bit. */
 int mbx_route(const int32_t* expert_ids, int64_t n, int num_experts, int end_bit, int pad, int32_t* indices,
@@ -122,7 +130,8 @@ int mbx_slot_rows(const int32_t* indices, const int32_t* bin_ids, const int32_t*
  * each product rounded to the storage type and the sum taken in fp32, like the
  * reference's two passes but without the [tokens, top_k, hidden] temporary.
  * slot_rows: the map of mbx_slot_rows(), or NULL to have it built here in scratch
- * (4 * tokens * top_k bytes; not used otherwise). */
+ * (4 * tokens * top_k bytes; not used otherwise).  x has padded_bins[num_bins-1] rows, or
+ * tokens * top_k if padded_bins is NULL: an entry of slot_rows at or past that reads as "no row". */
 int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
                 const int32_t* indices, const int32_t* bin_ids, const int32_t* bins,
                 const int32_t* padded_bins, int num_bins, const void* weights, int w_dtype,
@@ -137,7 +146,8 @@ int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
  * process ends) instead of in caller-provided scratch.  It calls no allocator.  tokens * top_k above
  * MBX_STATIC_SCATTER_MAX_SLOTS returns MBX_ERANGE.  All calls on one GPU share that one buffer: calls that may
  * overlap on a GPU (different streams, different threads) race and must be ordered by the caller.  The buffer's
- * address is looked up on the first call on each device; make that call outside stream capture. */
+ * address is looked up by mbx_init() or on the first call on each device; a first call on a stream that is being
+ * captured returns MBX_ECAPTURE and enqueues nothing (call mbx_init() on that device beforehand). */
 #define MBX_STATIC_SCATTER_MAX_SLOTS (1 << 20)
 int mbx_scatter_static(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
                        const int32_t* indices, const int32_t* bin_ids, const int32_t* bins,
@@ -253,7 +263,7 @@ int mbx_gmm_glu(const void* a, const void* b1, const void* b2, void* x1, void* x
  * x: [x_rows, k]; b1, b2: [E, n, k]; c, c2, h: [rows, n].  The results are bit-identical to mbx_gather / mbx_padded_gather
  * followed by mbx_gmm / mbx_gmm_act / mbx_gmm_glu.  An assignment outside [0, x_rows * top_k) reads as a row of zeros.
  * MBX_EUNSUPPORTED (the caller gathers and multiplies in two steps): what mbx_gmm_act / mbx_gmm_glu do not take, x of
- * 2 GiB or more, x_rows * top_k above INT32_MAX, the library running with MBX_MFMA=32. */
+ * 2 GiB or more, x_rows * top_k above INT32_MAX. */
 int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int top_k, const int32_t* x_bins,
                    const void* b1, const void* b2, void* c, void* c2, void* h, int dtype, const int32_t* bins,
                    int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
@@ -265,8 +275,7 @@ int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int to
  *   d1 = round(g * x2) * act'(x1)     (the gradient of sdd_out;  x1 = sdd_out, x2 = v1_out, all [rows, n])
  *   d2 = g * round(act(x1))           (the gradient of v1_out)
  * with the roundings of the separate steps; g itself is not stored.  act: MBX_ACT_SILU or MBX_ACT_GELU_TANH.
- * MBX_EUNSUPPORTED (the caller runs mbx_gmm and mbx_glu_backward): the cases of mbx_gmm_act, and the 32 x 32 x 16
- * main loop. */
+ * MBX_EUNSUPPORTED (the caller runs mbx_gmm and mbx_glu_backward): the cases of mbx_gmm_act. */
 int mbx_gmm_dglu(const void* a, const void* b, const void* x1, const void* x2, void* d1, void* d2, int dtype,
                  const int32_t* bins, int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
 

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, 'libmbx.so')
 I16, I32, I64 = 0, 1, 2
 BF16, F16, F32 = 0, 1, 2
 NN, NT, TN = 0, 1, 2
-EINVAL, ESCRATCH, ERANGE, EUNSUPPORTED = -1, -2, -3, -4
+EINVAL, ESCRATCH, ERANGE, EUNSUPPORTED, ECAPTURE = -1, -2, -3, -4, -5
 
 ITYPE = {torch.int16: I16, torch.int32: I32, torch.int64: I64}
 DTYPE = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
@@ -24,6 +24,7 @@ _vp, _i, _i64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_siz
 _SIGNATURES = {
     'mbx_version': (ctypes.c_int, []),
     'mbx_error_string': (ctypes.c_char_p, [_i]),
+    'mbx_init': (_i, []),
     'mbx_histogram': (_i, [_vp, _i, _i64, _i64, _i, _vp, _vp]),
     'mbx_sort_scratch_bytes': (_sz, [_i64, _i, _i]),
     'mbx_sort': (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _sz, _vp]),

@@ -57,6 +57,17 @@ def remember_slot_rows(indices, bins, padded_bins, rows):
         pass
 
 
+def forget_slot_rows(indices):
+    """Drops the slot -> row map kept on `indices` (see _slot_rows): for callers that rewrite `indices`, `bins` or
+    `padded_bins` in ways torch does not see (raw pointers, a graph replay into them).  The next permutation call
+    builds a new map.  A map that is stale all the same cannot take the kernels out of range: they read it with the
+    row count of the expert-major buffer as a bound."""
+    try:
+        del indices._mbx_slot_rows
+    except AttributeError:
+        pass
+
+
 def _slot_rows(indices, bin_ids, bins, padded_bins):
     """int32 [n_slots]: the row of the expert-major (optionally padded) buffer that holds each slot.  One map
     serves all gathers and scatters of a routing decision, forward and backward, so it is kept on the `indices`

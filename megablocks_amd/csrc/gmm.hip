@@ -2,10 +2,11 @@
 //
 //   NN: c[r_e] = a[r_e] @ b[e]        NT: c[r_e] = a[r_e] @ b[e]^T       TN: c[e] = a[r_e]^T @ b[r_e]
 //
-// Tiling: one workgroup computes a BM x BN tile of c with v_mfma_f32_32x32x16 (bf16 or f16
-// inputs, fp32 accumulators).  Operand tiles are staged through LDS, double buffered, with
-// the global loads of tile t+1 in flight while tile t is multiplied.  An operand whose
-// reduction dimension is contiguous in memory ("KC": a in NN/NT, b in NT) is kept as
+// Two implementations.  The product path is the direct-to-LDS kernels of gmm_dma.h (v_mfma_f32_16x16x32, LDS rings
+// filled by buffer_load ... lds, persistent workgroups with an XCD-aware tile schedule).  This file holds their launch
+// logic, and, for the shapes they do not take, a register-staged kernel (v_mfma_f32_32x32x16, operand tiles loaded
+// into registers, stored to a double-buffered LDS tile) and an element-wise kernel for any shape, alignment and fp32.
+// In all of them an operand whose reduction dimension is contiguous in memory ("KC": a in NN/NT, b in NT) is kept as
 // [row][k] in LDS and read with 128-bit LDS loads; an operand whose reduction dimension is
 // strided ("MC": b in NN, both in TN) is kept as [k][col] and read with the gfx950
 // transposing LDS load (ds_read_b64_tr_b16), which hands every lane the four k-consecutive
@@ -488,30 +489,12 @@ __global__ void __launch_bounds__(256) gelu_backward_vec_kernel(void* __restrict
 // Tile shapes.  256x256x64 with four waves (2x2, 128x128 each) keeps the accumulators in
 // 256 registers per lane and needs 144 KiB of the 160 KiB LDS for two stages.
 typedef Tile<256, 256, 64, 2, 2, 8, 32> TileBig;
+// The tiles of the direct-to-LDS kernels (gmm_dma.h): 256 x 256 x 64, four waves of 128 x 128, three A and two B
+// stages of 32 KiB; and the half-height tile (NN / NT only: the row tile follows the expert's row count) for the last
+// row tile of an expert when it is at most half full, for the tail of a launch, and for launches of small experts;
+// its smaller stages allow a three-deep ring (4 x 16 KiB + 3 x 32 KiB).
 typedef dma::Tile<256, 256, 2, 2, 64, 2> TileDma;
-// Half-height tile (NN / NT only: the row tile follows the expert's row count) for the last row tile of
-// an expert when it is at most half full, for the tail of a launch, and for launches of small experts;
-// its smaller stages allow a three-deep ring.
-typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;   // 4 x 16 KiB + 3 x 32 KiB
-// the same two tiles on the 16 x 16 x 32 instruction
-typedef dma::Tile<256, 256, 2, 2, 64, 2, 16> TileDma16;
-typedef dma::Tile<128, 256, 1, 4, 64, 3, 16> TileDmaSmallM16;
-
-// Which instruction the direct-to-LDS kernels multiply with: 16 x 16 x 32 unless MBX_MFMA=32 is set in the
-// environment (read once).  On operands with random mantissas the power limit lets a loop of 16 x 16 x 32 MFMAs alone
-// run at 2.0 PFLOP/s where 32 x 32 x 16 reaches 1.76 (it moves half the accumulator registers per FLOP), and the
-// 16 x 16 x 32 kernels hold a shader clock of 1.8 - 1.95 GHz on such operands where the others drop to 1.6 - 1.7.
-// The price is issue slots: a wave alone on its SIMD issues one independent instruction every four cycles, an MFMA
-// takes two of those slots, and a 16-cycle MFMA leaves room for two more where a 32-cycle one leaves six, so the
-// loads, LDS reads and address arithmetic of a K tile have to be dealt out one or two to a gap (block_multiply16).
-// Layer step with 16 x 16 x 32 against 32 x 32 x 16, same box, alternating runs: c3 -4.3 %, c4 -3.0 %, c2 -2.2 %.
-static inline bool use_mfma16() {
-  static const bool choice = [] {
-    const char* v = getenv("MBX_MFMA");
-    return !(v && v[0] == '3' && v[1] == '2');
-  }();
-  return choice;
-}
+typedef dma::Tile<128, 256, 1, 4, 64, 3> TileDmaSmallM;
 
 template <int DT, bool A_MC, bool B_MC, typename T>
 constexpr size_t lds_bytes() {
@@ -580,7 +563,7 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
 // TS is the tile the tail of an NN / NT launch is cut into (TS = T: never cut).
 // a2 / b2 non-null (NN / NT only): c = a @ b[e] + a2 @ b2[e], the second pair shaped like the first.
 // epi / extra (NT, one operand pair only): dma::kEpiAct with the second output, dma::kEpiDact with the second input.
-// Rows of `a` gathered on the fly (NT; no epilogue, kEpiAct or kEpiGlu*; 16 x 16 x 32 tiles only): see GatherRows.
+// Rows of `a` gathered on the fly (NT; no epilogue, kEpiAct or kEpiGlu*): see GatherRows.
 struct GatherRows {
   const int32_t* slots = nullptr;      // non-null: a is [src_rows, k], read through the row map
   const int32_t* src_bins = nullptr;
@@ -657,38 +640,26 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
 #define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI) MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, false)
   if (gather.slots) {
     if (layout != MBX_NT || a2 || !gather.src_bins || gather.top_k <= 0) return MBX_EINVAL;
-    if constexpr (T::MF == 16) {
-      switch (epi) {
-        case dma::kEpiNone: MBX_LAUNCH_ROWS_G(false, false, dma::kEpiNone, true); break;
-        case dma::kEpiAct: if (!extra) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiAct, true); break;
-        case dma::kEpiGluSilu: if (!extra || !b2 || !out2) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiGluSilu, true); break;
-        case dma::kEpiGluGelu: if (!extra || !b2 || !out2) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiGluGelu, true); break;
-        default: return MBX_EINVAL;
-      }
-      return launch_status();
-    } else {
-      return MBX_EUNSUPPORTED;
+    switch (epi) {
+      case dma::kEpiNone: MBX_LAUNCH_ROWS_G(false, false, dma::kEpiNone, true); break;
+      case dma::kEpiAct: if (!extra) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiAct, true); break;
+      case dma::kEpiGluSilu: if (!extra || !b2 || !out2) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiGluSilu, true); break;
+      case dma::kEpiGluGelu: if (!extra || !b2 || !out2) return MBX_EINVAL; MBX_LAUNCH_ROWS_G(false, false, dma::kEpiGluGelu, true); break;
+      default: return MBX_EINVAL;
     }
+    return launch_status();
   }
   if (dma::epi_is_glu(epi)) {
-    // b2 is the second matrix of the [w1 | v1] tiles (not a second operand pair); 16 x 16 x 32 tiles only
+    // b2 is the second matrix of the [w1 | v1] tiles (not a second operand pair)
     if (layout != MBX_NT || !extra || !b2 || !out2 || a2) return MBX_EINVAL;
-    if constexpr (T::MF == 16) {
-      if (epi == dma::kEpiGluSilu) MBX_LAUNCH_ROWS(false, false, dma::kEpiGluSilu); else MBX_LAUNCH_ROWS(false, false, dma::kEpiGluGelu);
-      return launch_status();
-    } else {
-      return MBX_EUNSUPPORTED;
-    }
+    if (epi == dma::kEpiGluSilu) MBX_LAUNCH_ROWS(false, false, dma::kEpiGluSilu); else MBX_LAUNCH_ROWS(false, false, dma::kEpiGluGelu);
+    return launch_status();
   }
   if (dma::epi_is_dglu(epi)) {
-    // a2 carries x2 of the gated activation (not a second operand pair); only the 16 x 16 x 32 tiles are instantiated
+    // a2 carries x2 of the gated activation (not a second operand pair)
     if (layout != MBX_NT || !extra || !a2 || !out2) return MBX_EINVAL;
-    if constexpr (T::MF == 16) {
-      if (epi == dma::kEpiDgluSilu) MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluSilu); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluGelu);
-      return launch_status();
-    } else {
-      return MBX_EUNSUPPORTED;
-    }
+    if (epi == dma::kEpiDgluSilu) MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluSilu); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluGelu);
+    return launch_status();
   }
   if (epi != dma::kEpiNone) {
     if (layout != MBX_NT || dual || !extra) return MBX_EINVAL;
@@ -777,14 +748,6 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     if (dma_ok) {
       // TN: the half-height tile only when the product has at most 128 rows (it is slower otherwise)
       const bool small_m = layout == MBX_TN ? k <= TileDmaSmallM::BM : half_height_only(rows, num_groups, n);
-      if (use_mfma16()) {
-        if (small_m) {
-          if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-          return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-        }
-        if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-        return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-      }
       if (small_m) {
         if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
         return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
@@ -816,14 +779,6 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   const bool small_m = half_height_only(rows, num_groups, n);
-  if (use_mfma16()) {
-    if (small_m) {
-      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
-      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
-    }
-    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
-    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
-  }
   if (small_m) {
     if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
     return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
@@ -834,7 +789,7 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
 
 // The NT product with an activation epilogue (epi: dma::kEpiAct / dma::kEpiDact), for the shapes the direct-to-LDS
 // kernels take; anything else is MBX_EUNSUPPORTED and the caller runs the product and the element-wise pass.
-// (kEpiDglu*: pre2 = x2, out2 = the second output; 16 x 16 x 32 main loop only.)
+// (kEpiDglu*: pre2 = x2, out2 = the second output.)
 // (kEpiGlu*: b2 = the second matrix, extra = the gated activation, out2 = the second product.)
 // gather.slots non-null: `a` is read through the row map (no epilogue, kEpiAct and kEpiGlu* only; `extra` may then be
 // null for no epilogue).
@@ -855,21 +810,12 @@ static int gmm_nt_epilogue(const void* a, const void* b, void* c, void* extra, i
   if (glu) ok = ok && aligned16(b2) && aligned16(out2) && dma_sizes_ok(k, n + TileDma::BN / 2);
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
-  if (use_mfma16()) {
-    if (half_height_only(rows, num_groups, n)) {
-      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
-      return gmm_dma<MBX_F16, TileDmaSmallM16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
-    }
-    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
-    return gmm_dma<MBX_F16, TileDma16, TileDmaSmallM16>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
-  }
-  if (dglu || glu || gather.slots) return MBX_EUNSUPPORTED;
   if (half_height_only(rows, num_groups, n)) {
-    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
-    return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
+    return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
   }
-  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
-  return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, nullptr, nullptr, epi, extra);
+  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
+  return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NT, s, pre2, b2, epi, extra, out2, gather);
 }
 
 int mbx_gmm_act(const void* a, const void* b, void* c, void* c_act, int dtype, const int32_t* bins, int num_groups,

@@ -1,7 +1,7 @@
 // Grouped-GEMM main loop with direct-to-LDS global loads and LDS rings of K tiles, and the kernels
 // that walk the tiles of a launch with it.
 //
-// Included by gmm.hip (uses its u32x4 / f32x16 types, mfma32, pack2 and the XCD tile mapping).
+// Included by gmm.hip (uses its u32x4 / f32x4 types, pack2 and the XCD constants).
 //
 // Why: with 256x256 output tiles a compute unit has to pull 64 bytes of operands per 16
 // MFMA-cycles.  Loads that pass through registers can only run one tile ahead and cost 64
@@ -35,19 +35,20 @@ namespace dma {
 // B load can be (the B stage to refill is still being read), so that global -> LDS loads leave the
 // compute unit at an even rate: the texture-address unit takes some 20 cycles per wave-wide load, is
 // shared by the four waves, and a wave whose load has to queue cannot issue its next MFMA either.
-// MF_: rows / columns of the matrix-core instruction: 32 (v_mfma_f32_32x32x16, 16 accumulator registers per product
-// tile, reduction length 16) or 16 (v_mfma_f32_16x16x32: 4 registers, reduction length 32).  Same peak rate, same LDS
-// bytes per FLOP for a given wave tile; the 16 x 16 x 32 form moves half the accumulator registers per FLOP.
-template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_, int MF_ = 32>
+// The matrix-core instruction is v_mfma_f32_16x16x32 (16 x 16 product tiles of four accumulator registers per lane,
+// reduction length 32): MF names its rows / columns.  It has the peak rate and the LDS bytes per FLOP of the
+// 32 x 32 x 16 form and moves half the accumulator registers per FLOP, which under this part's power limit is clock
+// (a loop of nothing but these instructions on operands with random mantissas sustains 2.05 GHz where the other
+// sustains 1.8); a main loop on the 32 x 32 x 16 form was 4 - 6 % slower on every workload and is gone.
+template <int BM_, int BN_, int WM_, int WN_, int BK_, int SB_>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1, MF = MF_;
-  static constexpr int KSTEP = MF == 32 ? 16 : 32;                             // reduction length of one MFMA
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, SB = SB_, SA = SB_ + 1, MF = 16;
+  static constexpr int KSTEP = 32;                                             // reduction length of one MFMA
   static constexpr int KS = BK / KSTEP;                                        // MFMA k-steps per tile
   static constexpr int WAVES = WM * WN, THREADS = WAVES * kWave;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / MF, TN = WTN / MF;
-  typedef typename std::conditional<MF == 32, f32x16, f32x4>::type Acc;        // one product tile of a lane
-  static_assert(MF == 32 || MF == 16, "matrix-core instruction shape");
+  typedef f32x4 Acc;                                                           // one product tile of a lane
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int A_INSTRS = A_BYTES / 1024, B_INSTRS = B_BYTES / 1024;  // wave-wide 1 KiB loads per tile
   static constexpr int LA = A_INSTRS / WAVES, LB = B_INSTRS / WAVES;          // ... per wave
@@ -94,84 +95,57 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
   return v;
 }
 
-// Per-lane byte offset (inside an operand tile) of the MFMA operand of the 32 rows/cols starting
-// at `r`, k-step 0.  KC: k-step s is the same address with bits 5.. XORed by 32 s.  MC: 16 rows (of
-// COLS columns) further per k-step.
-// MF = 16 (16 x 16 x 32 instruction): lane l holds row / column l % 16 and the eight k values 8 (l / 16) ..; k-step s is
-// 32 k further (KC: bits 6.. XORed by 64 s; MC: 32 rows).  The MC layout for this shape swizzles the pair index by
+// Per-lane byte offset (inside an operand tile) of the MFMA operand of the 16 rows / columns starting at `r`, k-step 0.
+// Lane l holds row / column l % 16 and the eight k values 8 (l / 16) ..; k-step s is 32 k further (KC: bits 6.. of the
+// address XORed by 64 s; MC: 32 rows of COLS columns).  The MC layout swizzles the 32-byte pair index by
 // 2 (k & 3) ^ ((k >> 3) & 1): the two 16-lane groups a transposing read serves per cycle hold k rows 8 apart.
-template <bool MC, int BK, int COLS, int MF = 32>
+template <bool MC, int BK, int COLS>
 __device__ __forceinline__ uint32_t frag_lane_offset(int r) {
   const int lane = lane_id();
   if (!MC) {
-    if (MF == 32) {
-      const int row = lane & 31;
-      const int swz = BK == 64 ? (row >> 1) & 7 : (row >> 2) & 3;
-      return (uint32_t)((r + row) * (BK * 2) + (((lane >> 5) ^ swz) << 4));
-    } else {
-      static_assert(MF == 32 || BK == 64, "16 x 16 x 32 operands are read from 128-byte rows");
-      const int row = lane & 15;
-      const int swz = (row >> 1) & 7;
-      return (uint32_t)((r + row) * (BK * 2) + (((lane >> 4) ^ swz) << 4));
-    }
+    static_assert(BK == 64, "operands are read from 128-byte rows");
+    const int row = lane & 15;
+    const int swz = (row >> 1) & 7;
+    return (uint32_t)((r + row) * (BK * 2) + (((lane >> 4) ^ swz) << 4));
   } else {
     const int g = lane >> 4, s = lane & 15;
-    if (MF == 32) {
-      const int k = (g >> 1) * 8 + (s >> 2);
-      const int pair = (r >> 4) + (g & 1);
-      return (uint32_t)(k * (COLS * 2) + ((pair ^ (2 * ((s >> 2) & 3))) << 5) + ((s & 3) << 3));
-    } else {
-      const int k = g * 8 + (s >> 2);
-      const int pair = r >> 4;
-      return (uint32_t)(k * (COLS * 2) + ((pair ^ (2 * ((s >> 2) & 3)) ^ (g & 1)) << 5) + ((s & 3) << 3));
-    }
+    const int k = g * 8 + (s >> 2);
+    const int pair = r >> 4;
+    return (uint32_t)(k * (COLS * 2) + ((pair ^ (2 * ((s >> 2) & 3)) ^ (g & 1)) << 5) + ((s & 3) << 3));
   }
 }
 
-// IMM: constant byte offset of the 32-row tile inside a KC operand tile (goes into the instruction).
-template <bool MC, int KS, int IMM = 0, int COLS = 256, int MF = 32>
-__device__ __forceinline__ u32x4 read_frag(uint32_t tile_addr, uint32_t lane_off) {
-  constexpr int KSTEP = MF == 32 ? 16 : 32;
-  if (!MC) {
-    return lds_read_b128<IMM>(tile_addr + (lane_off ^ (KS * KSTEP * 2)));
-  } else {
-    const u32x2 lo = lds_read_tr16_b64<KS * KSTEP * COLS * 2>(tile_addr + lane_off);
-    const u32x2 hi = lds_read_tr16_b64<KS * KSTEP * COLS * 2 + 4 * COLS * 2>(tile_addr + lane_off);
-    u32x4 v;
-    v[0] = lo[0]; v[1] = lo[1]; v[2] = hi[0]; v[3] = hi[1];
-    return v;
-  }
+// A fragment of a KC operand, k-step KS.  IMM: constant byte offset of the 16-row fragment inside the operand tile (goes
+// into the instruction).
+template <int KS, int IMM>
+__device__ __forceinline__ u32x4 read_frag_kc(uint32_t tile_addr, uint32_t lane_off) {
+  return lds_read_b128<IMM>(tile_addr + (lane_off ^ (KS * 32 * 2)));
 }
 
 // ---- global -> LDS ----
 // Byte offset (from the operand's buffer base) fetched by this lane in the wave's first load of
 // tile 0; `r0` is the tile origin in the non-reduction dimension, `ld_bytes` the row pitch.
-// MF = 16: the MC swizzle has the extra term (k >> 3) & 1 (see frag_lane_offset).  With 256 columns a load holds
-// k = 2 j, 2 j + 1 for load number j = wave + 4 q of the tile, so that term is the parity of q (`odd`); with 128
-// columns (k = 4 j ..) it is (wave >> 1) & 1.
-template <bool MC, int BK, int COLS, int MF = 32>
+// The MC swizzle has the term (k >> 3) & 1 (see frag_lane_offset).  With 256 columns a load holds k = 2 j, 2 j + 1
+// for load number j = wave + 4 q of the tile, so that term is the parity of q (`odd`); with 128 columns (k = 4 j ..) it
+// is (wave >> 1) & 1.
+template <bool MC, int BK, int COLS>
 __device__ __forceinline__ uint32_t load_lane_offset(int wave, int r0, uint32_t ld_bytes, bool odd = false) {
   const int lane = lane_id();
   if (!MC) {
-    if (BK == 64) {  // 8 rows x 8 chunks per instruction; instruction j holds rows 8j .. 8j + 7
-      const int row = lane >> 3, pc = lane & 7;
-      const int c = pc ^ ((4 * (wave & 1) + (row >> 1)) & 7);     // ((8j + row) >> 1) & 7 with j = wave (mod 2)
-      return (uint32_t)(r0 + row) * ld_bytes + (uint32_t)(c << 4);
-    } else {         // 16 rows x 4 chunks per instruction
-      const int row = lane >> 2, pc = lane & 3;
-      const int c = pc ^ ((row >> 2) & 3);
-      return (uint32_t)(r0 + row) * ld_bytes + (uint32_t)(c << 4);
-    }
+    static_assert(BK == 64, "8 rows x 8 chunks per instruction");   // instruction j holds rows 8j .. 8j + 7
+    const int row = lane >> 3, pc = lane & 7;
+    const int c = pc ^ ((4 * (wave & 1) + (row >> 1)) & 7);     // ((8j + row) >> 1) & 7 with j = wave (mod 2)
+    return (uint32_t)(r0 + row) * ld_bytes + (uint32_t)(c << 4);
   } else if (COLS == 256) {   // 2 k-rows x 32 chunks per instruction; instruction j holds k = 2j, 2j + 1
     const int kl = lane >> 5, pc = lane & 31;
     const int k3 = (2 * (wave & 1) + kl) & 3;                     // (2j + kl) & 3 with j = wave (mod 2)
-    const int x = (2 * k3) ^ ((MF == 16 && odd) ? 1 : 0);
+    const int x = (2 * k3) ^ (odd ? 1 : 0);
     const int c = ((((pc >> 1) ^ x) << 1) | (pc & 1));
     return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
   } else {                    // 128 columns: 4 k-rows x 16 chunks per instruction; instruction j holds k = 4j .. 4j + 3
     static_assert(!MC || COLS == 256 || COLS == 128, "strided operand tile width");
     const int kl = lane >> 4, pc = lane & 15;
-    const int x = (2 * kl) ^ (MF == 16 ? (wave >> 1) & 1 : 0);
+    const int x = (2 * kl) ^ ((wave >> 1) & 1);
     const int c = ((((pc >> 1) ^ x) << 1) | (pc & 1));
     return (uint32_t)kl * ld_bytes + (uint32_t)(r0 * 2) + (uint32_t)(c << 4);
   }
@@ -222,221 +196,6 @@ struct Args {
   uint32_t gather_row[8];
 };
 
-// acc = (clear ? 0 : acc) + A_tile * B_tile over all K tiles.  On return no load is in flight and no LDS
-// read is pending, but other waves may still be reading the last stages.
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false>
-__device__ __forceinline__ void block_multiply32(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
-  static_assert(T::MF == 32, "the schedule below is written for the 32 x 32 x 16 instruction");
-  const lds_ptr lds = (lds_ptr)lds_generic;
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
-
-  constexpr int BK = T::BK, SA = T::SA, SB = T::SB, LA = T::LA, LB = T::LB;
-  static_assert(T::KS == 4, "the schedule below is written for four k-steps per K tile");
-  constexpr uint32_t B_RING = (uint32_t)SA * T::A_BYTES;   // the B stages follow the A stages
-  const uint32_t a_lane = load_lane_offset<A_MC, BK, T::BM>(wave, g.a_r0, g.a_ld_bytes);
-  const uint32_t b_lane = load_lane_offset<B_MC, BK, T::BN>(wave, g.b_r0, g.b_ld_bytes);
-  const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
-  const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
-  // The q-th wave-wide load of this wave's share of an operand tile is load number j = wave + q WAVES
-  // of the tile: 1 KiB of LDS at j KiB, global rows j ROWS onwards.  Byte offset into the operand =
-  // lane part (a_lane / b_lane) + scalar part; the scalar part of K tile kt, load j is
-  // kt a_step + j a_jstep.  A tile index at or past nk gets bit 31 set in the scalar part (operands are
-  // below 2 GiB): the load is then out of range, fetches nothing and writes zeros into a stage nobody
-  // reads, which keeps the loop and its vmcnt bookkeeping uniform.
-  constexpr uint32_t A_ROWS = (uint32_t)(1024 / ((A_MC ? T::BM : BK) * 2)), B_ROWS = (uint32_t)(1024 / ((B_MC ? T::BN : BK) * 2));   // operand rows per load
-  const uint32_t a_jstep = A_ROWS * g.a_ld_bytes, b_jstep = B_ROWS * g.b_ld_bytes;
-  auto scalar_off = [&](bool is_b, int kt, int q) -> uint32_t {   // prologue: K tiles of the first operand pair
-    const uint32_t j = (uint32_t)(wave + q * T::WAVES);
-    const uint32_t v = is_b ? (uint32_t)kt * b_step + j * b_jstep : (uint32_t)kt * a_step + j * a_jstep;
-    return v | (kt < g.nk ? 0u : 0x80000000u);
-  };
-  __amdgpu_buffer_rsrc_t ra = g.rsrc_a, rb = g.rsrc_b;   // the operand pair the loads being issued read
-  auto lds_off = [&](bool is_b, int stage, int q) -> uint32_t {
-    return (is_b ? B_RING + (uint32_t)stage * T::B_BYTES : (uint32_t)stage * T::A_BYTES) + (uint32_t)(wave + q * T::WAVES) * 1024u;
-  };
-  auto issue = [&](bool is_b, uint32_t sc, uint32_t dst) {
-    if (is_b) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(b_lane + sc), 0, 0, 0);
-    } else {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(a_lane + sc), 0, 0, 0);
-    }
-  };
-  auto issue_group = [&](bool is_b, int kt, int stage, int q0, int count) {   // prologue
-    uint32_t sc = scalar_off(is_b, kt, q0), dst = lds_off(is_b, stage, q0);
-    for (int i = 0; i < count; ++i) {
-      issue(is_b, sc, dst);
-      sc += T::WAVES * (is_b ? b_jstep : a_jstep);
-      dst += T::WAVES * 1024u;
-    }
-  };
-
-  // per-lane LDS offsets of the MFMA operands (KC: one base, 32-row tiles at +32 rows; MC: one per tile)
-  constexpr int KC_TILE = 32 * BK * 2;
-  uint32_t fa_off[A_MC ? T::TM : 1], fb_off[B_MC ? T::TN : 1];
-  if (A_MC) {
-#pragma unroll
-    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true, BK, T::BM>(wm + i * 32);
-  } else {
-    fa_off[0] = frag_lane_offset<false, BK, T::BM>(wm);
-  }
-  if (B_MC) {
-#pragma unroll
-    for (int j = 0; j < T::TN; ++j) fb_off[j] = frag_lane_offset<true, BK, T::BN>(wn + j * 32);
-  } else {
-    fb_off[0] = frag_lane_offset<false, BK, T::BN>(wn);
-  }
-
-  u32x4 fa[2][T::TM], fb[2][T::TN];
-  // m-th operand read (of TM + TN) of k-step KSTEP of the tiles at A_ADDR / B_ADDR into register buffer BUF
-#define MBX_READ_ONE(KSTEP, BUF, A_ADDR, B_ADDR, M)                                                              \
-  do {                                                                                                           \
-    if constexpr ((M) < T::TM) {                                                                                 \
-      constexpr int i_ = (M);                                                                                    \
-      if constexpr (A_MC) fa[BUF][i_] = read_frag<true, KSTEP, 0, T::BM>(A_ADDR, fa_off[A_MC ? i_ : 0]);                   \
-      else fa[BUF][i_] = read_frag<false, KSTEP, i_ * KC_TILE>(A_ADDR, fa_off[0]);                               \
-    } else if constexpr ((M) < T::TM + T::TN) {                                                                  \
-      constexpr int j_ = (M) - T::TM;                                                                            \
-      if constexpr (B_MC) fb[BUF][j_] = read_frag<true, KSTEP, 0, T::BN>(B_ADDR, fb_off[B_MC ? j_ : 0]);                   \
-      else fb[BUF][j_] = read_frag<false, KSTEP, j_ * KC_TILE>(B_ADDR, fb_off[0]);                               \
-    }                                                                                                            \
-  } while (0)
-#define MBX_READ_FRAGS(KSTEP, BUF, A_ADDR, B_ADDR)                                                               \
-  do {                                                                                                           \
-    static_for<T::TM + T::TN>([&](auto mi_) { constexpr int m_ = decltype(mi_)::value; MBX_READ_ONE(KSTEP, BUF, A_ADDR, B_ADDR, m_); }); \
-  } while (0)
-  // the MFMAs may only start once the operands have arrived: tie them to the wait through "+v"
-#define MBX_WAIT_FRAGS(BUF) wait_frags(fa[BUF], fb[BUF])
-  // One k-step: TM x TN MFMAs on register buffer CUR_BUF.  Interleaved with them, so that neither
-  // the LDS nor the texture-address unit makes the wave wait with the matrix core idle:
-  //   * the operand reads of the next k-step (NEXT_KSTEP of the tiles at NEXT_A / NEXT_B) into the other buffer,
-  //   * NLOADS global->LDS loads of operand IS_B at the running scalar offset SC into LDS at DST (both
-  //     advanced here),
-  //   * PREP(), the scalar bookkeeping for the following k-steps, behind one of the later MFMAs.
-  // A wave issues at most one instruction every four cycles, eight per MFMA: every instruction placed
-  // between the MFMAs counts, also the scalar ones, and none should be left for the gap between k-steps.
-  // The accumulator tile is c^T (operands swapped): a lane owns runs of four consecutive columns
-  // of one row of c and can store them as one 8-byte word.
-#define MBX_STEP(CUR_BUF, NEXT_KSTEP, NEXT_A, NEXT_B, IS_B, SC, DST, NLOADS, PREP)                               \
-  do {                                                                                                           \
-    /* The operand reads go behind the first TM + TN MFMAs; with 16 MFMAs per k-step the loads go behind   */  \
-    /* every second MFMA of the other half and the bookkeeping between them, so that no MFMA has more than */  \
-    /* a handful of instructions queued behind it.  With 8 MFMAs per k-step the loads are spread over all. */  \
-    constexpr int n_ = T::TM * T::TN, half_ = n_ / 2;                                                            \
-    constexpr bool late_ = half_ >= T::TM + T::TN && half_ / (NLOADS) >= 2;                                      \
-    constexpr int every_ = (late_ ? half_ : n_) / (NLOADS), first_ = late_ ? half_ : 0;                          \
-    static_assert(every_ >= 2, "not enough MFMAs per k-step to hide the loads behind");                          \
-    MBX_WAIT_FRAGS(CUR_BUF);                                                                                     \
-    __builtin_amdgcn_sched_barrier(0);                                                                           \
-    static_for<n_>([&](auto mi_) {                                                                               \
-      constexpr int m_ = decltype(mi_)::value;                                                                   \
-      /* boustrophedon order over the TM x TN products: consecutive MFMAs differ in one operand only */         \
-      constexpr int i_ = m_ / T::TN, j_ = (i_ & 1) ? T::TN - 1 - m_ % T::TN : m_ % T::TN;                        \
-      acc[i_][j_] = mfma32<DT>(fb[CUR_BUF][j_], fa[CUR_BUF][i_], acc[i_][j_]);                                   \
-      MBX_READ_ONE(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                               \
-      if (m_ >= first_ && (m_ - first_) % every_ == every_ - 1 && (m_ - first_) / every_ < (NLOADS)) {           \
-        issue(IS_B, SC, DST);                                                                                    \
-        SC += T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                                           \
-        DST += T::WAVES * 1024u;                                                                                 \
-      }                                                                                                          \
-      if (m_ == (late_ ? n_ - 4 : half_ + 1)) PREP();                                                            \
-      __builtin_amdgcn_sched_barrier(0);                                                                         \
-    });                                                                                                          \
-  } while (0)
-
-  const int nk = g.nk;
-  auto clear_acc = [&]() {
-#pragma unroll
-    for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < T::TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  };
-  // Iteration kt multiplies K tile kt (A stage kt % SA, B stage kt % SB) and issues, spread evenly
-  // over its four k-steps:
-  //   k-step 0: the second half of B tile kt + SB - 1 -> B stage (kt - 1) % SB   (free since the barrier of kt - 1)
-  //   k-steps 1, 2: the halves of A tile kt + SB      -> A stage (kt - 1) % SA   (likewise)
-  //   barrier: every wave has tile kt in registers and tile kt + 1 has landed
-  //   k-step 3: the first half of B tile kt + SB      -> B stage kt % SB         (free since that barrier)
-  // Loads complete in order, so "tile kt + 1 has landed" is "at most WAIT_LOOP of my loads in flight".
-  constexpr int WAIT_PROLOGUE = (SB - 2) * (LA + LB) + LA + LB / 2;
-  constexpr int WAIT_LOOP = (SB - 1) * LA + (SB - 2) * LB;
-  if (nk > 0) {
-    // prologue: tiles 0 .. SB-2, the A part and half of the B part of tile SB-1, then wait for tile 0
-#pragma unroll
-    for (int t = 0; t < SB - 1; ++t) {
-      issue_group(false, t, t, 0, LA);
-      issue_group(true, t, t, 0, LB);
-    }
-    issue_group(false, SB - 1, SB - 1, 0, LA);
-    issue_group(true, SB - 1, SB - 1, 0, LB / 2);
-  }
-  __builtin_amdgcn_sched_barrier(0);   // the loads are on their way before the accumulators are cleared
-  if (clear) clear_acc();
-  if (nk > 0) {
-    wait_vmcnt<WAIT_PROLOGUE>();
-    __builtin_amdgcn_s_barrier();
-    MBX_READ_FRAGS(0, 0, lds_base, lds_base + B_RING);
-
-    // Running state, all scalar.  LDS addresses of the stages being multiplied (tile kt) and of the
-    // next ones; LDS offset and scalar global offset of the A loads of this iteration (tile kt + SB,
-    // stage (kt - 1) % SA) and of the B loads that start in its k-step 3 (tile kt + SB, stage kt % SB).
-    constexpr uint32_t A_RING_END = (uint32_t)SA * T::A_BYTES, B_RING_END = B_RING + (uint32_t)SB * T::B_BYTES;
-    uint32_t a_rd = lds_base, b_rd = lds_base + B_RING, a_rd_next = 0, b_rd_next = 0;
-    uint32_t a_dst0 = lds_off(false, SA - 1, 0), b_dst0 = lds_off(true, 0, 0);
-    uint32_t a_sc0 = (uint32_t)SB * a_step + (uint32_t)wave * a_jstep, b_sc0 = (uint32_t)SB * b_step + (uint32_t)wave * b_jstep;
-    const uint32_t a_dst_end = A_RING_END + (uint32_t)wave * 1024u, b_dst_end = B_RING_END + (uint32_t)wave * 1024u;
-    // the loads in flight: B continues with the second half of tile SB - 1
-    uint32_t sc_b = scalar_off(true, SB - 1, LB / 2), dst_b = lds_off(true, SB - 1, LB / 2), sc_a = 0, dst_a = 0;
-    uint32_t past = 0;
-    for (int kt = 0; kt < nk; ++kt) {
-      auto prep0 = [&]() {   // the A loads of k-steps 1 and 2
-        past = kt + SB < nk ? 0u : 0x80000000u;
-        sc_a = a_sc0 | past;
-        dst_a = a_dst0;
-        if (DUAL) ra = kt + SB >= g.nk1 ? g.rsrc_a2 : g.rsrc_a;
-      };
-      auto prep1 = [&]() {
-        a_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * a_jstep : a_sc0 + a_step;   // K tile kt + SB + 1
-        a_dst0 += T::A_BYTES;
-        a_dst0 = a_dst0 >= a_dst_end ? a_dst0 - A_RING_END : a_dst0;
-      };
-      auto prep2 = [&]() {   // the B loads of k-step 3 and of k-step 0 of the next iteration; the next stages to read
-        sc_b = b_sc0 | past;
-        dst_b = b_dst0;
-        if (DUAL) rb = kt + SB >= g.nk1 ? g.rsrc_b2 : g.rsrc_b;
-        a_rd_next = a_rd + T::A_BYTES;
-        a_rd_next = a_rd_next >= lds_base + A_RING_END ? lds_base : a_rd_next;
-        b_rd_next = b_rd + T::B_BYTES;
-        b_rd_next = b_rd_next >= lds_base + B_RING_END ? lds_base + B_RING : b_rd_next;
-      };
-      auto prep3 = [&]() {
-        b_sc0 = DUAL && kt + SB + 1 == g.nk1 ? (uint32_t)wave * b_jstep : b_sc0 + b_step;
-        b_dst0 += T::B_BYTES;
-        b_dst0 = b_dst0 >= b_dst_end ? b_dst0 - (uint32_t)SB * T::B_BYTES : b_dst0;
-      };
-      MBX_STEP(0, 1, a_rd, b_rd, true, sc_b, dst_b, LB / 2, prep0);
-      MBX_STEP(1, 2, a_rd, b_rd, false, sc_a, dst_a, LA / 2, prep1);
-      MBX_STEP(0, 3, a_rd, b_rd, false, sc_a, dst_a, LA / 2, prep2);
-      MBX_WAIT_FRAGS(1);
-      wait_vmcnt<WAIT_LOOP>();
-      __builtin_amdgcn_s_barrier();
-      MBX_STEP(1, 0, a_rd_next, b_rd_next, true, sc_b, dst_b, LB / 2, prep3);   // past the last tile this reads stale LDS into dead registers
-      a_rd = a_rd_next;
-      b_rd = b_rd_next;
-    }
-    wait_vmcnt<0>();   // no load may still be writing LDS when the workgroup's LDS is handed on
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // nor an LDS read still be landing in a register the epilogue reuses
-  }
-
-#undef MBX_READ_FRAGS
-#undef MBX_WAIT_FRAGS
-#undef MBX_READ_ONE
-#undef MBX_STEP
-}
-
 // acc += a-fragment x b-fragment with v_mfma_f32_16x16x32, written as inline asm with the accumulator tied to one
 // register tuple ("+a": an AGPR tuple, source and destination): with the builtin, whose destination may differ from
 // its accumulator source, the register allocator gave the 64 four-register tiles of a wave other registers at the
@@ -469,7 +228,7 @@ __device__ __forceinline__ void mfma16_settle() { asm volatile("s_nop 15\n\ts_no
 // multiple of the row pitch to one lane offset.  The loads are the same 16-byte pieces of 128-byte row segments.
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false>
 __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
-  static_assert(T::MF == 16 && T::KS == 2, "two k-steps of 32 per K tile");
+  static_assert(T::KS == 2, "two k-steps of 32 per K tile");
   static_assert(!GLU || (!B_MC && !DUAL && T::LB % 2 == 0), "two matrices side by side in the B tile");
   static_assert(!GATHER || (!A_MC && !DUAL && T::BK == 64), "gathered rows: a KC operand, one operand pair");
   const lds_ptr lds = (lds_ptr)lds_generic;
@@ -482,10 +241,10 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
   // a 256-column MC operand takes its lane offsets from the parity of the load's index inside the tile
   constexpr bool A_QDEP = A_MC && T::BM == 256, B_QDEP = B_MC && T::BN == 256;
   static_assert((LA / 2) % 2 == 0 && (LB / 2) % 2 == 0, "every group of loads starts at an even load index");
-  const uint32_t a_lane = load_lane_offset<A_MC, BK, T::BM, 16>(wave, g.a_r0, g.a_ld_bytes, false);
-  const uint32_t b_lane = load_lane_offset<B_MC, BK, T::BN, 16>(wave, g.b_r0, g.b_ld_bytes, false);
-  const uint32_t a_lane1 = A_QDEP ? load_lane_offset<A_MC, BK, T::BM, 16>(wave, g.a_r0, g.a_ld_bytes, true) : a_lane;
-  const uint32_t b_lane1 = B_QDEP ? load_lane_offset<B_MC, BK, T::BN, 16>(wave, g.b_r0, g.b_ld_bytes, true) : b_lane;
+  const uint32_t a_lane = load_lane_offset<A_MC, BK, T::BM>(wave, g.a_r0, g.a_ld_bytes, false);
+  const uint32_t b_lane = load_lane_offset<B_MC, BK, T::BN>(wave, g.b_r0, g.b_ld_bytes, false);
+  const uint32_t a_lane1 = A_QDEP ? load_lane_offset<A_MC, BK, T::BM>(wave, g.a_r0, g.a_ld_bytes, true) : a_lane;
+  const uint32_t b_lane1 = B_QDEP ? load_lane_offset<B_MC, BK, T::BN>(wave, g.b_r0, g.b_ld_bytes, true) : b_lane;
   const uint32_t a_step = A_MC ? BK * g.a_ld_bytes : BK * 2;   // bytes per K tile
   const uint32_t b_step = B_MC ? BK * g.b_ld_bytes : BK * 2;
   constexpr uint32_t A_ROWS = (uint32_t)(1024 / ((A_MC ? T::BM : BK) * 2)), B_ROWS = (uint32_t)(1024 / ((B_MC ? T::BN : BK) * 2));
@@ -530,15 +289,15 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
   uint32_t fa_off[A_MC ? T::TM : 1], fb_off[B_MC ? T::TN : 1];
   if (A_MC) {
 #pragma unroll
-    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true, BK, T::BM, 16>(wm + i * 16);
+    for (int i = 0; i < T::TM; ++i) fa_off[i] = frag_lane_offset<true, BK, T::BM>(wm + i * 16);
   } else {
-    fa_off[0] = frag_lane_offset<false, BK, T::BM, 16>(wm);
+    fa_off[0] = frag_lane_offset<false, BK, T::BM>(wm);
   }
   if (B_MC) {
 #pragma unroll
-    for (int j = 0; j < T::TN; ++j) fb_off[j] = frag_lane_offset<true, BK, T::BN, 16>(wn + j * 16);
+    for (int j = 0; j < T::TN; ++j) fb_off[j] = frag_lane_offset<true, BK, T::BN>(wn + j * 16);
   } else {
-    fb_off[0] = frag_lane_offset<false, BK, T::BN, 16>(wn);
+    fb_off[0] = frag_lane_offset<false, BK, T::BN>(wn);
   }
 
   if (A_MC) {
@@ -569,7 +328,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
         fa[BUF][i_][2 * h_] = t_[0];                                                                             \
         fa[BUF][i_][2 * h_ + 1] = t_[1];                                                                         \
       } else {                                                                                                   \
-        fa[BUF][(R)] = read_frag<false, KSTEP, (R) * KC_TILE, 256, 16>(A_ADDR, fa_off[0]);                       \
+        fa[BUF][(R)] = read_frag_kc<KSTEP, (R) * KC_TILE>(A_ADDR, fa_off[0]);                       \
       }                                                                                                          \
     } else if constexpr ((R) < NS) {                                                                             \
       constexpr int r_ = (R) - NSA;                                                                              \
@@ -579,7 +338,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
         fb[BUF][j_][2 * h_] = t_[0];                                                                             \
         fb[BUF][j_][2 * h_ + 1] = t_[1];                                                                         \
       } else {                                                                                                   \
-        fb[BUF][r_] = read_frag<false, KSTEP, r_ * KC_TILE, 256, 16>(B_ADDR, fb_off[0]);                         \
+        fb[BUF][r_] = read_frag_kc<KSTEP, r_ * KC_TILE>(B_ADDR, fb_off[0]);                         \
       }                                                                                                          \
     }                                                                                                            \
   } while (0)
@@ -731,9 +490,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
 
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false>
 __device__ __forceinline__ void block_multiply(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds) {
-  static_assert((!GLU && !GATHER) || T::MF == 16, "two matrices side by side, gathered rows: 16 x 16 x 32 loop only");
-  if constexpr (T::MF == 32) block_multiply32<DT, A_MC, B_MC, T, DUAL>(g, acc, clear, lds);
-  else block_multiply16<DT, A_MC, B_MC, T, DUAL, GLU, GATHER>(g, acc, clear, lds);
+  block_multiply16<DT, A_MC, B_MC, T, DUAL, GLU, GATHER>(g, acc, clear, lds);
 }
 
 // ---- activation in the epilogue (tanh-GELU: megablocks/layers/arguments.py:19, megablocks/layers/gelu.py:9-13) ----
@@ -930,12 +687,10 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
   const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
   // accumulator (i, j), register r of lane l holds c[m][n] with
-  //   32 x 32 x 16: m = m_base + wm + 32 i + (l % 32),  n = n_base + wn + 32 j + 8 (r / 4) + 4 (l / 32) + (r % 4)
-  //   16 x 16 x 32: m = m_base + wm + 16 i + (l % 16),  n = n_base + wn + 16 j + 4 (l / 16) + r
-  // i.e. runs of four consecutive columns per lane: Q runs per product tile, at column run_col(q), of row tile_row.
-  constexpr int MF = T::MF, Q = MF == 32 ? 4 : 1;
-  const int tile_row = MF == 32 ? (lane & 31) : (lane & 15);
-  auto run_col = [&](int q) -> int { return MF == 32 ? q * 8 + (lane >> 5) * 4 : (lane >> 4) * 4; };
+  //   m = m_base + wm + 16 i + (l % 16),  n = n_base + wn + 16 j + 4 (l / 16) + r
+  // i.e. a run of four consecutive columns per lane and product tile.
+  constexpr int MF = T::MF;
+  const int tile_row = lane & 15, run_col = (lane >> 4) * 4;
   {
     // Staged through LDS (free by now) so that every global store instruction writes whole rows of the
     // tile: 64 lanes x 16 bytes = two 512-byte row segments, instead of 32 scattered 16-byte pieces.
@@ -946,16 +701,12 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
       const int ml = wm + i * MF + tile_row;
 #pragma unroll
       for (int j = 0; j < T::TN; ++j) {
-#pragma unroll
-        for (int q = 0; q < Q; ++q) {
-          const int nl = wn + j * MF + run_col(q);
-          const typename T::Acc& v = acc[i][j];
-          const int o = MF == 32 ? q * 4 : 0;                    // first register of the run
-          u32x2 w;
-          w[0] = pack2<DT>(v[o + 0], v[o + 1]);
-          w[1] = pack2<DT>(v[o + 2], v[o + 3]);
-          *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
-        }
+        const int nl = wn + j * MF + run_col;
+        const typename T::Acc& v = acc[i][j];
+        u32x2 w;
+        w[0] = pack2<DT>(v[0], v[1]);
+        w[1] = pack2<DT>(v[2], v[3]);
+        *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
       }
     }
     __syncthreads();
@@ -1321,7 +1072,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
                 uint16_t* __restrict__ out2, const int32_t* __restrict__ slots, const int32_t* __restrict__ src_bins,
                 int top_k, int src_rows, uint32_t top_k_magic, int top_k_shift, int half_limit) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK && T::MF == TS::MF, "tail tile");
+  static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "tail tile");
   static_assert(!(DUAL && (epi_is_dglu(EPI) || epi_is_glu(EPI))), "a2 / b2 are the second operand pair, the epilogue's x2 or the second matrix");
   constexpr int kTileCols = epi_is_glu(EPI) ? T::BN / 2 : T::BN;   // output columns of a tile
   constexpr bool kSplit = T::BM != TS::BM;
@@ -1431,7 +1182,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
     // without them).  Lane l of wave w issues load w + 4 q of the tile, which holds rows 8 (w + 4 q) + l / 8.
     static_assert(!GATHER || (T::LA >= TS::LA && T::LA <= 8 && T::BK == 64 && T::WAVES == TS::WAVES), "the row map is fetched for the taller tile");
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane_row = lane_id() >> 3;
-    const uint32_t piece = load_lane_offset<false, T::BK, T::BM, 16>(wave, 0, 0u, false);   // pitch 0: the piece inside the row
+    const uint32_t piece = load_lane_offset<false, T::BK, T::BM>(wave, 0, 0u, false);   // pitch 0: the piece inside the row
     const int64_t slots_end = (int64_t)src_rows * top_k;
     int next_slot[T::LA];
     auto fetch_slots = [&](int e, int start, int row0) {

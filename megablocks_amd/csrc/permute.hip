@@ -250,7 +250,8 @@ gather_tokens_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, in
     const int c0 = (int)(item % chunks) * 4 * kWave;
     const u32x4* src = (const u32x4*)(x + t * hidden);
     const int64_t s0 = t * top_k;
-    const int my_row = lane < top_k ? inv[s0 + lane] : -1;
+    int my_row = lane < top_k ? inv[s0 + lane] : -1;
+    my_row = my_row < out_rows ? my_row : -1;             // a map of another routing cannot take a store out of range
     const float my_scale = (weights && lane < top_k) ? load_as_f32(weights, s0 + lane, w_dtype) : 1.f;
     {
       u32x4 v[4];
@@ -284,6 +285,16 @@ gather_tokens_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, in
   zero_unowned_rows<DT>(out, out_rows, hidden, indices, bins, padded_bins, num_bins, (int)(tokens * top_k), wave_id, waves);
 }
 
+// A slot -> row map read with a bound: a row at or past `limit` reads as "no row" (-1).
+struct BoundedRows {
+  const int32_t* __restrict__ map;
+  int limit;
+  __device__ __forceinline__ int operator[](int64_t s) const {
+    const int r = map[s];
+    return r < limit ? r : -1;
+  }
+};
+
 // ------------------------------------------------------------------ combine (scatter)
 // out[t] = sum_j round(x[inv[t*k+j]] * w[t*k+j]); one wave per token.  Each product is
 // rounded to the storage type before the fp32 sum, as the reference's scaled copy into a
@@ -293,12 +304,16 @@ gather_tokens_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, in
 // one-row-at-a-time loop.
 template <int DT, bool VEC, int BATCH>
 __global__ void __launch_bounds__(kRowThreads)
-combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ inv,
-               const void* __restrict__ weights, int w_dtype, void* __restrict__ out_) {
+combine_kernel(const void* __restrict__ x_, int64_t tokens, int hidden, int top_k, const int32_t* __restrict__ inv_,
+               const void* __restrict__ weights, int w_dtype, void* __restrict__ out_,
+               const int32_t* __restrict__ row_limit_ptr, int row_limit_value) {
   typedef typename Elem<DT>::type E;
   const E* x = (const E*)x_;
   E* out = (E*)out_;
   const int lane = lane_id(), wave = threadIdx.x / kWave;
+  // Rows of x the map may name: below the last padded bin bound (read here) or a bound the host knows.  A map that does
+  // not belong to this routing (kept from another one) can then make the result wrong, never a read out of range.
+  const BoundedRows inv{inv_, row_limit_ptr ? *row_limit_ptr : row_limit_value};
   for (int64_t t = (int64_t)blockIdx.x * kRowWaves + wave; t < tokens; t += (int64_t)gridDim.x * kRowWaves) {
     E* dst = out + t * hidden;
     const int64_t s0 = t * top_k;
@@ -445,7 +460,8 @@ scatter_backward_kernel(const void* __restrict__ grad_, const void* __restrict__
   for (int64_t t = wave_id; t < tokens; t += waves) {
     const u32x4* g = (const u32x4*)(grad + t * hidden);
     const int64_t s0 = t * top_k;
-    const int my_row = lane < top_k ? inv[s0 + lane] : -1;
+    int my_row = lane < top_k ? inv[s0 + lane] : -1;
+    my_row = my_row < out_rows ? my_row : -1;             // x and dx have out_rows rows
     const float my_scale = lane < top_k ? load_as_f32(weights, s0 + lane, w_dtype) : 0.f;
     int row[BATCH];
     float scale[BATCH], acc[BATCH];
@@ -623,8 +639,10 @@ int mbx_gather(const void* x, int dtype, int64_t tokens, int hidden, int top_k, 
 // the process ends; in host code the array's name is only a handle for hipGetSymbolAddress.
 static __device__ __align__(256) int32_t g_static_slot_rows[MBX_STATIC_SCATTER_MAX_SLOTS];
 
-// Device address of g_static_slot_rows on the current device, looked up once per device.
-static int static_slot_rows(int32_t** out) {
+// Device address of g_static_slot_rows on the current device, looked up once per device (mbx_init(), or the first
+// call of mbx_scatter_static on the device).  The lookup is a runtime call that may not be made while `capturing`
+// (a stream, or null) records a graph: then MBX_ECAPTURE, and nothing has been enqueued.
+static int static_slot_rows(int32_t** out, hipStream_t capturing = nullptr, bool check_capture = false) {
   constexpr int kMaxDevices = 64;
   static std::mutex lock;
   static int32_t* address[kMaxDevices];
@@ -633,6 +651,11 @@ static int static_slot_rows(int32_t** out) {
   if (dev < 0 || dev >= kMaxDevices) return MBX_EINVAL;
   std::lock_guard<std::mutex> guard(lock);
   if (!address[dev]) {
+    if (check_capture) {
+      hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+      MBX_HIP_CHECK(hipStreamIsCapturing(capturing, &status));
+      if (status != hipStreamCaptureStatusNone) return MBX_ECAPTURE;
+    }
     void* p = nullptr;
     MBX_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_slot_rows)));
     if (!p) return MBX_EINVAL;
@@ -660,18 +683,22 @@ int mbx_slot_rows(const int32_t* indices, const int32_t* bin_ids, const int32_t*
 }
 
 // The combine launch of mbx_scatter / mbx_scatter_static: `inv` is the slot -> row map.
+// x has *limit_ptr rows (a bound on the device: the last padded bin bound), or limit_value rows if limit_ptr is null.
 static int launch_combine(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* inv,
-                          const void* weights, int w_dtype, void* out, hipStream_t s) {
+                          const void* weights, int w_dtype, void* out, const int32_t* limit_ptr, int limit_value,
+                          hipStream_t s) {
   const bool vec = can_vec(dtype, hidden, x, out);
-#define CALL(DT, V)                                                                                                             \
-  do {                                                                                                                          \
-    if (top_k == 1) combine_kernel<DT, V, 1><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
-    else if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
-    else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
-    else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
+#define CALL_B(DT, V, B) combine_kernel<DT, V, B><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out, limit_ptr, limit_value)
+#define CALL(DT, V)                            \
+  do {                                         \
+    if (top_k == 1) CALL_B(DT, V, 1);          \
+    else if (top_k <= 2) CALL_B(DT, V, 2);     \
+    else if (top_k <= 4) CALL_B(DT, V, 4);     \
+    else CALL_B(DT, V, 8);                     \
   } while (0)
   MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
 #undef CALL
+#undef CALL_B
   return launch_status();
 }
 
@@ -692,7 +719,13 @@ int mbx_scatter(const void* x, int dtype, int64_t tokens, int hidden, int top_k,
     build_slot_rows(indices, bin_ids, bins, padded_bins, num_bins, n_slots, (int32_t*)scratch, s);
     inv = (const int32_t*)scratch;
   }
-  return launch_combine(x, dtype, tokens, hidden, top_k, inv, weights, w_dtype, out, s);
+  return launch_combine(x, dtype, tokens, hidden, top_k, inv, weights, w_dtype, out,
+                        padded_bins && num_bins > 0 ? padded_bins + (num_bins - 1) : nullptr, (int)n_slots, s);
+}
+
+int mbx_init(void) {
+  int32_t* map = nullptr;
+  return static_slot_rows(&map);
 }
 
 int mbx_scatter_static(const void* x, int dtype, int64_t tokens, int hidden, int top_k, const int32_t* indices,
@@ -705,12 +738,13 @@ int mbx_scatter_static(const void* x, int dtype, int64_t tokens, int hidden, int
   const int64_t n_slots = tokens * top_k;
   if (n_slots > MBX_STATIC_SCATTER_MAX_SLOTS) return MBX_ERANGE;   // more slots than the static map holds
   int32_t* map = nullptr;
-  const int rc = static_slot_rows(&map);
-  if (rc) return rc;
   hipStream_t s = as_stream(stream);
+  const int rc = static_slot_rows(&map, s, true);
+  if (rc) return rc;
   // every entry the combine reads is rewritten here (fill, then the inverse map): nothing of the previous call is used
   build_slot_rows(indices, bin_ids, bins, padded_bins, num_bins, n_slots, map, s);
-  return launch_combine(x, dtype, tokens, hidden, top_k, map, weights, w_dtype, out, s);
+  return launch_combine(x, dtype, tokens, hidden, top_k, map, weights, w_dtype, out,
+                        padded_bins && num_bins > 0 ? padded_bins + (num_bins - 1) : nullptr, (int)n_slots, s);
 }
 
 int mbx_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int hidden, int top_k,
@@ -810,17 +844,7 @@ int mbx_binned_scatter(const void* x, int dtype, int64_t tokens, int hidden, int
   hipStream_t s = as_stream(stream);
   const int rc = binned_inverse(indices, bins, num_bins, capacity, n_slots, inv, s);
   if (rc) return rc;
-  const bool vec = can_vec(dtype, hidden, x ? x : out, out);
-#define CALL(DT, V)                                                                                                             \
-  do {                                                                                                                          \
-    if (top_k == 1) combine_kernel<DT, V, 1><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);      \
-    else if (top_k <= 2) combine_kernel<DT, V, 2><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
-    else if (top_k <= 4) combine_kernel<DT, V, 4><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out); \
-    else combine_kernel<DT, V, 8><<<row_grid(tokens), kRowThreads, 0, s>>>(x, tokens, hidden, top_k, inv, weights, w_dtype, out);                 \
-  } while (0)
-  MBX_DISPATCH_DT_VEC(dtype, vec, CALL)
-#undef CALL
-  return launch_status();
+  return launch_combine(x ? x : out, dtype, tokens, hidden, top_k, inv, weights, w_dtype, out, nullptr, (int)((int64_t)num_bins * capacity), s);
 }
 
 int mbx_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int hidden, int top_k,

@@ -214,7 +214,8 @@ route_scan_kernel(int32_t* __restrict__ table, int ndigits, int nblocks, int32_t
 // slot_rows (with IOTA, i.e. on the first pass, whose values are the key's positions in the input; NULL: not wanted):
 // also writes, for the key at input position i that lands at sorted position p, the row of the expert-major buffer
 // that holds it: p itself, or with padded_bins the row p - bins[e - 1] + padded_bins[e - 1] of expert e's padded
-// block (-1 for an expert id outside [0, num_bins)) -- the map inverse_map_kernel of the permutation kernels builds.
+// block (-1 for a key whose digit is at or past num_bins) -- the map inverse_map_kernel of the permutation kernels
+// builds.
 template <typename T, bool IOTA>
 __global__ void __launch_bounds__(kSortThreads)
 radix_scatter_kernel(const T* __restrict__ keys_in, const T* __restrict__ vals_in, int64_t n,
@@ -268,8 +269,12 @@ radix_scatter_kernel(const T* __restrict__ keys_in, const T* __restrict__ vals_i
       if (IOTA && slot_rows != nullptr) {
         int32_t row = pos;
         if (padded_bins != nullptr) {
-          const int64_t e = (int64_t)key[it];
-          if (e < 0 || e >= num_bins) row = -1;
+          // The expert of a key is its digit here, as it is for the counts the bins were made of (route_scan_kernel):
+          // an id outside [0, num_bins) is then either one more row of the expert its low bits name, counted in that
+          // expert's bins, or (digit at or past num_bins) sorted behind the last bin and in nobody's rows.  Every row
+          // of the padded buffer inside a bin so has exactly one slot or is padding.
+          const int e = (int)dig[it];
+          if (e >= num_bins) row = -1;
           else if (e > 0) row = pos - bins[e - 1] + padded_bins[e - 1];
         }
         slot_rows[i] = row;
@@ -429,6 +434,7 @@ const char* mbx_error_string(int code) {
   if (code == MBX_ESCRATCH) return "mbx: scratch buffer missing or too small";
   if (code == MBX_ERANGE) return "mbx: size out of the supported range";
   if (code == MBX_EUNSUPPORTED) return "mbx: shape or type not handled by this entry point";
+  if (code == MBX_ECAPTURE) return "mbx: first call on this device under stream capture; call mbx_init() beforehand";
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mbx: unknown error";
 }

@@ -153,5 +153,9 @@ class MoE(torch.nn.Module):
 
     def forward(self, x: torch.Tensor):
         x = common.cast_if_autocast_enabled(x)
-        scores, expert_weights, top_experts, top_experts32 = self.router.route(x)
-        return self.experts(x, scores, expert_weights, top_experts if top_experts32 is None else top_experts32)
+        # Called as a module (moe.py:468), so that hooks on the router and routers that only define forward() work.
+        # LearnedRouter hangs the int32 copy of its indices, which its kernel writes anyway, on the int64 tensor it
+        # returns; the routing takes that copy (no cast, moe.py:160) unless something has replaced or rewritten the
+        # indices on the way here.
+        scores, expert_weights, top_experts = self.router(x)
+        return self.experts(x, scores, expert_weights, router.int32_indices(top_experts))

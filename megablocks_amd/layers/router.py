@@ -150,6 +150,15 @@ class _SoftmaxTopK(torch.autograd.Function):
         return grad_logits, None, None, None
 
 
+def int32_indices(expert_indices: torch.Tensor) -> torch.Tensor:
+    """The int32 copy LearnedRouter.forward attached to its indices, if `expert_indices` still is that tensor with
+    that content; else `expert_indices` itself (the routing then casts, as moe.py:160 does)."""
+    attached = getattr(expert_indices, '_mbx_int32', None)
+    if attached is not None and attached[1] == expert_indices._version and attached[0].shape == expert_indices.shape:
+        return attached[0]
+    return expert_indices
+
+
 class LearnedRouter(torch.nn.Module):
 
     def __init__(self, args: Arguments):
@@ -171,7 +180,11 @@ class LearnedRouter(torch.nn.Module):
         return torch.topk(scores, self.args.moe_top_k, dim=-1)
 
     def forward(self, x: torch.Tensor):
-        return self.route(x)[:3]
+        scores, expert_weights, expert_indices, expert_indices32 = self.route(x)
+        if expert_indices32 is not None:
+            # out of band: the same indices as int32, valid while the int64 tensor is the one returned here, unmodified
+            expert_indices._mbx_int32 = (expert_indices32, expert_indices._version)
+        return scores, expert_weights, expert_indices
 
     def route(self, x: torch.Tensor):
         """forward's (scores, expert_weights, expert_indices) and, where the router kernel wrote them, the indices as

@@ -510,64 +510,6 @@ def test_fused_gated_activation_matches_the_two_step_formulation(dtype, act_name
     assert torch.equal(gated_activation(fn, odd, odd), fn(odd) * odd)
 
 
-_OTHER_MFMA_CHECK = r'''
-import sys, torch
-sys.path.insert(0, sys.argv[1])
-from megablocks_amd import grouped_gemm_util as gg
-torch.manual_seed(0)
-def rel(a, b):
-    return float((a.double() - b.double()).norm() / b.double().norm())
-worst = 0.0
-for dtype in (torch.bfloat16, torch.float16):
-    for groups, rows, k, n in ((8, 4096, 512, 768), (5, 1500, 320, 264), (64, 8192, 1024, 512), (3, 900, 1408, 2048)):
-        cuts = torch.sort(torch.randint(0, rows + 1, (groups - 1,)))[0]
-        sizes = torch.diff(torch.cat([torch.zeros(1, dtype=torch.int64), cuts, torch.tensor([rows])]))
-        if groups > 2:
-            sizes[2] += sizes[1]; sizes[1] = 0                      # an empty group
-        a = torch.randn(rows, k, device='cuda').to(dtype)
-        a2 = torch.randn(rows, k, device='cuda').to(dtype)
-        bn = (torch.randn(groups, k, n, device='cuda') * 0.1).to(dtype)
-        bn2 = (torch.randn(groups, k, n, device='cuda') * 0.1).to(dtype)
-        bt = bn.transpose(1, 2).contiguous()
-        g = torch.randn(rows, n, device='cuda').to(dtype)
-        bounds = torch.cumsum(sizes, 0).tolist()
-        want_nn = torch.cat([a[lo:hi].float() @ bn[e].float() for e, (lo, hi) in enumerate(zip([0] + bounds[:-1], bounds))])
-        want_dual = want_nn + torch.cat([a2[lo:hi].float() @ bn2[e].float() for e, (lo, hi) in enumerate(zip([0] + bounds[:-1], bounds))])
-        want_tn = torch.stack([a[lo:hi].float().t() @ g[lo:hi].float() for lo, hi in zip([0] + bounds[:-1], bounds)])
-        worst = max(worst, rel(gg.backend.gmm(a, bn, sizes), want_nn), rel(gg.backend.gmm(a, bt, sizes, trans_b=True), want_nn),
-                    rel(gg.backend.gmm(a, g, sizes, trans_a=True), want_tn), rel(gg.gmm_dual(a, bn, a2, bn2, sizes), want_dual))
-        assert int(torch.count_nonzero(gg.backend.gmm(a, g, sizes, trans_a=True)[1])) == 0 or groups <= 2
-        # the epilogue forms: this main loop has the GELU ones; the gated ones fall back to their separate passes
-        x2 = torch.randn(rows, n, device='cuda').to(dtype)
-        p1, act = gg.gmm_act(a, bt, sizes, fuse=True)
-        q1, act2 = gg.gmm_act(a, bt, sizes, fuse=False)
-        assert torch.equal(p1, q1)
-        worst = max(worst, rel(act.float(), act2.float()))
-        x1, xx2, h = gg.gmm_glu(a, bt, bt, sizes, 0, fuse=True)
-        y1, yy2, h2 = gg.gmm_glu(a, bt, bt, sizes, 0, fuse=False)
-        assert torch.equal(x1, y1) and torch.equal(h, h2)
-        d1, d2 = gg.gmm_dglu(a, bt, p1, x2, sizes, 0, fuse=True)
-        e1, e2 = gg.gmm_dglu(a, bt, p1, x2, sizes, 0, fuse=False)
-        assert torch.equal(d1, e1) and torch.equal(d2, e2)
-print('worst', worst)
-assert worst < 1e-2, worst
-'''
-
-
-def test_gmm_on_the_32x32x16_instruction():
-    """MBX_MFMA=32 selects the main loop built on v_mfma_f32_32x32x16 instead of the default 16x16x32 one (read once
-    per process, hence the child process): the three layouts and the two-pair product against fp32 torch, and the
-    epilogue forms against their two-step formulations (the gated ones are two-step under this main loop)."""
-    import os
-    import subprocess
-    import sys
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, MBX_MFMA='32')
-    proc = subprocess.run([sys.executable, '-c', _OTHER_MFMA_CHECK, root], env=env, capture_output=True, text=True, timeout=300)
-    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
-    assert 'worst' in proc.stdout
-
-
 EPILOGUE = [  # groups, rows, k, n -- full and half-height tiles, partial last column tile, shapes off the fused path
     (8, 4096, 1024, 4096), (64, 16384, 1024, 1024), (5, 1500, 320, 264), (3, 700, 128, 1408), (1, 37, 64, 8),
     (4, 1000, 72, 256), (16, 6000, 2048, 520), (72, 5000, 128, 264),
@@ -723,10 +665,27 @@ def test_gmm_on_rows_gathered_on_the_fly(gg, tokens, experts, top_k, k, n, block
     c, h = gg.gmm_gather(src, w1, sizes, act=gg.ACT_GELU_TANH)
     want_c, want_h = gg.gmm_act(a, w1, sizes, fuse=True)
     assert torch.equal(c, want_c) and torch.equal(h, want_h)
+    # ... and, directly, the CPU oracle's gather (kernels.py:107-170) and grouped product on the same inputs, with the
+    # activations of mlp.py:521-522 / glu.py:201-204 applied to the product as stored
+    cpu = lambda t: None if t is None else t.cpu()
+    if padded_bins is None:
+        o_a = oracle.gather(cpu(x), cpu(indices), cpu(bin_ids), None, cpu(bins), top_k)
+    else:
+        o_a = oracle.padded_gather(cpu(x), cpu(indices), cpu(bin_ids), None, cpu(bins), cpu(padded_bins), top_k)
+    assert torch.equal(a.cpu(), o_a)
+    o_x1 = oracle.gmm(o_a, cpu(w1), cpu(sizes), trans_b=True)
+    o_x2 = oracle.gmm(o_a, cpu(v1), cpu(sizes), trans_b=True)
+    gelu = lambda t: torch.nn.functional.gelu(t.float(), approximate='tanh').to(dtype)
+    silu = lambda t: torch.nn.functional.silu(t.float()).to(dtype)
+    if rows:
+        assert rel_err(c.cpu(), o_x1) < TOL and rel_err(h.cpu(), gelu(o_x1)) < TOL
     for act in (0, 1):
         x1, x2, h = gg.gmm_gather(src, w1, sizes, b2=v1, act=act)
         w_x1, w_x2, w_h = gg.gmm_glu(a, w1, v1, sizes, act, fuse=True)
         assert torch.equal(x1, w_x1) and torch.equal(x2, w_x2) and torch.equal(h, w_h)
+        if rows:
+            o_h = ((silu, gelu)[act](o_x1).float() * o_x2.float()).to(dtype)
+            assert rel_err(x1.cpu(), o_x1) < TOL and rel_err(x2.cpu(), o_x2) < TOL and rel_err(h.cpu(), o_h) < TOL
     assert bool((guard == 7.0).all())
 
 

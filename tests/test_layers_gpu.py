@@ -114,6 +114,48 @@ def test_dmoe_forward_backward_vs_oracle(syn, tokens, hidden, ffn, experts, top_
         assert rel_err(layer.router.layer.weight.grad, want_grads['router']) < 5 * tol
 
 
+@pytest.mark.parametrize('mlp_type,activation', [('mlp', 'relu'), ('glu', 'gelu_exact'), ('mlp', 'silu')])
+@pytest.mark.parametrize('mlp_impl,memopt', [('grouped', False), ('grouped', True), ('sparse', False)])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+def test_dmoe_with_an_activation_the_library_has_no_kernel_for(syn, mlp_type, activation, mlp_impl, memopt, dtype):
+    """`activation_fn` is the user's (arguments.py:30): anything but SiLU for the gated experts or tanh-GELU takes
+    torch's own forward and autograd (mlp.py:478-483 "else autograd", glu.py:120-124) around the library's grouped
+    products.  Forward and every gradient against the oracle with the same callable."""
+    import torch.nn.functional as F
+    fn = {'relu': F.relu, 'gelu_exact': F.gelu, 'silu': F.silu}[activation]
+    w = syn.Workload('t', 700, 128, 384, 4, 2, mlp_type, mlp_impl, dtype, 'logits')
+    inp = syn.make_inputs(w, seed=11)
+    if dtype != torch.float32:
+        for k in ('x', 'grad', 'w1', 'w2', 'v1', 'expert_weights'):
+            if inp[k] is not None:
+                inp[k] = inp[k].to(dtype).float()
+    leaves = {k: inp[k].clone().requires_grad_(True) for k in ('x', 'w1', 'w2', 'expert_weights')}
+    v1 = None if inp['v1'] is None else inp['v1'].clone().requires_grad_(True)
+    want, _ = oracle.dmoe_forward(leaves['x'], leaves['expert_weights'], inp['top_experts'], leaves['w1'], leaves['w2'], v1,
+                                  num_experts=w.experts, top_k=w.top_k, activation=fn)
+    want.backward(inp['grad'])
+    layer = syn.build_layer(w, inp, memory_optimized=memopt)
+    layer.experts.mlp.args.activation_fn = fn
+    x = inp['x'].to(dtype).cuda().requires_grad_(True)
+    ew = inp['expert_weights'].to(dtype).cuda().requires_grad_(True)
+    from megablocks_amd import _lib
+    _lib.profile_hook = []
+    try:
+        out = syn.layer_step(layer, w, x, inp['grad'].to(dtype).cuda(), (inp['scores'].to(dtype).cuda(), ew, inp['top_experts'].cuda()))
+        torch.cuda.synchronize()
+        launched = {name for name, *_ in _lib.profile_hook}
+    finally:
+        _lib.profile_hook = None
+    assert not launched & {'gmm_nt_act', 'gmm_nt_dact', 'gmm_nt_glu', 'gmm_nt_dglu'}   # no epilogue was mistaken for it
+    tol = 1e-4 if dtype == torch.float32 else 1e-2
+    assert rel_err(out, want.detach()) < tol and rel_err(x.grad, leaves['x'].grad) < tol
+    mlp = layer.experts.mlp
+    assert rel_err(mlp.w1.grad, leaves['w1'].grad) < tol and rel_err(mlp.w2.grad, leaves['w2'].grad) < tol
+    if v1 is not None:
+        assert rel_err(mlp.v1.grad, v1.grad) < tol
+    assert rel_err(ew.grad, leaves['expert_weights'].grad) < tol
+
+
 @pytest.mark.parametrize('mlp_impl,memopt', [('grouped', False), ('grouped', True), ('sparse', False), ('sparse', True)])
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 def test_dmoe_mlp_with_activation_epilogues_vs_oracle(syn, monkeypatch, mlp_impl, memopt, dtype):
@@ -907,6 +949,10 @@ def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, m
     from megablocks_amd import grouped_gemm_util as gg
     w = syn.Workload('t', 1500, 256, 768, 8, 2, mlp_type, mlp_impl, dtype, 'logits')
     inp = syn.make_inputs(w, seed=9)
+    for k in ('x', 'grad', 'w1', 'v1', 'w2', 'expert_weights'):
+        if inp[k] is not None:
+            inp[k] = inp[k].to(dtype).float()
+    oracle_out, _, oracle_grads, _ = _oracle_step(w, inp, True)
     layer = syn.build_layer(w, inp)
     routing = lambda ew: (inp['scores'].to(dtype).cuda(), ew, inp['top_experts'].cuda())
     grad = inp['grad'].to(dtype).cuda()
@@ -936,6 +982,7 @@ def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, m
     assert 'gather' in launched
     got, _, launched = step('auto', False)
     assert torch.equal(got, want) and 'gather' not in launched
+    assert rel_err(got, oracle_out) < 1e-2                                    # the fused forward against the CPU oracle
     want, want_grads, launched = step('auto', True)                           # gradients recorded: not fused by default
     assert launched.count('gather') == 1 and launched.index('gather') < launched.index(first)
     got, got_grads, launched = step('1', True)
@@ -944,6 +991,11 @@ def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, m
     assert len(got_grads) == len(want_grads) >= 4
     for g, wg in zip(got_grads, want_grads):
         assert torch.equal(g, wg)
+    # ... and the fused step against the oracle's forward and autograd
+    assert rel_err(got, oracle_out) < 1e-2
+    names = ['x', 'expert_weights', 'w1'] + (['v1'] if mlp_type == 'glu' else []) + ['w2']
+    for name, g in zip(names, got_grads):
+        assert rel_err(g, oracle_grads[name]) < 1e-2, name
 
 
 @pytest.mark.parametrize('mlp_type,tokens,hs,ffn,ne,top_k', [('mlp', 2048, 1024, 1024, 64, 1), ('glu', 1024, 512, 1408, 8, 2)])
@@ -1015,3 +1067,59 @@ def test_memory_optimized_dmoe_forward_without_gradients_gathers_in_the_first_pr
         finally:
             _lib.profile_hook = None
     assert torch.equal(got, want) and 'gather' not in launched
+
+
+def test_router_is_called_as_a_module(syn):
+    """moe.py:468 calls `self.router(x)`: forward hooks on the router run, a hook may replace the routing, and a router
+    that only defines forward() works.  The int32 indices the built-in router passes out of band are used only while
+    the int64 tensor it returned is what arrives, unmodified."""
+    from megablocks_amd.layers import router as router_mod
+    w = syn.Workload('t', 512, 128, 256, 8, 2, 'mlp', 'grouped', torch.bfloat16, 'router', normalize=1)
+    inp = syn.make_inputs(w, seed=13)
+    layer = syn.build_layer(w, inp)
+    x = inp['x'].bfloat16().cuda().view(w.tokens, 1, w.hidden)
+    with torch.no_grad():
+        base = layer(x)
+        scores, weights, indices = layer.router(x)
+        assert router_mod.int32_indices(indices).dtype == torch.int32
+        assert torch.equal(router_mod.int32_indices(indices).long(), indices)
+        seen = []
+        handle = layer.router.register_forward_hook(lambda mod, args, out: seen.append(out[2].shape))
+        assert torch.equal(layer(x), base) and seen == [indices.shape]
+        handle.remove()
+        # a hook that reroutes every token to experts (0, 1): the layer must follow the hook, not the stale int32 copy
+        def reroute(mod, args, out):
+            s, wgt, idx = out
+            new = torch.zeros_like(idx)
+            new[:, 1] = 1
+            return s, wgt, new
+        handle = layer.router.register_forward_hook(reroute)
+        rerouted = layer(x)
+        handle.remove()
+        tpe_hooked = []
+        orig = layer.experts.forward_fn
+        def spy(xx, ew, te):
+            out, tpe = orig(xx, ew, te)
+            tpe_hooked.append(tpe.cpu())
+            return out, tpe
+        layer.experts.forward_fn = spy
+        handle = layer.router.register_forward_hook(reroute)
+        assert torch.equal(layer(x), rerouted)
+        handle.remove()
+        layer.experts.forward_fn = orig
+        assert tpe_hooked[0].tolist() == [w.tokens, w.tokens] + [0] * (w.experts - 2)
+        # in-place modification of the returned indices invalidates the attached copy
+        scores, weights, indices = layer.router(x)
+        indices.zero_()
+        assert router_mod.int32_indices(indices) is indices
+
+        class ForwardOnlyRouter(torch.nn.Module):
+            def __init__(self, inner):
+                super().__init__()
+                self.layer = inner.layer
+                self.inner = inner
+            def forward(self, xx):
+                s, wgt, idx = self.inner(xx)
+                return s, wgt, idx.clone()
+        layer.router = ForwardOnlyRouter(layer.router)
+        assert torch.equal(layer(x), base)

@@ -526,3 +526,22 @@ def test_route_with_ids_outside_the_experts_stays_in_range(blocking):
     rows = indices._mbx_slot_rows[1][:n].cpu()
     limit = int(pbins[-1]) if blocking else n
     assert int(rows.min()) >= -1 and int(rows.max()) < max(limit, n)
+    # order, counts and row map agree on the expert of such an id (its low bits): the bins cover the sorted order up to
+    # the ids whose low bits name no expert, and every row inside a bin has exactly one slot or is padding, so a gather
+    # through this routing leaves no row of the expert-major buffer unwritten
+    low = (top & ((1 << end_bit) - 1)).long()
+    assert torch.equal(tpe.cpu().long(), torch.bincount(low[low < experts], minlength=experts))
+    owned = rows[rows >= 0]
+    assert owned.unique().numel() == owned.numel() and owned.numel() == int((low < experts).sum()) + (0 if blocking else int((low >= experts).sum()))
+    poison = torch.full((max(limit, n), 64), float('nan'), dtype=torch.bfloat16, device='cuda')
+    del poison                                            # the gather's output is likely to land on this block
+    for top_k in (2, 1):                                  # one wave per token with the row map / one wave per output row
+        x = torch.randn(n // top_k, 64, generator=g).bfloat16().cuda()
+        if blocking:
+            out = ops.padded_gather(x, indices, bin_ids, bins, pbins, top_k)
+        else:
+            out = ops.gather(x, indices, bin_ids, bins, top_k)
+        assert not bool(torch.isnan(out.float()).any())
+        want = torch.zeros_like(out)
+        want[owned.cuda().long()] = x[((rows >= 0).nonzero().flatten() // top_k).cuda()]
+        assert torch.equal(out, want)
