@@ -223,6 +223,20 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
                  const int32_t* bins, int num_groups, int64_t rows, int k, int n, int layout,
                  mbx_stream_t stream);
 
+/* mbx_gmm (a2 == b2 == NULL) / mbx_gmm_dual with a workspace: device memory the launch may use to cut the tiles of its
+ * last, partly filled round of workgroups along the reduction (MBX_NN with long reductions: a Mixtral-shaped second
+ * product has 4.25 rounds of tiles on 256 compute units, and the quarter round costs as much as a whole one).  Parts
+ * of a tile are summed in a fixed order: results do not change from run to run, but differ in the last bits from
+ * those of a launch without workspace.  grouped_gemm.backend.gmm allocates what it needs through torch; this library
+ * allocates nothing, so the caller lends the memory:
+ *   workspace: mbx_gmm_workspace_bytes() bytes, 16-byte aligned (less: fewer tiles are cut; NULL: none are), whose
+ *   first 4096 bytes are zero before the first launch that uses it.  Every launch leaves them zero again.  Launches
+ *   that may run at the same time (different streams) need workspaces of their own. */
+size_t mbx_gmm_workspace_bytes(void);
+int mbx_gmm_ws(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype, const int32_t* bins,
+               int num_groups, int64_t rows, int k, int n, int layout, void* workspace, size_t workspace_bytes,
+               mbx_stream_t stream);
+
 /* The first product of the expert MLP with its activation, megablocks/layers/mlp.py:521-522 / 414-416
  * (`x = gmm(x, w1, batch_sizes, trans_b=True); x = activation_fn(x)`), in one launch:
  *   c[r_e] = a[r_e] @ b[e]^T (b is [E, n, k]),   c_act = act(c)

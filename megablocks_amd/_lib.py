@@ -44,6 +44,8 @@ _SIGNATURES = {
     'mbx_binned_scatter_wgrad': (_i, [_vp, _vp, _i, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _vp]),
     'mbx_gmm': (_i, [_vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_dual': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
+    'mbx_gmm_workspace_bytes': (_sz, []),
+    'mbx_gmm_ws': (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp, _sz, _vp]),
     'mbx_gmm_act': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_dact': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_glu': (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),

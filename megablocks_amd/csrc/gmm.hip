@@ -564,6 +564,13 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
 // a2 / b2 non-null (NN / NT only): c = a @ b[e] + a2 @ b2[e], the second pair shaped like the first.
 // epi / extra (NT, one operand pair only): dma::kEpiAct with the second output, dma::kEpiDact with the second input.
 // Rows of `a` gathered on the fly (NT; no epilogue, kEpiAct or kEpiGlu*): see GatherRows.
+// Device memory a launch may use for the parts of tiles it cuts along the reduction (gmm_rows_kernel's split-K tail):
+// kWorkspaceCounters int32 counters, zero before the launch and zero again after it, then room for fp32 tiles.
+constexpr size_t kWorkspaceCounters = 1024, kWorkspacePartBytes = (size_t)256 * 256 * 4, kWorkspaceParts = 320;
+struct Workspace {
+  void* base = nullptr;
+  size_t bytes = 0;
+};
 struct GatherRows {
   const int32_t* slots = nullptr;      // non-null: a is [src_rows, k], read through the row map
   const int32_t* src_bins = nullptr;
@@ -572,7 +579,7 @@ struct GatherRows {
 template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
             int layout, hipStream_t s, const void* a2 = nullptr, const void* b2 = nullptr, int epi = dma::kEpiNone,
-            void* extra = nullptr, void* out2 = nullptr, GatherRows gather = GatherRows()) {
+            void* extra = nullptr, void* out2 = nullptr, GatherRows gather = GatherRows(), Workspace ws = Workspace()) {
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
   const uint16_t* ap2 = (const uint16_t*)a2;
@@ -629,13 +636,25 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
   uint32_t gather_magic = 0;
   int gather_shift = 0;
   if (gather.slots) dma::gather_divisor(gather.top_k, gather_magic, gather_shift);
+  // the workspace as the kernel takes it: counters, parts (16-byte aligned), how many parts of a T tile fit
+  int32_t* ws_counters = nullptr;
+  float* ws_parts = nullptr;
+  int ws_capacity = 0;
+  if (ws.base && ((uintptr_t)ws.base & 15u) == 0 && ws.bytes > kWorkspaceCounters * sizeof(int32_t) && (int)grid / 2 <= (int)kWorkspaceCounters) {
+    ws_counters = (int32_t*)ws.base;
+    ws_parts = (float*)((char*)ws.base + kWorkspaceCounters * sizeof(int32_t));
+    const size_t fit = (ws.bytes - kWorkspaceCounters * sizeof(int32_t)) / ((size_t)T::BM * T::BN * sizeof(float));
+    ws_capacity = (int)(fit > 0x7fffffff ? 0x7fffffff : fit);
+    if (ws_capacity < 2) ws_parts = nullptr;
+  }
 #define MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, GATHER)                                                    \
   do {                                                                                                \
     auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL, EPI, GATHER>;                             \
     int rc = allow_lds(kern, lds);                                                                    \
     if (rc) return rc;                                                                                \
     kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2,  \
-                                       gather.slots, gather.src_bins, gather.top_k, gather.src_rows, gather_magic, gather_shift, half_limit);  \
+                                       gather.slots, gather.src_bins, gather.top_k, gather.src_rows, gather_magic, gather_shift, half_limit,  \
+                                       ws_counters, ws_parts, ws_capacity);                           \
   } while (0)
 #define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI) MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, false)
   if (gather.slots) {
@@ -719,8 +738,13 @@ using namespace mbx;
 
 extern "C" {
 
-int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bins, int num_groups, int64_t rows, int k,
-            int n, int layout, mbx_stream_t stream) {
+size_t mbx_gmm_workspace_bytes(void) { return kWorkspaceCounters * sizeof(int32_t) + kWorkspaceParts * kWorkspacePartBytes; }
+
+static int gmm_dual_ws(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype, const int32_t* bins,
+                       int num_groups, int64_t rows, int k, int n, int layout, Workspace ws, mbx_stream_t stream);
+
+static int gmm_ws(const void* a, const void* b, void* c, int dtype, const int32_t* bins, int num_groups, int64_t rows, int k,
+                  int n, int layout, Workspace ws, mbx_stream_t stream) {
   if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
   if (layout != MBX_NN && layout != MBX_NT && layout != MBX_TN) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
@@ -748,12 +772,13 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
     if (dma_ok) {
       // TN: the half-height tile only when the product has at most 128 rows (it is slower otherwise)
       const bool small_m = layout == MBX_TN ? k <= TileDmaSmallM::BM : half_height_only(rows, num_groups, n);
+      const GatherRows none;
       if (small_m) {
-        if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-        return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+        if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, nullptr, nullptr, dma::kEpiNone, nullptr, nullptr, none, ws);
+        return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, nullptr, nullptr, dma::kEpiNone, nullptr, nullptr, none, ws);
       }
-      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
-      return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s);
+      if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, nullptr, nullptr, dma::kEpiNone, nullptr, nullptr, none, ws);
+      return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, nullptr, nullptr, dma::kEpiNone, nullptr, nullptr, none, ws);
     }
     if (dtype == MBX_BF16) return gmm_mfma<MBX_BF16, TileBig>(a, b, c, bins, num_groups, rows, k, n, layout, s);
     return gmm_mfma<MBX_F16, TileBig>(a, b, c, bins, num_groups, rows, k, n, layout, s);
@@ -765,8 +790,29 @@ int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bin
   }
 }
 
+int mbx_gmm(const void* a, const void* b, void* c, int dtype, const int32_t* bins, int num_groups, int64_t rows, int k,
+            int n, int layout, mbx_stream_t stream) {
+  return gmm_ws(a, b, c, dtype, bins, num_groups, rows, k, n, layout, Workspace(), stream);
+}
+
 int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype, const int32_t* bins,
                  int num_groups, int64_t rows, int k, int n, int layout, mbx_stream_t stream) {
+  return gmm_dual_ws(a, b, a2, b2, c, dtype, bins, num_groups, rows, k, n, layout, Workspace(), stream);
+}
+
+int mbx_gmm_ws(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype, const int32_t* bins,
+               int num_groups, int64_t rows, int k, int n, int layout, void* workspace, size_t workspace_bytes,
+               mbx_stream_t stream) {
+  if ((a2 == nullptr) != (b2 == nullptr)) return MBX_EINVAL;
+  Workspace ws;
+  ws.base = workspace;
+  ws.bytes = workspace ? workspace_bytes : 0;
+  if (a2) return gmm_dual_ws(a, b, a2, b2, c, dtype, bins, num_groups, rows, k, n, layout, ws, stream);
+  return gmm_ws(a, b, c, dtype, bins, num_groups, rows, k, n, layout, ws, stream);
+}
+
+static int gmm_dual_ws(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype, const int32_t* bins,
+                       int num_groups, int64_t rows, int k, int n, int layout, Workspace ws, mbx_stream_t stream) {
   if (num_groups < 0 || rows < 0 || k < 0 || n < 0) return MBX_EINVAL;
   if (layout != MBX_NN && layout != MBX_NT) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
@@ -779,12 +825,13 @@ int mbx_gmm_dual(const void* a, const void* b, const void* a2, const void* b2, v
   if (!ok) return MBX_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   const bool small_m = half_height_only(rows, num_groups, n);
+  const GatherRows none;
   if (small_m) {
-    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
-    return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2, dma::kEpiNone, nullptr, nullptr, none, ws);
+    return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2, dma::kEpiNone, nullptr, nullptr, none, ws);
   }
-  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
-  return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2);
+  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2, dma::kEpiNone, nullptr, nullptr, none, ws);
+  return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, layout, s, a2, b2, dma::kEpiNone, nullptr, nullptr, none, ws);
 }
 
 // The NT product with an activation epilogue (epi: dma::kEpiAct / dma::kEpiDact), for the shapes the direct-to-LDS

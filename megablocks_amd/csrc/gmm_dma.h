@@ -677,7 +677,22 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 // second input of kEpiDact, x1 of kEpiDglu*; `pre2` and `out2` (kEpiDglu* only, laid out alike): x2 and the second
 // output (c gets round(g x2) act'(x1), out2 gets g round(act(x1))).  These take the staged path only (the launch
 // checks pitch and alignment).
-template <int DT, typename T, int EPI = kEpiNone>
+// STAGED: the caller has already put the rounded tile into the staging area (stage_product_tile() for every product
+// tile, after a barrier of its own); acc is not read.
+template <int DT, typename T>
+__device__ __forceinline__ void stage_product_tile(char* lds_generic, int i, int j, const f32x4& v) {
+  const lds_ptr lds = (lds_ptr)lds_generic;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
+  const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
+  constexpr int ROW = T::BN * 2 + 16;
+  const int ml = wm + i * T::MF + (lane & 15), nl = wn + j * T::MF + (lane >> 4) * 4;
+  u32x2 w;
+  w[0] = pack2<DT>(v[0], v[1]);
+  w[1] = pack2<DT>(v[2], v[3]);
+  *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
+}
+
+template <int DT, typename T, int EPI = kEpiNone, bool STAGED = false>
 __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][T::TN], uint16_t* __restrict__ c, int64_t ldc,
                                             int m_base, int m_lim, int n_base, int n_lim, char* lds_generic,
                                             uint16_t* __restrict__ extra = nullptr, const uint16_t* __restrict__ pre2 = nullptr,
@@ -694,19 +709,21 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
   {
     // Staged through LDS (free by now) so that every global store instruction writes whole rows of the
     // tile: 64 lanes x 16 bytes = two 512-byte row segments, instead of 32 scattered 16-byte pieces.
-    __syncthreads();
     constexpr int ROW = T::BN * 2 + 16;   // bytes; the 16-byte pad spreads the rows of a column over the banks
+    if constexpr (!STAGED) {
+      __syncthreads();
 #pragma unroll
-    for (int i = 0; i < T::TM; ++i) {
-      const int ml = wm + i * MF + tile_row;
+      for (int i = 0; i < T::TM; ++i) {
+        const int ml = wm + i * MF + tile_row;
 #pragma unroll
-      for (int j = 0; j < T::TN; ++j) {
-        const int nl = wn + j * MF + run_col;
-        const typename T::Acc& v = acc[i][j];
-        u32x2 w;
-        w[0] = pack2<DT>(v[0], v[1]);
-        w[1] = pack2<DT>(v[2], v[3]);
-        *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
+        for (int j = 0; j < T::TN; ++j) {
+          const int nl = wn + j * MF + run_col;
+          const typename T::Acc& v = acc[i][j];
+          u32x2 w;
+          w[0] = pack2<DT>(v[0], v[1]);
+          w[1] = pack2<DT>(v[2], v[3]);
+          *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
+        }
       }
     }
     __syncthreads();
@@ -1070,7 +1087,8 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
                 const int32_t* __restrict__ bins, int num_groups, int64_t rows, int k, int n, int tiles_n,
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra,
                 uint16_t* __restrict__ out2, const int32_t* __restrict__ slots, const int32_t* __restrict__ src_bins,
-                int top_k, int src_rows, uint32_t top_k_magic, int top_k_shift, int half_limit) {
+                int top_k, int src_rows, uint32_t top_k_magic, int top_k_shift, int half_limit,
+                int32_t* __restrict__ ws_counters, float* ws_parts, int ws_capacity) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "tail tile");
   static_assert(!(DUAL && (epi_is_dglu(EPI) || epi_is_glu(EPI))), "a2 / b2 are the second operand pair, the epilogue's x2 or the second matrix");
@@ -1082,17 +1100,46 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
   const RowTiles<T::BM> tiles(bins, num_groups, tiles_n, (int)rows, kSplit && B_MC, 8);
   const int total = tiles.total;
   const int full_rounds = total / P, rest = total - full_rounds * P;
-  const bool split = kSplit && rest > 0 && 2 * rest <= P;
-  const int big_rounds = full_rounds + ((rest > 0 && !split) ? 1 : 0);
 
   Args g;
   g.a_ld_bytes = (uint32_t)k * 2;
   g.b_ld_bytes = (uint32_t)(B_MC ? n : k) * 2;
-  g.nk1 = k / T::BK;
-  g.nk = DUAL ? 2 * g.nk1 : g.nk1;
+  const int nk1 = k / T::BK, nk_all = DUAL ? 2 * nk1 : nk1;
+  g.nk1 = nk1;
+  g.nk = nk_all;
   g.a_r0 = 0;   // the buffers of a and c start at the tile's first row: byte offsets stay small whatever the row count
-  // Work items of this workgroup: one tile per round, then (if the tail is split) one half tile.
-  const int items = big_rounds + ((kSplit && split) ? 1 : 0);
+  // The last, partly filled round.  Its `rest` tiles leave P - rest compute units idle for a whole tile's time, which
+  // with long reductions and few rounds is a large part of the launch (a Mixtral-shaped second product: 1088 tiles on
+  // 256 compute units, 4.25 rounds).  When at most half of the compute units would be busy:
+  //   * with a workspace (kSplitK launches: NN, no epilogue): every tail tile is cut along the reduction into
+  //     `ksplit` = P / rest parts, one per workgroup, each a full-size tile over a `ksplit`-th of the K tiles.  A part
+  //     writes its fp32 accumulators to the workspace and counts itself in; the workgroup that finds it was the last
+  //     adds the parts up in part order (so the sum does not depend on who was last), rounds and stores the tile.
+  //     Nobody waits for anybody.  The tail then takes 1 / ksplit of a round plus the reduction;
+  //   * else the tail's tiles are cut into two half-height tiles each (TS), which take 0.7 of a full tile's time.
+  constexpr bool kSplitK = B_MC && EPI == kEpiNone && !GATHER;
+  constexpr int kMaxKSplit = 8, kMinPartTiles = 8;
+  int ksplit = 1;
+  if constexpr (kSplitK) {
+    if (ws_parts != nullptr && rest > 0 && 2 * rest <= P) {
+      int s_ = P / rest;
+      s_ = s_ > kMaxKSplit ? kMaxKSplit : s_;
+      s_ = s_ > nk_all / kMinPartTiles ? nk_all / kMinPartTiles : s_;
+      s_ = (int64_t)s_ * rest > ws_capacity ? ws_capacity / rest : s_;
+      ksplit = s_ < 2 ? 1 : s_;
+    }
+  }
+  const bool split = ksplit == 1 && kSplit && rest > 0 && 2 * rest <= P;
+  const int big_rounds = full_rounds + ((rest > 0 && !split && ksplit == 1) ? 1 : 0);
+  // Work items of this workgroup: one tile per round, then (if the tail is cut) one part or one half tile.
+  const int items = big_rounds + ((ksplit > 1 || (kSplit && split)) ? 1 : 0);
+  // first K tile of part p of a reduction cut into ksplit parts; with two operand pairs a cut within SB K tiles of the
+  // pairs' boundary moves onto it (the main loop changes pairs at least SB + 1 K tiles into a call)
+  auto part_begin = [&](int p_) -> int {
+    int t_ = (int)((int64_t)p_ * nk_all / ksplit);
+    if (DUAL && t_ - nk1 < T::SB + 1 && nk1 - t_ < T::SB + 1) t_ = nk1;
+    return t_;
+  };
   // the tile with first row row0 of expert e (rows start .. end - 1), column tile tn
   auto compute_tile = [&](int e, int end, int tn, int row0, bool use_ts) {
     const uint32_t a_bytes = clip_bytes((rows - row0) * k * 2);   // rows past the tile's are fetched, never stored
@@ -1145,6 +1192,94 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
       if (r < big_rounds) {
         id = (r * kXcds + xcd) * run + (member + r) % run;   // as in locate()
         if (id >= total) break;
+      } else if (kSplitK && ksplit > 1) {
+        if constexpr (kSplitK) {
+          // part `part` of tail tile `tile`: consecutive workgroups of an XCD take the same part of consecutive tiles
+          const int j = xcd * run + member;
+          if (j >= ksplit * rest) break;
+          const int tile = j % rest, part = j / rest;
+          int e, start, end, tm, tn;
+          tiles.find(full_rounds * P + tile, e, start, end, tm, tn);
+          const int row0 = start + tm * T::BM;
+          const int t0 = part_begin(part), t1 = part + 1 < ksplit ? part_begin(part + 1) : nk_all;
+          // the operands from K tile t0 on: of the second pair when the part lies in it, with the change of pairs at
+          // its place when the part straddles it, never otherwise
+          const bool second = DUAL && t0 >= nk1;
+          const int kt0 = second ? t0 - nk1 : t0;                      // first K tile inside its pair
+          const uint16_t* const pa = (second ? a2 : a) + (int64_t)row0 * k + (int64_t)kt0 * T::BK;
+          const uint16_t* const pb = (second ? b2 : b) + (int64_t)e * k * n + (int64_t)kt0 * T::BK * n;
+          const int64_t a_left = (rows - row0) * k - (int64_t)kt0 * T::BK, b_left = ((int64_t)k - (int64_t)kt0 * T::BK) * n;
+          g.rsrc_a = make_rsrc(pa, clip_bytes(a_left * 2));
+          g.rsrc_b = make_rsrc(pb, clip_bytes(b_left * 2));
+          g.rsrc_a2 = DUAL ? make_rsrc(a2 + (int64_t)row0 * k, clip_bytes((rows - row0) * k * 2)) : g.rsrc_a;
+          g.rsrc_b2 = DUAL ? make_rsrc(b2 + (int64_t)e * k * n, (uint32_t)((int64_t)k * n * 2)) : g.rsrc_b;
+          g.nk = t1 - t0;
+          g.nk1 = DUAL && !second && t1 > nk1 ? nk1 - t0 : 0x3fffffff;
+          g.b_r0 = tn * kTileCols;
+          typename T::Acc acc[T::TM][T::TN];
+          block_multiply<DT, false, B_MC, T, DUAL>(g, acc, true, lds);
+          g.nk = nk_all;
+          g.nk1 = nk1;
+          // The part's accumulators as they lie in the registers: 16 bytes per lane and product tile, addressed as a
+          // buffer with the lane's offset in a register and the product tile's in a scalar (64-bit addresses per
+          // store would take two registers each, which this kernel does not have).  Eight tiles at a time, so that the
+          // compiler does not gather all 256 registers of a part in one place.
+          constexpr uint32_t kPartBytes = (uint32_t)T::BM * T::BN * 4, kTileStep = (uint32_t)T::THREADS * 16;
+          const uint32_t lane_off = threadIdx.x * 16u;
+          const __amdgpu_buffer_rsrc_t mine = make_rsrc((const char*)ws_parts + (size_t)j * kPartBytes, kPartBytes);
+          static_for<T::TM>([&](auto ii) {
+            constexpr int i = decltype(ii)::value;
+#pragma unroll
+            for (int jj = 0; jj < T::TN; ++jj)
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][jj]), mine, (int)lane_off, (int)((i * T::TN + jj) * kTileStep), 0);
+            __builtin_amdgcn_sched_barrier(0);
+          });
+          __threadfence();                       // the part is visible to the whole device before it is counted
+          __syncthreads();                       // ... every wave's share of it; and nobody reads the LDS stages any more
+          int* const flag = (int*)lds;
+          if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(ws_counters + tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+          __syncthreads();
+          const bool last = *flag == ksplit - 1;  // uniform
+          if (last) {
+            __threadfence();                     // the other parts as their workgroups published them
+            // The sum of the parts, in part order whoever came last, goes straight to the staging area of the store:
+            // one row of product tiles at a time, the parts of up to four workgroups in flight together.
+            static_for<T::TM>([&](auto ii) {
+              constexpr int i = decltype(ii)::value;
+              f32x4 sum[T::TN];
+#pragma unroll 1
+              for (int p0 = 0; p0 < ksplit; p0 += 4) {
+                u32x4 v[4][T::TN];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                  if (p0 + u < ksplit) {
+                    const __amdgpu_buffer_rsrc_t theirs = make_rsrc((const char*)ws_parts + ((size_t)(p0 + u) * rest + tile) * kPartBytes, kPartBytes);
+#pragma unroll
+                    for (int jj = 0; jj < T::TN; ++jj)
+                      v[u][jj] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(theirs, (int)lane_off, (int)((i * T::TN + jj) * kTileStep), 0));
+                  }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                  if (p0 + u < ksplit) {
+#pragma unroll
+                    for (int jj = 0; jj < T::TN; ++jj) {
+                      const f32x4 w = __builtin_bit_cast(f32x4, v[u][jj]);
+                      sum[jj] = (p0 == 0 && u == 0) ? w : sum[jj] + w;
+                    }
+                  }
+                }
+              }
+#pragma unroll
+              for (int jj = 0; jj < T::TN; ++jj) stage_product_tile<DT, T>(lds, i, jj, sum[jj]);
+              __builtin_amdgcn_sched_barrier(0);
+            });
+            if (threadIdx.x == 0) ws_counters[tile] = 0;   // as the launch found it
+            block_store<DT, T, kEpiNone, true>(acc, c + (int64_t)row0 * n, n, 0, end - row0, g.b_r0, n, lds);
+          }
+          tile_done();
+        }
+        continue;
       } else {
         const int j = xcd * run + member;
         if (j >= 2 * rest) break;

@@ -80,6 +80,29 @@ def note_bins(batch_sizes: torch.Tensor, bins: torch.Tensor):
         _remember(batch_sizes, (bins.view(-1), batch_sizes._version, None))
 
 
+# Device memory the NN products lend the library for the parts of the tiles of their last round of workgroups
+# (`mbx_gmm_ws`): one buffer per device and stream, made at the first product on that stream and kept.  Launches on
+# one stream run one after the other, so they can share it; launches on different streams may overlap, so they do not.
+# A stream that is being captured gets its buffer from the capture's memory pool like any tensor made during a capture
+# (its zero-fill is a kernel of the graph; the buffer stays with this module, so later captures on a stream with the
+# same handle reuse it).  MBX_GMM_WORKSPACE=0: none (every tile is computed by one workgroup; results differ in the
+# last bits).
+GMM_WORKSPACE = os.environ.get('MBX_GMM_WORKSPACE', '1') != '0'
+_workspaces = {}
+
+
+def _workspace(device):
+    """(pointer, bytes) of the current stream's workspace on `device`; (None, 0) if switched off."""
+    if not GMM_WORKSPACE:
+        return None, 0
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _lib.stream().value)
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(lib.mbx_gmm_workspace_bytes(), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return _lib.ptr(ws), ws.numel()
+
+
 def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None, _record_as=None):
     """out[r_e] = a[r_e] @ b[e] (`trans_b`: @ b[e].T); `trans_a`: out[e] = a[r_e].T @ b[r_e].
 
@@ -124,8 +147,9 @@ def gmm(a, b, batch_sizes, trans_a=False, trans_b=False, c=None, _record_as=None
             raise ValueError('gmm: c has the wrong shape, dtype or layout')
     with _lib.device_of(a), _lib.record(_record_as or ('gmm_nn', 'gmm_nt', 'gmm_tn')[layout], rows=rows, k=k, n=n,
                                               elem=a.element_size(), groups=groups):
-        _lib.check(lib.mbx_gmm(_lib.ptr(a), _lib.ptr(b), _lib.ptr(c), dt, _lib.ptr(bins), groups, rows, k, n, layout,
-                               _lib.stream()), 'gmm')
+        ws, ws_bytes = _workspace(a.device) if layout == _lib.NN else (None, 0)
+        _lib.check(lib.mbx_gmm_ws(_lib.ptr(a), _lib.ptr(b), None, None, _lib.ptr(c), dt, _lib.ptr(bins), groups, rows, k, n,
+                                  layout, ws, ws_bytes, _lib.stream()), 'gmm')
     return c
 
 
@@ -150,8 +174,9 @@ def gmm_dual(a, b, a2, b2, batch_sizes, trans_b=False, c=None):
         raise ValueError('gmm_dual: c has the wrong shape, dtype or layout')
     with _lib.device_of(a), _lib.record('gmm_nt_dual' if trans_b else 'gmm_nn_dual', rows=rows, k=2 * k, n=n,
                                               elem=a.element_size(), groups=groups) as rec:
-        rc = lib.mbx_gmm_dual(_lib.ptr(a), _lib.ptr(b), _lib.ptr(a2), _lib.ptr(b2), _lib.ptr(c), _lib.dtype_of(a),
-                              _lib.ptr(bins), groups, rows, k, n, layout, _lib.stream())
+        ws, ws_bytes = _workspace(a.device) if layout == _lib.NN else (None, 0)
+        rc = lib.mbx_gmm_ws(_lib.ptr(a), _lib.ptr(b), _lib.ptr(a2), _lib.ptr(b2), _lib.ptr(c), _lib.dtype_of(a),
+                            _lib.ptr(bins), groups, rows, k, n, layout, ws, ws_bytes, _lib.stream())
         if rc == _lib.EUNSUPPORTED:
             rec.cancel()
     if rc == _lib.EUNSUPPORTED:

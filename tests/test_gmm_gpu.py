@@ -292,6 +292,67 @@ def test_gmm_tile_schedules(gg, name, groups, rows, k, n):
         assert torch.equal(again, got)                              # same schedule, same summation order: bit-identical
 
 
+SPLIT_TAILS = [  # row tiles, column tiles, k (per operand pair): the tail of `row tiles x column tiles` tiles on 256
+    # compute units is cut along the reduction into min(256 // tail, 8, K tiles // 8) parts
+    (12, 1, 1024),    # 12 tiles, 16 K tiles: two parts
+    (12, 1, 4096),    # eight parts
+    (68, 16, 1024),   # four full rounds and 64 tiles: four parts (the shape of a Mixtral-sized second product, shorter)
+    (85, 1, 768),     # three parts; with two operand pairs the middle one straddles the change of pairs
+    (51, 1, 1280),    # five parts
+    (36, 1, 1792),    # seven parts
+    (3, 43, 640),     # 129 tiles: more than half a round, not cut
+    (64, 5, 512),     # a whole round and 64 tiles, reductions too short to cut (8 K tiles): half-height tiles
+]
+
+
+@pytest.mark.parametrize('row_tiles,col_tiles,k', SPLIT_TAILS)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_gmm_tail_cut_along_the_reduction(gg, row_tiles, col_tiles, k, dtype):
+    """NN products whose last round of workgroups is at most half full compute its tiles in parts along K, summed through
+    the workspace in a fixed order (mbx_gmm_ws): against fp32, block by block; bit-identical from run to run; the
+    workspace's counters are zero again afterwards; without workspace the same values to rounding of the sums' order."""
+    from megablocks_amd import _lib
+    groups, n = 4, 256 * col_tiles
+    per = [256 * (row_tiles // groups)] * groups
+    per[0] += 256 * (row_tiles % groups) - 100                       # a ragged last row tile in one expert
+    if per[2] >= 256:
+        per[2] -= 256
+        per[3] += 256
+    sizes = torch.tensor(per, dtype=torch.int64)
+    rows = int(sizes.sum())
+    torch.manual_seed(row_tiles * 100 + col_tiles)
+    a = torch.randn(rows, k, device='cuda').to(dtype)
+    b = (torch.randn(groups, k, n, device='cuda') * 0.1).to(dtype)
+    a2 = torch.randn(rows, k, device='cuda').to(dtype)
+    b2 = (torch.randn(groups, k, n, device='cuda') * 0.1).to(dtype)
+    ref = _ref_gpu(a, b, sizes, False, False)
+    ref2 = ref + _ref_gpu(a2, b2, sizes, False, False)
+    guard = torch.full((rows + 64, n), 7.0, device='cuda', dtype=dtype)
+    got = gg.backend.gmm(a, b, sizes)
+    assert rel_err(got, ref) < TOL and max_block_err(got, ref) < 2 * TOL
+    got2 = gg.gmm_dual(a, b, a2, b2, sizes)
+    assert rel_err(got2, ref2) < TOL and max_block_err(got2, ref2) < 2 * TOL
+    for _ in range(3):
+        assert torch.equal(gg.backend.gmm(a, b, sizes), got) and torch.equal(gg.gmm_dual(a, b, a2, b2, sizes), got2)
+    ws = gg._workspaces[(torch.cuda.current_device(), _lib.stream().value)]
+    assert int(ws[:4096].count_nonzero()) == 0                      # every launch leaves the counters as it found them
+    assert bool((guard == 7.0).all())
+    # the C ABI without a workspace: one workgroup per tile (or half tile)
+    bins = torch.cumsum(sizes, 0).int().cuda()
+    plain = torch.empty_like(got)
+    _lib.check(_lib.lib.mbx_gmm(_lib.ptr(a), _lib.ptr(b), _lib.ptr(plain), _lib.dtype_of(a), _lib.ptr(bins), groups, rows, k, n,
+                                _lib.NN, _lib.stream()))
+    assert rel_err(plain, ref) < TOL and rel_err(plain.float(), got.float()) < 2e-3
+    # a workspace too small for two parts per tail tile, or misaligned: ignored
+    small = torch.zeros(4096 + 100, dtype=torch.uint8, device='cuda')
+    out = torch.empty_like(got)
+    _lib.check(_lib.lib.mbx_gmm_ws(_lib.ptr(a), _lib.ptr(b), None, None, _lib.ptr(out), _lib.dtype_of(a), _lib.ptr(bins), groups,
+                                   rows, k, n, _lib.NN, _lib.ptr(small), small.numel(), _lib.stream()))
+    assert torch.equal(out, plain)
+    assert _lib.lib.mbx_gmm_ws(_lib.ptr(a), _lib.ptr(b), _lib.ptr(a2), None, _lib.ptr(out), _lib.dtype_of(a), _lib.ptr(bins), groups,
+                               rows, k, n, _lib.NN, None, 0, _lib.stream()) == _lib.EINVAL
+
+
 MIXED_ROWS = [  # per-expert row counts around the boundaries between full (256-row) and half-height (128-row) tiles
     [256, 257, 300, 384, 385, 129, 128, 1, 0, 512, 640, 127],
     [300] * 48,                       # full and half-height tiles alternate along the tile list, several rounds
