@@ -1225,53 +1225,60 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
           // store would take two registers each, which this kernel does not have).  Eight tiles at a time, so that the
           // compiler does not gather all 256 registers of a part in one place.
           constexpr uint32_t kPartBytes = (uint32_t)T::BM * T::BN * 4, kTileStep = (uint32_t)T::THREADS * 16;
+          constexpr int kThroughCaches = 0x11;   // cache policy bits sc0 | sc1 of a buffer access: system scope
           const uint32_t lane_off = threadIdx.x * 16u;
           const __amdgpu_buffer_rsrc_t mine = make_rsrc((const char*)ws_parts + (size_t)j * kPartBytes, kPartBytes);
           static_for<T::TM>([&](auto ii) {
             constexpr int i = decltype(ii)::value;
 #pragma unroll
             for (int jj = 0; jj < T::TN; ++jj)
-              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][jj]), mine, (int)lane_off, (int)((i * T::TN + jj) * kTileStep), 0);
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][jj]), mine, (int)lane_off, (int)((i * T::TN + jj) * kTileStep), kThroughCaches);
             __builtin_amdgcn_sched_barrier(0);
           });
-          __threadfence();                       // the part is visible to the whole device before it is counted
-          __syncthreads();                       // ... every wave's share of it; and nobody reads the LDS stages any more
+          // The parts go between workgroups on different XCDs, whose L2 caches do not see each other: they are stored
+          // and loaded past the caches (write-through stores, loads that always miss) instead of between a release
+          // and an acquire fence, which here would mean a write-back of the whole L2 by every wave of every part
+          // and an invalidation under the workgroups that are still multiplying.  A part is counted in once every
+          // wave's stores have been acknowledged; the counter is a device-wide atomic.
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();                       // every wave's share of the part is out; nobody reads the LDS stages any more
           int* const flag = (int*)lds;
-          if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(ws_counters + tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+          if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(ws_counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           __syncthreads();
           const bool last = *flag == ksplit - 1;  // uniform
           if (last) {
-            __threadfence();                     // the other parts as their workgroups published them
             // The sum of the parts, in part order whoever came last, goes straight to the staging area of the store:
             // one row of product tiles at a time, the parts of up to four workgroups in flight together.
-            static_for<T::TM>([&](auto ii) {
-              constexpr int i = decltype(ii)::value;
-              f32x4 sum[T::TN];
+            constexpr int kRowsAtOnce = 1, kTilesAtOnce = kRowsAtOnce * T::TN;   // rows of product tiles per batch of loads
+            static_assert(T::TM % kRowsAtOnce == 0, "batches of the reduction");
+            static_for<T::TM / kRowsAtOnce>([&](auto ii) {
+              constexpr int t0_ = decltype(ii)::value * kTilesAtOnce;         // first product tile of the batch
+              f32x4 sum[kTilesAtOnce];
 #pragma unroll 1
               for (int p0 = 0; p0 < ksplit; p0 += 4) {
-                u32x4 v[4][T::TN];
+                u32x4 v[4][kTilesAtOnce];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                   if (p0 + u < ksplit) {
                     const __amdgpu_buffer_rsrc_t theirs = make_rsrc((const char*)ws_parts + ((size_t)(p0 + u) * rest + tile) * kPartBytes, kPartBytes);
 #pragma unroll
-                    for (int jj = 0; jj < T::TN; ++jj)
-                      v[u][jj] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(theirs, (int)lane_off, (int)((i * T::TN + jj) * kTileStep), 0));
+                    for (int t = 0; t < kTilesAtOnce; ++t)
+                      v[u][t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(theirs, (int)lane_off, (int)((t0_ + t) * kTileStep), kThroughCaches));
                   }
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                   if (p0 + u < ksplit) {
 #pragma unroll
-                    for (int jj = 0; jj < T::TN; ++jj) {
-                      const f32x4 w = __builtin_bit_cast(f32x4, v[u][jj]);
-                      sum[jj] = (p0 == 0 && u == 0) ? w : sum[jj] + w;
+                    for (int t = 0; t < kTilesAtOnce; ++t) {
+                      const f32x4 w = __builtin_bit_cast(f32x4, v[u][t]);
+                      sum[t] = (p0 == 0 && u == 0) ? w : sum[t] + w;
                     }
                   }
                 }
               }
 #pragma unroll
-              for (int jj = 0; jj < T::TN; ++jj) stage_product_tile<DT, T>(lds, i, jj, sum[jj]);
+              for (int t = 0; t < kTilesAtOnce; ++t) stage_product_tile<DT, T>(lds, (t0_ + t) / T::TN, (t0_ + t) % T::TN, sum[t]);
               __builtin_amdgcn_sched_barrier(0);
             });
             if (threadIdx.x == 0) ws_counters[tile] = 0;   // as the launch found it
