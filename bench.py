@@ -59,6 +59,8 @@ def parse():
     ap.add_argument('--operand-patterns', action='store_true',
                     help='also time the grouped GEMM launches on all-zero and all-one operands (same shapes): what the '
                          'same instruction stream gives when the operands cost no switching power')
+    ap.add_argument('--tile-ticks', action='store_true',
+                    help='only: per-tile phase times of the grouped products, from the build with time stamps (libmbx_ticks.so)')
     ap.add_argument('--mfma-ceiling', action='store_true',
                     help='also run a loop of matrix-core instructions alone (no LDS, no memory) on all-zero, all-one and '
                          'N(0,1) bf16 operands: the rate and shader clock the power limit allows on such values')
@@ -334,6 +336,81 @@ def operand_pattern_leg(w, inp):
     return res
 
 
+def tile_ticks_leg(w, inp):
+    """Where the time of an output tile goes, for the three grouped products of this workload's shapes: the kernels of
+    libmbx_ticks.so (the library compiled with -DMBX_TICKS; loaded instead of libmbx.so by this leg) stamp every tile
+    with the constant-rate clock (100 MHz) when it starts, when its first K tile has landed, after its last MFMA, after
+    its last store has been issued and after the workgroup's LDS has been handed on.  One launch per product is read
+    back; times are microseconds per tile, averaged over the launch's tiles."""
+    import ctypes
+
+    import torch
+
+    from megablocks_amd import _lib
+    from megablocks_amd import grouped_gemm_util as gg
+
+    if not hasattr(_lib.lib, 'mbx_debug_set_ticks'):
+        raise RuntimeError('bench.py --tile-ticks needs megablocks_amd/libmbx_ticks.so (python megablocks_amd/build.py)')
+    set_ticks = _lib.lib.mbx_debug_set_ticks
+    set_ticks.restype, set_ticks.argtypes = ctypes.c_int, [ctypes.c_void_p]
+    dev = torch.device('cuda', 0)
+    if w.routing == 'router':
+        logits = inp['x'].to(dev).float() @ inp['router_weight'].to(dev).float().t()
+        top = logits.topk(w.top_k, dim=-1).indices
+    else:
+        top = inp['top_experts'].to(dev)
+    sizes = torch.bincount(top.flatten(), minlength=w.experts).to(torch.int64)
+    rows = int(sizes.sum())
+    a = torch.randn(rows, w.hidden, device=dev).to(w.dtype)
+    mid = torch.randn(rows, w.ffn, device=dev).to(w.dtype)
+    w1 = (torch.randn(w.experts, w.ffn, w.hidden, device=dev) * 0.02).to(w.dtype)
+    workgroups, tiles, ids = 16384, 64, 8                               # kTickWorkgroups, kTickTiles, kTickIds of gmm_dma.h
+    buf = torch.zeros(workgroups * tiles * ids, dtype=torch.int64, device=dev)
+    res = {'what': 'per-tile phase times (us) from the time stamps of libmbx_ticks.so, one launch per product', 'products': {}}
+    for name, fn in (('gmm_nt', lambda: gg.backend.gmm(a, w1, sizes, trans_b=True)),
+                     ('gmm_nn', lambda: gg.backend.gmm(mid, w1, sizes)),
+                     ('gmm_tn', lambda: gg.backend.gmm(mid, a, sizes, trans_a=True))):
+        _lib.check(set_ticks(None), 'set_ticks')
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        buf.zero_()
+        torch.cuda.synchronize()
+        _lib.check(set_ticks(ctypes.c_void_p(buf.data_ptr())), 'set_ticks')
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        torch.cuda.synchronize()
+        _lib.check(set_ticks(None), 'set_ticks')
+        t = buf.view(workgroups, tiles, ids).cpu().double() / 100.0     # microseconds
+        done = (t[:, :, 0] > 0) & (t[:, :, 1] > 0) & (t[:, :, 5] > 0)
+        n = int(done.sum())
+        phase = lambda x, y: float((t[:, :, y] - t[:, :, x])[done].mean())
+        nxt = torch.zeros_like(done)
+        nxt[:, :-1] = done[:, :-1] & done[:, 1:]
+        between = (t[:, 1:, 0] - t[:, :-1, 5])[nxt[:, :-1]]
+        start = t[:, :, 0][done].min()
+        # a workgroup's first tile has no stores of a tile before it in flight; its last one may be a part of a tile
+        # (mbx_gmm_ws: the tail of an NN launch) whose "stores" include the reduction of the parts
+        per_ordinal = {}
+        for o in range(min(tiles, 8)):
+            if int(done[:, o].sum()):
+                sel = done[:, o]
+                per_ordinal[str(o)] = [round(float((t[:, o, y] - t[:, o, x])[sel].mean()), 2) for x, y in ((0, 1), (1, 2), (2, 4))]
+        res['products'][name] = dict(
+            launch_ms=round(e0.elapsed_time(e1), 4), tiles=n, workgroups=int(done.any(dim=1).sum()),
+            start_to_first_k_tile=round(phase(0, 1), 2),
+            of_which=dict(find_the_tile=round(phase(0, 6), 2), request_first_k_tiles=round(phase(6, 7), 2),
+                          clear_accumulators=round(phase(7, 3), 2), wait_for_first_k_tile=round(phase(3, 1), 2)),
+            main_loop=round(phase(1, 2), 2),
+            last_mfma_to_last_store_issued=round(phase(2, 4), 2), hand_over=round(phase(4, 5), 2),
+            between_tiles_of_a_workgroup=round(float(between.mean()), 2) if between.numel() else None,
+            tile_total=round(phase(0, 5), 2), by_ordinal_of_the_tile_in_its_workgroup_start_loop_store=per_ordinal,
+            first_tile_start_to_last_tile_end_ms=round(float(t[:, :, 5][done].max() - start) / 1000.0, 4))
+    return res
+
+
 def mfma_ceiling_leg():
     """A loop of matrix-core instructions alone (libmbx_probe.so: operands and accumulators stay in registers; no LDS
     reads, no memory traffic), about a second per case, on operands that are all zero, all one, and N(0,1) bf16
@@ -443,6 +520,8 @@ def main():
         print(f'bench.py: this build runs on one GPU holding all experts; --gpus {args.gpus} is not supported '
               '(the expert-parallel all-to-all is out of scope).', file=sys.stderr)
         sys.exit(2)
+    if args.tile_ticks:   # before the package is imported: it loads the library named here
+        os.environ['MBX_LIBRARY'] = os.path.join(ROOT, 'megablocks_amd', 'libmbx_ticks.so')
     import torch
 
     from megablocks_amd import synthetic
@@ -452,6 +531,10 @@ def main():
         import dataclasses
         w = dataclasses.replace(w, tokens=args.tokens)
     inp = synthetic.make_inputs(w, seed=0)
+    if args.tile_ticks:
+        print(json.dumps({'config': {'workload': f'{w.name}: {w.description}', 'tokens': w.tokens},
+                          'tile_ticks': tile_ticks_leg(w, inp)}))
+        return
     ms_per_step, ms_wall, agg, layer = gpu_leg(args, w, inp)
 
     slots_scale = 1.0

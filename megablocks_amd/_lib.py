@@ -9,7 +9,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, 'libmbx.so')
+# MBX_LIBRARY: another build of the library to load instead (measurements: libmbx_ticks.so)
+LIB_PATH = os.environ.get('MBX_LIBRARY') or os.path.join(_HERE, 'libmbx.so')
 
 I16, I32, I64 = 0, 1, 2
 BF16, F16, F32 = 0, 1, 2

@@ -16,6 +16,8 @@ CSRC = os.path.join(HERE, 'csrc')
 BUILD = os.path.join(HERE, 'build')
 LIB = os.path.join(HERE, 'libmbx.so')
 PROBE_LIB = os.path.join(HERE, 'libmbx_probe.so')
+# the library with per-tile time stamps in the grouped-GEMM kernels (csrc/gmm_dma.h, MBX_TICKS), for bench.py --tile-ticks
+TICKS_LIB = os.path.join(HERE, 'libmbx_ticks.so')
 PROBE_SOURCE = 'probe.hip'
 SOURCES = ['routing.hip', 'permute.hip', 'gmm.hip', 'elementwise.hip', 'router.hip']
 HEADERS = [os.path.join(CSRC, 'common.h'), os.path.join(CSRC, 'gmm_dma.h'),
@@ -57,6 +59,14 @@ def build(force: bool = False, verbose: bool = False) -> str:
             if verbose:
                 print(' '.join(cmd), flush=True)
             procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    # gmm.hip a second time with the time stamps compiled in
+    gmm_src, ticks_obj = os.path.join(CSRC, 'gmm.hip'), os.path.join(BUILD, 'gmm_ticks.o')
+    ticks_stale = force or not os.path.exists(ticks_obj) or os.path.getmtime(ticks_obj) < max(os.path.getmtime(gmm_src), newest_header)
+    if ticks_stale:
+        cmd = [hipcc] + FLAGS + ['-DMBX_TICKS', '-c', gmm_src, '-o', ticks_obj]
+        if verbose:
+            print(' '.join(cmd), flush=True)
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     probe_src = os.path.join(CSRC, PROBE_SOURCE)
     probe_cmd = None
     if force or not os.path.exists(PROBE_LIB) or os.path.getmtime(PROBE_LIB) < max(os.path.getmtime(probe_src), newest_header):
@@ -68,8 +78,10 @@ def build(force: bool = False, verbose: bool = False) -> str:
         out, _ = p.communicate()
         if p.returncode != 0:
             raise RuntimeError(f'command failed: {" ".join(cmd)}\n{out}')
-    if [c for c, _ in procs if c is not probe_cmd] or force or not os.path.exists(LIB):
+    if [c for c, _ in procs if c is not probe_cmd] or force or not os.path.exists(LIB) or not os.path.exists(TICKS_LIB):
         _run([hipcc, '-shared', '-fPIC', f'--offload-arch={ARCH}', '-o', LIB] + objs)
+        _run([hipcc, '-shared', '-fPIC', f'--offload-arch={ARCH}', '-o', TICKS_LIB] +
+             [ticks_obj if o.endswith(os.sep + 'gmm.o') else o for o in objs])
     return LIB
 
 

@@ -738,6 +738,13 @@ using namespace mbx;
 
 extern "C" {
 
+#ifdef MBX_TICKS
+// libmbx_ticks.so only: where the kernels of gmm_dma.h put their per-tile time stamps (see there); NULL: nowhere.
+int mbx_debug_set_ticks(void* buffer) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(dma::g_ticks), &buffer, sizeof(buffer));
+}
+#endif
+
 size_t mbx_gmm_workspace_bytes(void) { return kWorkspaceCounters * sizeof(int32_t) + kWorkspaceParts * kWorkspacePartBytes; }
 
 static int gmm_dual_ws(const void* a, const void* b, const void* a2, const void* b2, void* c, int dtype, const int32_t* bins,

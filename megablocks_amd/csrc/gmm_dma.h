@@ -65,6 +65,23 @@ struct Tile {
 
 typedef __attribute__((address_space(3))) char* lds_ptr;
 
+// Measurement build only (libmbx_ticks.so, compiled with -DMBX_TICKS; the library proper has none of this): the first
+// lane of a workgroup stamps the phases of every output tile with the constant-rate clock (s_memrealtime, 100 MHz) into
+//   g_ticks[(workgroup * kTickTiles + ordinal of the tile in the workgroup) * kTickIds + id]
+// id 0: tile starts, 6: its operands are known, 7: the first K tiles are requested, 3: the accumulators are cleared,
+// 1: the first K tile has landed, 2: last MFMA done, 4: the tile's last store issued, 5: LDS handed on.
+#ifdef MBX_TICKS
+__device__ uint64_t* g_ticks;
+constexpr int kTickWorkgroups = 16384, kTickTiles = 64, kTickIds = 8;   // the buffer's shape (8 bytes per entry)
+__device__ __forceinline__ void tick(int ordinal, int id) {
+  if (threadIdx.x == 0 && g_ticks != nullptr && ordinal >= 0 && ordinal < kTickTiles && blockIdx.x < kTickWorkgroups)
+    g_ticks[((size_t)blockIdx.x * kTickTiles + ordinal) * kTickIds + id] = __builtin_amdgcn_s_memrealtime();
+}
+#define MBX_TICK(ordinal, id) tick(ordinal, id)
+#else
+#define MBX_TICK(ordinal, id) ((void)0)
+#endif
+
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
 // expression in the body (it selects instruction immediates).
 template <typename F, int... I>
@@ -194,6 +211,7 @@ struct Args {
   // a lane's LA loads of a K tile fetches the 16 bytes at gather_row[q] (+ the K tile's offset); bit 31 set: the row
   // is a row of zeros.
   uint32_t gather_row[8];
+  int tick_ordinal = -1;                  // MBX_TICKS builds: which tile of the workgroup this is
 };
 
 // acc += a-fragment x b-fragment with v_mfma_f32_16x16x32, written as inline asm with the accumulator tied to one
@@ -392,6 +410,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
   constexpr int WAIT_PROLOGUE = (SB - 1) * (LA + LB);        // tile 0 has landed
   constexpr int WAIT_LOOP = (SB - 2) * (LA + LB) + LA;       // tile kt + 1 has landed: everything up to B tile kt + 1
   static_assert(SB * (LA + LB) < 64, "vmcnt is a 6-bit counter");
+  MBX_TICK(g.tick_ordinal, 6);
   if (nk > 0) {
 #pragma unroll
     for (int t = 0; t < SB; ++t) {
@@ -400,6 +419,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
     }
   }
   __builtin_amdgcn_sched_barrier(0);
+  MBX_TICK(g.tick_ordinal, 7);
   if (clear) {
 #pragma unroll
     for (int i = 0; i < T::TM; ++i)
@@ -409,8 +429,10 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
         for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
   }
   if (nk > 0) {
+    MBX_TICK(g.tick_ordinal, 3);
     wait_vmcnt<WAIT_PROLOGUE>();
     __builtin_amdgcn_s_barrier();
+    MBX_TICK(g.tick_ordinal, 1);
     mfma16_settle();   // the accumulators were written by vector-ALU instructions
     static_for<NS>([&](auto mi_) { constexpr int m_ = decltype(mi_)::value; MBX_READ_SLOT16(0, 0, lds_base, lds_base + B_RING, m_); });
 
@@ -907,7 +929,9 @@ __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__
                                            const uint16_t* __restrict__ pre2 = nullptr, uint16_t* __restrict__ out2 = nullptr) {
   typename T::Acc acc[T::TM][T::TN];
   block_multiply<DT, A_MC, B_MC, T, DUAL, epi_is_glu(EPI), GATHER>(g, acc, true, lds);
+  MBX_TICK(g.tick_ordinal, 2);
   block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra, pre2, out2);
+  MBX_TICK(g.tick_ordinal, 4);
 }
 
 
@@ -1198,6 +1222,8 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
           const int j = xcd * run + member;
           if (j >= ksplit * rest) break;
           const int tile = j % rest, part = j / rest;
+          g.tick_ordinal = r;
+          MBX_TICK(r, 0);
           int e, start, end, tm, tn;
           tiles.find(full_rounds * P + tile, e, start, end, tm, tn);
           const int row0 = start + tm * T::BM;
@@ -1218,6 +1244,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
           g.b_r0 = tn * kTileCols;
           typename T::Acc acc[T::TM][T::TN];
           block_multiply<DT, false, B_MC, T, DUAL>(g, acc, true, lds);
+          MBX_TICK(r, 2);
           g.nk = nk_all;
           g.nk1 = nk1;
           // The part's accumulators as they lie in the registers: 16 bytes per lane and product tile, addressed as a
@@ -1284,7 +1311,9 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
             if (threadIdx.x == 0) ws_counters[tile] = 0;   // as the launch found it
             block_store<DT, T, kEpiNone, true>(acc, c + (int64_t)row0 * n, n, 0, end - row0, g.b_r0, n, lds);
           }
+          MBX_TICK(r, 4);
           tile_done();
+          MBX_TICK(r, 5);
         }
         continue;
       } else {
@@ -1294,6 +1323,8 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
         half = j & 1;
         use_ts = true;
       }
+      g.tick_ordinal = r;
+      MBX_TICK(r, 0);
       int e, start, end, tm, tn;
       tiles.find(id, e, start, end, tm, tn);
       const int row0 = start + tm * T::BM + half * TS::BM;
@@ -1318,6 +1349,7 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
         block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
       }
       tile_done();
+      MBX_TICK(r, 5);
     }
   } else {
     // The assignments of a tile's rows are fetched while the tile before it is computed (the tile's loads cannot start
@@ -1539,6 +1571,8 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
   const int64_t member = blockIdx.x / kXcds;
   const int64_t first = (member / 32) * 32 * chunk + member % 32;
   for (int64_t i = first; i < first + (int64_t)32 * chunk && i < items; i += 32) {
+    g.tick_ordinal = (int)((i - first) / 32);
+    MBX_TICK(g.tick_ordinal, 0);
     int slot, t;   // position of the expert in the longest-first order, tile slot inside the expert
     if (whole) {
       const int q = (int)(i / per_group);
@@ -1574,6 +1608,7 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
       tn_tile<DT, T, SEGMENTED>(g, a, b, c_e, start, end, k, n, seg_rows, lds);
     }
     tile_done();
+    MBX_TICK(g.tick_ordinal, 5);
   }
 }
 
