@@ -282,6 +282,25 @@ int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int to
                    const void* b1, const void* b2, void* c, void* c2, void* h, int dtype, const int32_t* bins,
                    int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
 
+/* The weight gradient of the experts' first product(s) on token rows that were never gathered: the backward's
+ * `gmm(dsdd_out, x, batch_sizes, trans_a=True)` of megablocks/layers/mlp.py:485-491 / glu.py:154-159, where x is what
+ * megablocks/layers/dmoe.py:219 / :273 gathered (`ops.padded_gather` / `ops.gather`), with that gather done by the
+ * operand loads -- the counterpart of mbx_gmm_gather for the training step, so that the gathered copy exists in neither
+ * pass:
+ *   c[e] = a[r_e]^T @ X[r_e],   X[first(e) + r] = x[indices[x_first(e) + r] / top_k] for r < x_bins[e] - x_first(e), else 0
+ * (a: [rows, k]; x: [x_rows, n]; c: [E, k, n]; bins, x_bins, first, x_first as for mbx_gmm_gather).  Bit-identical to
+ * mbx_gather / mbx_padded_gather followed by mbx_gmm(MBX_TN).
+ * row_table: scratch of mbx_gmm_tn_gather_table_bytes(x_rows, top_k, num_groups) bytes (16-byte aligned) in which the
+ * call builds the byte offset of every assignment's row, in the order the kernel's loads want them; table_ready != 0:
+ * an earlier call with the same indices, x_bins, top_k, x_rows, num_groups and n has left it there (the two weight
+ * gradients of a GLU layer share one).  MBX_ESCRATCH: no table, or too small or misaligned a one.
+ * MBX_EUNSUPPORTED (the caller gathers and calls mbx_gmm): fp32, k or n not multiples of 8, operands not 16-byte
+ * aligned, k of 128 or less, x or an operand of 2 GiB or more. */
+size_t mbx_gmm_tn_gather_table_bytes(int64_t x_rows, int top_k, int num_groups);
+int mbx_gmm_tn_gather(const void* a, const void* x, int64_t x_rows, const int32_t* indices, int top_k, const int32_t* x_bins,
+                      void* c, int dtype, const int32_t* bins, int num_groups, int64_t rows, int k, int n, void* row_table,
+                      size_t row_table_bytes, int table_ready, mbx_stream_t stream);
+
 /* The backward of the GLU experts' gated activation on the product that feeds it, megablocks/layers/glu.py:135-153
  * (`gmm(ddsd_out, w2, trans_b=True, c=dactivation_fn_out)`, then autograd's gradient of
  * `activation_fn(sdd_out) * v1_out`, glu.py:120-124), in one launch:

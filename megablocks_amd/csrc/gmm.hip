@@ -572,9 +572,14 @@ struct Workspace {
   size_t bytes = 0;
 };
 struct GatherRows {
-  const int32_t* slots = nullptr;      // non-null: a is [src_rows, k], read through the row map
+  const int32_t* slots = nullptr;      // non-null: a (NT) / b (TN) is [src_rows, .], read through the row map
   const int32_t* src_bins = nullptr;
   int top_k = 1, src_rows = 0;
+  // TN only: the table of row offsets the kernel reads (4 bytes per sorted assignment, n_slots of them), and whether an
+  // earlier call with the same slots, top_k, src_rows and n has already filled it
+  uint32_t* row_table = nullptr;
+  int64_t n_slots = 0;
+  bool table_ready = false;
 };
 template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
@@ -610,7 +615,28 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (grid > 0x7fffffff) return MBX_ERANGE;
     // whole experts per XCD (if the kernel finds them balanced): for reductions of a few K tiles only
     const int whole_ok = avg_rows < 1024 ? 1 : 0;
-    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, shape.bm, shape.bn, chunk, (int)seg_rows, whole_ok);
+    if (gather.slots) {
+      // the rows of b picked through the sorted assignments: the full tile only, one segment
+      if (!gather.src_bins || !gather.row_table || gather.top_k <= 0 || gather.n_slots > 0x7fffffff) return MBX_EINVAL;
+      if (segmented || !std::is_same<T, TS>::value) return MBX_EUNSUPPORTED;
+      if (!gather.table_ready) {
+        uint32_t magic = 0;
+        int shift = 0;
+        dma::gather_divisor(gather.top_k, magic, shift);
+        dma::gather_row_table_kernel<<<(unsigned)ceil_div(dma::row_table_entries(gather.n_slots, num_groups), 256), 256, 0, s>>>(
+            gather.slots, gather.src_bins, num_groups, (int)gather.n_slots, gather.src_rows, (uint32_t)n * 2u, magic, shift, gather.row_table);
+      }
+      if constexpr (T::BM == 256 && T::SB == 2) {
+        auto gkern = dma::gmm_tn_kernel<DT, T, T, false, true>;
+        int grc = allow_lds(gkern, lds);
+        if (grc) return grc;
+        gkern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, shape.bm, shape.bn, chunk, (int)seg_rows, whole_ok, gather.row_table, gather.src_bins, gather.src_rows, (int)gather.n_slots);
+        return launch_status();
+      } else {
+        return MBX_EUNSUPPORTED;
+      }
+    }
+    kern<<<(unsigned)grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, (int)rows, k, n, tiles_m, tiles_n, shape.bm, shape.bn, chunk, (int)seg_rows, whole_ok, nullptr, nullptr, 0, 0);
     return launch_status();
   }
   constexpr size_t lds = T::LDS_BYTES > TS::LDS_BYTES ? T::LDS_BYTES : TS::LDS_BYTES;
@@ -907,6 +933,40 @@ int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int to
   gather.src_rows = (int)x_rows;
   const int epi = b2 ? (act == MBX_ACT_SILU ? dma::kEpiGluSilu : dma::kEpiGluGelu) : h ? dma::kEpiAct : dma::kEpiNone;
   return gmm_nt_epilogue(x, b1, c, h, dtype, bins, num_groups, rows, k, n, act, epi, stream, nullptr, c2, b2, gather);
+}
+
+size_t mbx_gmm_tn_gather_table_bytes(int64_t x_rows, int top_k, int num_groups) {
+  if (x_rows < 0 || top_k <= 0 || num_groups < 0) return 0;
+  return (size_t)dma::row_table_entries(x_rows * top_k, num_groups) * 4;
+}
+
+int mbx_gmm_tn_gather(const void* a, const void* x, int64_t x_rows, const int32_t* indices, int top_k, const int32_t* x_bins,
+                      void* c, int dtype, const int32_t* bins, int num_groups, int64_t rows, int k, int n, void* row_table,
+                      size_t row_table_bytes, int table_ready, mbx_stream_t stream) {
+  if (x_rows < 0 || top_k <= 0 || k < 0 || n < 0 || num_groups < 0 || rows < 0) return MBX_EINVAL;
+  if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
+  if (num_groups == 0 || (int64_t)k * n == 0) return 0;
+  if (!c || !bins || !indices || (rows > 0 && !a) || (x_rows > 0 && !x)) return MBX_EINVAL;
+  if (rows > 0x7fffffff) return MBX_ERANGE;
+  const int64_t n_slots = x_rows * top_k;
+  // the kernel with the full tile, 16-byte pieces of rows, one segment of the reduction, row offsets of 31 bits
+  const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(x) && aligned16(c) && k % 8 == 0 && n % 8 == 0 && dma_sizes_ok(k, n) &&
+                  k > TileDmaSmallM::BM && n_slots <= 0x7fffffff && x_rows * (int64_t)n * 2 < ((int64_t)1 << 31) &&
+                  rows * (int64_t)(k > n ? k : n) * 2 < ((int64_t)1 << 31);
+  if (!ok) return MBX_EUNSUPPORTED;
+  if (!row_table || row_table_bytes < mbx_gmm_tn_gather_table_bytes(x_rows, top_k, num_groups) || ((uintptr_t)row_table & 15u)) return MBX_ESCRATCH;
+  if (x_rows == 0) x = a ? a : c;   // no row is read; the buffer descriptor still wants an address
+  GatherRows gather;
+  gather.slots = indices;
+  gather.src_bins = x_bins ? x_bins : bins;
+  gather.top_k = top_k;
+  gather.src_rows = (int)x_rows;
+  gather.row_table = (uint32_t*)row_table;
+  gather.n_slots = n_slots;
+  gather.table_ready = table_ready != 0;
+  hipStream_t s = as_stream(stream);
+  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDma>(a, x, c, bins, num_groups, rows, k, n, MBX_TN, s, nullptr, nullptr, dma::kEpiNone, nullptr, nullptr, gather);
+  return gmm_dma<MBX_F16, TileDma, TileDma>(a, x, c, bins, num_groups, rows, k, n, MBX_TN, s, nullptr, nullptr, dma::kEpiNone, nullptr, nullptr, gather);
 }
 
 int mbx_gmm_dglu(const void* a, const void* b, const void* x1, const void* x2, void* d1, void* d2, int dtype,

@@ -211,8 +211,37 @@ struct Args {
   // a lane's LA loads of a K tile fetches the 16 bytes at gather_row[q] (+ the K tile's offset); bit 31 set: the row
   // is a row of zeros.
   uint32_t gather_row[8];
+  // GATHER_B instantiations (TN): the rows of the B tile (an MC operand: its rows are the reduction) are rows of the
+  // matrix behind rsrc_b picked by a row map.  The map comes as a table of byte offsets, one 4-byte entry per row of
+  // the reduction (bit 31 flipped: an entry read past the end of the table, i.e. zero, then means "no row"), read
+  // through row_table (words of a buffer descriptor over the expert's part of the table).  gather_row / gather_row2:
+  // the entries of this lane's loads of K tiles 0 and 1, fetched by the caller while the tile before was computed.
+  uint32_t gather_row2[8];
+  u32x4 row_table;
   int tick_ordinal = -1;                  // MBX_TICKS builds: which tile of the workgroup this is
 };
+
+// Row tables (see Args::row_table) are laid out for the loads that read them: 64 entries per K tile of an expert, in the
+// order in which the lanes want them.  Load q (of 8) of wave w (of 4) holds rows 2 j and 2 j + 1 of the K tile,
+// j = w + 4 q, lanes 0 .. 31 the first; so the eight entries a lane needs for a K tile (q = 0 .. 7, row parity kl =
+// lane / 32) sit together at entries (2 w + kl) 8 .. + 7, and a lane fetches them with two 16-byte loads.
+// row_entry_slot(): where the entry of row r of a K tile is; row_of_entry_slot(): its inverse.
+constexpr int kRowTableTile = 64;   // entries per K tile
+__host__ __device__ constexpr int row_entry_slot(int r) { return (((r >> 1) & 3) * 2 + (r & 1)) * 8 + (r >> 3); }
+__host__ __device__ constexpr int row_of_entry_slot(int p) { return 2 * ((p >> 4) + 4 * (p & 7)) + ((p >> 3) & 1); }
+// Expert e's part of a table starts at entry (number of assignments before it) + 64 e: room for its last K tile to be
+// whole without reaching into the next expert's part.
+__host__ __device__ constexpr int64_t row_table_entries(int64_t n_slots, int num_groups) { return n_slots + (int64_t)kRowTableTile * num_groups; }
+__device__ __forceinline__ uint32_t row_entry_lane_offset(int wave) { return (uint32_t)(2 * wave + (lane_id() >> 5)) * 32u; }
+// The eight entries of this lane for the K tile at byte offset soff of the table (inline asm, so that the compiler
+// does not count the loads among those it waits for: the main loop's own waits cover them).
+__device__ __forceinline__ void fetch_row_entries(uint32_t (&dst)[8], const u32x4& table, uint32_t voff, uint32_t soff) {
+  u32x4 lo, hi;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(lo) : "v"(voff), "s"(table), "s"(soff));
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:16" : "=v"(hi) : "v"(voff), "s"(table), "s"(soff));
+#pragma unroll
+  for (int q = 0; q < 4; ++q) { dst[q] = lo[q]; dst[4 + q] = hi[q]; }
+}
 
 // acc += a-fragment x b-fragment with v_mfma_f32_16x16x32, written as inline asm with the accumulator tied to one
 // register tuple ("+a": an AGPR tuple, source and destination): with the builtin, whose destination may differ from
@@ -244,11 +273,15 @@ __device__ __forceinline__ void mfma16_settle() { asm volatile("s_nop 15\n\ts_no
 // GATHER: the rows of the A tile (KC operand) are gathered rows of a matrix: each of a lane's LA loads of a K tile gets
 // a byte offset of its own (its row's, worked out once per tile from the row map), where the plain tile adds a
 // multiple of the row pitch to one lane offset.  The loads are the same 16-byte pieces of 128-byte row segments.
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false>
+// GATHER_B: the rows of the B tile (MC operand of 256 columns: the reduction runs over its rows) are gathered rows of a
+// matrix: each of a lane's LB loads of a K tile takes the byte offset of its row from a table (Args::row_table), which
+// it fetches a K tile ahead -- right after the load that used the entry for the K tile before, into the same register.
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false, bool GATHER_B = false>
 __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds_generic) {
   static_assert(T::KS == 2, "two k-steps of 32 per K tile");
   static_assert(!GLU || (!B_MC && !DUAL && T::LB % 2 == 0), "two matrices side by side in the B tile");
   static_assert(!GATHER || (!A_MC && !DUAL && T::BK == 64), "gathered rows: a KC operand, one operand pair");
+  static_assert(!GATHER_B || (B_MC && !DUAL && !GLU && T::BN == 256 && T::SB == 2 && T::LB == 8 && T::WAVES == 4), "gathered rows of a strided operand");
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -279,6 +312,16 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
 #pragma unroll
     for (int q = 0; q < LA; ++q) a_row[q] = g.gather_row[q];
   }
+  // GATHER_B: the lane's row offsets for the B loads it issues next (load q: b_row[q]); the column part of the address
+  // with the table's bit 31 folded in; where the lane's entries sit in a K tile's part of the table
+  uint32_t b_row[GATHER_B ? LB : 1];
+  const uint32_t b_col = GATHER_B ? load_lane_offset<B_MC, BK, T::BN>(wave, g.b_r0, 0u, false) + 0x80000000u : 0u;
+  const uint32_t b_col1 = GATHER_B ? load_lane_offset<B_MC, BK, T::BN>(wave, g.b_r0, 0u, true) + 0x80000000u : 0u;
+  const uint32_t entry_lane = GATHER_B ? row_entry_lane_offset(wave) : 0u;
+  if constexpr (GATHER_B) {
+#pragma unroll
+    for (int q = 0; q < LB; ++q) b_row[q] = g.gather_row[q];
+  }
   __amdgpu_buffer_rsrc_t ra = g.rsrc_a, rb = g.rsrc_b;
   const __amdgpu_buffer_rsrc_t rb_upper = GLU ? g.rsrc_b2 : g.rsrc_b;
   auto lds_off = [&](bool is_b, int stage, int q) -> uint32_t {
@@ -288,7 +331,11 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
   // q: the load's index among the wave's loads of the tile (GATHER, A loads: which row offset)
   auto issue = [&](bool is_b, uint32_t sc, uint32_t dst, bool odd, bool upper, int q) {
     if (is_b) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(GLU && upper ? rb_upper : rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? b_lane1 : b_lane) + sc), 0, 0, 0);
+      if constexpr (GATHER_B) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)(b_row[GATHER_B ? q : 0] + (odd ? b_col1 : b_col)), 0, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(GLU && upper ? rb_upper : rb, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((odd ? b_lane1 : b_lane) + sc), 0, 0, 0);
+      }
     } else {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(lds + dst), 16, (int)((GATHER ? a_row[GATHER ? q : 0] : odd ? a_lane1 : a_lane) + sc), 0, 0, 0);
     }
@@ -386,8 +433,12 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
       constexpr int i_ = m_ / T::TN, j_ = (i_ & 1) ? T::TN - 1 - m_ % T::TN : m_ % T::TN;                        \
       mfma16_acc<DT>(acc[i_][j_], fb[CUR_BUF][j_], fa[CUR_BUF][i_]);                                             \
       MBX_READ_SLOT16(NEXT_KSTEP, (CUR_BUF) ^ 1, NEXT_A, NEXT_B, m_);                                            \
-      if constexpr (m_ >= (LOAD0) && (m_ - (LOAD0)) % (EVERY) == 0 && (m_ - (LOAD0)) / (EVERY) < (NL))           \
+      if constexpr (m_ >= (LOAD0) && (m_ - (LOAD0)) % (EVERY) == 0 && (m_ - (LOAD0)) / (EVERY) < (NL)) {         \
         issue(IS_B, SC, DST, (((m_ - (LOAD0)) / (EVERY)) & 1) != 0, (IS_B) && (m_ - (LOAD0)) / (EVERY) >= (NL) / 2, (m_ - (LOAD0)) / (EVERY)); \
+        if constexpr (GATHER_B && (IS_B) && (m_ - (LOAD0)) / (EVERY) == (NL) - 1) {   /* the last B load of the K tile has its address: the entries of the next one */ \
+          fetch_row_entries(b_row_next, g.row_table, entry_lane, entry_sc);                                      \
+        }                                                                                                        \
+      }                                                                                                          \
       if constexpr (m_ > (LOAD0) && (m_ - (LOAD0) - 1) % (EVERY) == 0 && (m_ - (LOAD0) - 1) / (EVERY) < (NL)) {  \
         SC += T::WAVES * ((IS_B) ? b_jstep : a_jstep);                                                           \
         DST += T::WAVES * 1024u;                                                                                 \
@@ -407,15 +458,26 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
   } while (0)
 
   const int nk = g.nk;
-  constexpr int WAIT_PROLOGUE = (SB - 1) * (LA + LB);        // tile 0 has landed
+  constexpr int WAIT_PROLOGUE = (SB - 1) * (LA + LB) + (GATHER_B ? LB : 0);   // tile 0 has landed
   constexpr int WAIT_LOOP = (SB - 2) * (LA + LB) + LA;       // tile kt + 1 has landed: everything up to B tile kt + 1
   static_assert(SB * (LA + LB) < 64, "vmcnt is a 6-bit counter");
   MBX_TICK(g.tick_ordinal, 6);
+  uint32_t entry_sc = (uint32_t)(SB + 1) * (kRowTableTile * 4);   // GATHER_B: the table's part of the K tile whose entries the loop fetches next
+  uint32_t b_row_next[8];                                           // ... and where they arrive
   if (nk > 0) {
 #pragma unroll
     for (int t = 0; t < SB; ++t) {
       issue_group(false, t, t, 0, LA);
+      if constexpr (GATHER_B) {
+        if (t == 1) {
+#pragma unroll
+          for (int q = 0; q < LB; ++q) b_row[q] = g.gather_row2[q];
+        }
+      }
       issue_group(true, t, t, 0, LB);
+    }
+    if constexpr (GATHER_B) {   // K tile SB's entries, for the first loads of the loop
+      fetch_row_entries(b_row_next, g.row_table, entry_lane, (uint32_t)SB * (kRowTableTile * 4));
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -476,6 +538,12 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
       wait_frags(fa[1], fb[1]);
       wait_vmcnt<WAIT_LOOP>();
       __builtin_amdgcn_s_barrier();
+      if constexpr (GATHER_B) {   // the entries fetched a K tile ago have arrived: they are the ones the loads of k-step 1 use
+        asm volatile("" : "+v"(b_row_next[0]), "+v"(b_row_next[1]), "+v"(b_row_next[2]), "+v"(b_row_next[3]),
+                          "+v"(b_row_next[4]), "+v"(b_row_next[5]), "+v"(b_row_next[6]), "+v"(b_row_next[7]));
+#pragma unroll
+        for (int q = 0; q < LB; ++q) b_row[GATHER_B ? q : 0] = b_row_next[q];
+      }
       // k-step 1: the B loads from the first gaps on; q0 .. q3 set up the next iteration (its A loads, the stages it
       // reads after the ones this k-step prefetches from)
       auto q0 = [&]() { past = kt + 1 + SB < nk ? 0u : 0x80000000u; };
@@ -500,6 +568,7 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
         b_rd_next = b_rd_nn;
       };
       MBX_STEP16(1, 0, a_rd_next, b_rd_next, true, sc_b, dst_b, LB, 1, B_EVERY, q0, q1, q2, q3, q4, false);   // past the last tile this reads stale LDS into dead registers
+      if constexpr (GATHER_B) entry_sc += kRowTableTile * 4;
     }
     wait_vmcnt<0>();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -510,9 +579,9 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
 #undef MBX_STEP16
 }
 
-template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false>
+template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, bool GLU = false, bool GATHER = false, bool GATHER_B = false>
 __device__ __forceinline__ void block_multiply(const Args& g, typename T::Acc (&acc)[T::TM][T::TN], bool clear, char* lds) {
-  block_multiply16<DT, A_MC, B_MC, T, DUAL, GLU, GATHER>(g, acc, clear, lds);
+  block_multiply16<DT, A_MC, B_MC, T, DUAL, GLU, GATHER, GATHER_B>(g, acc, clear, lds);
 }
 
 // ---- activation in the epilogue (tanh-GELU: megablocks/layers/arguments.py:19, megablocks/layers/gelu.py:9-13) ----
@@ -1478,17 +1547,24 @@ static inline int64_t tn_grid(int tiles_m, int tiles_n, TnBlocks shape, int num_
 
 // One output tile of expert e's product: rows [g.a_r0, g.a_r0 + TT::BM) x columns [g.b_r0, g.b_r0 + TT::BN) of
 // c[e] = a[start:end]^T @ b[start:end].
-template <int DT, typename TT, bool SEGMENTED>
+// GATHER: b is the matrix the rows are picked from (its buffer, g.rsrc_b, and the row table, g.row_table /
+// g.gather_row / g.gather_row2, are the caller's business).
+template <int DT, typename TT, bool SEGMENTED, bool GATHER = false>
 __device__ __forceinline__ void tn_tile(Args& g, const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
                                         uint16_t* __restrict__ c_e, int start, int end, int k, int n, int seg_rows,
                                         char* lds) {
+  static_assert(!(GATHER && SEGMENTED), "gathered rows: one segment");
   if constexpr (!SEGMENTED) {
     // the buffers cover exactly the rows of this expert: later rows read as zero
     const int64_t group_rows = end - start;
     g.rsrc_a = make_rsrc(a + (int64_t)start * k, (uint32_t)(group_rows * k * 2));
-    g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
+    if constexpr (!GATHER) g.rsrc_b = make_rsrc(b + (int64_t)start * n, (uint32_t)(group_rows * n * 2));
     g.nk = (int)((group_rows + TT::BK - 1) / TT::BK);
-    block_gemm<DT, true, true, TT>(g, c_e, n, g.a_r0, k, g.b_r0, n, lds);
+    typename TT::Acc acc[TT::TM][TT::TN];
+    block_multiply<DT, true, true, TT, false, false, false, GATHER>(g, acc, true, lds);
+    MBX_TICK(g.tick_ordinal, 2);
+    block_store<DT, TT>(acc, c_e, n, g.a_r0, k, g.b_r0, n, lds);
+    MBX_TICK(g.tick_ordinal, 4);
   } else {
     // The reduction runs over the expert's rows in segments of at most seg_rows rows, each with buffers
     // of its own that cover exactly its rows.
@@ -1514,12 +1590,20 @@ __device__ __forceinline__ void tn_tile(Args& g, const uint16_t* __restrict__ a,
 // TS = T switches this off.
 // SEGMENTED: an expert's rows of a or b may reach 2 GiB (the launch passes seg_rows, the number of rows that
 // stays below it); otherwise the whole of a and b is smaller than that.
-template <int DT, typename T, typename TS, bool SEGMENTED>
+// GATHER: b is [src_rows, n] and row r of expert e's rows of the reduction is b[row of the r-th of its sorted
+// assignments], zeros past the expert's last assignment: the weight gradient on the rows that
+// megablocks/ops/gather.py:20-38 / padded_gather.py:20-55 would have copied out first (megablocks/layers/mlp.py:456-491,
+// glu.py:128-166: `gmm(dsdd_out, x, batch_sizes, trans_a=True)` with x the gathered tokens).  row_table: one entry per
+// sorted assignment, the byte offset of its row in b with bit 31 flipped (gather_row_table_kernel); src_bins: the
+// inclusive bins of the sorted assignments (`bins` are the row bins of a, which may be padded per expert).
+template <int DT, typename T, typename TS, bool SEGMENTED, bool GATHER = false>
 __global__ void __launch_bounds__(T::THREADS)
 gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ c,
               const int32_t* __restrict__ bins, int num_groups, int rows, int k, int n, int tiles_m, int tiles_n,
-              int bm, int bn, int chunk, int seg_rows, int whole_ok) {
+              int bm, int bn, int chunk, int seg_rows, int whole_ok, const uint32_t* __restrict__ row_table,
+              const int32_t* __restrict__ src_bins, int src_rows, int n_slots) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
+  static_assert(!GATHER || (!SEGMENTED && std::is_same<T, TS>::value), "gathered rows: one tile shape, one segment");
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "last-row tile");
   constexpr bool kMixed = T::BM != TS::BM;
   const int blocks_m = (tiles_m + bm - 1) / bm, blocks_n = (tiles_n + bn - 1) / bn;
@@ -1570,46 +1654,155 @@ gmm_tn_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, ui
   // workgroup they would be spread over `chunk` blocks at once.
   const int64_t member = blockIdx.x / kXcds;
   const int64_t first = (member / 32) * 32 * chunk + member % 32;
-  for (int64_t i = first; i < first + (int64_t)32 * chunk && i < items; i += 32) {
-    g.tick_ordinal = (int)((i - first) / 32);
-    MBX_TICK(g.tick_ordinal, 0);
+  const int64_t last = first + (int64_t)32 * chunk < items ? first + (int64_t)32 * chunk : items;
+  // entry i of this XCD's list -> expert, its rows and the tile; false for the padding of the block enumeration
+  // (uniform over the workgroup)
+  struct Entry { int e, start, end, tm, tn; };
+  auto decode = [&](int64_t i, Entry& t_) -> bool {
     int slot, t;   // position of the expert in the longest-first order, tile slot inside the expert
     if (whole) {
       const int q = (int)(i / per_group);
       slot = q * kXcds + ((q & 1) ? kXcds - 1 - xcd : xcd);
       t = (int)(i % per_group);
-      if (slot >= num_groups) continue;
+      if (slot >= num_groups) return false;
     } else {
       slot = (int)(i / per_xcd);
       t = ((xcd + slot) % kXcds) * per_xcd + (int)(i % per_xcd);
-      if (t >= per_group) continue;
+      if (t >= per_group) return false;
     }
-    int blk, in, tm, tn;
+    int blk, in;
     if (bm == kTnBlockM && bn == kTnBlockN) {   // the usual case, with constant divisors
       blk = t / (kTnBlockM * kTnBlockN), in = t % (kTnBlockM * kTnBlockN);
-      tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
+      t_.tm = (blk % blocks_m) * kTnBlockM + in % kTnBlockM, t_.tn = (blk / blocks_m) * kTnBlockN + in / kTnBlockM;
     } else {
       blk = t / (bm * bn), in = t % (bm * bn);
-      tm = (blk % blocks_m) * bm + in % bm, tn = (blk / blocks_m) * bn + in / bm;
+      t_.tm = (blk % blocks_m) * bm + in % bm, t_.tn = (blk / blocks_m) * bn + in / bm;
     }
-    if (tm >= tiles_m || tn >= tiles_n) continue;   // padding of the block enumeration (uniform over the workgroup)
-    int e = slot;
-    if (ranked) e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(__ballot(rank == slot)));
+    if (t_.tm >= tiles_m || t_.tn >= tiles_n) return false;
+    t_.e = slot;
+    if (ranked) t_.e = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(__ballot(rank == slot)));
     // bounds inside [0, rows] and in order whatever the table holds: a wrong table cannot take a load out of range
-    const int start = e > 0 ? clamp_row(bins[e - 1], rows) : 0;
-    int end = clamp_row(bins[e], rows);
-    end = end < start ? start : end;
-    g.a_r0 = tm * T::BM;
-    g.b_r0 = tn * T::BN;
-    uint16_t* const c_e = c + (int64_t)e * k * n;
-    if (kMixed && k - g.a_r0 <= TS::BM) {
-      tn_tile<DT, TS, SEGMENTED>(g, a, b, c_e, start, end, k, n, seg_rows, lds);
-    } else {
-      tn_tile<DT, T, SEGMENTED>(g, a, b, c_e, start, end, k, n, seg_rows, lds);
+    t_.start = t_.e > 0 ? clamp_row(bins[t_.e - 1], rows) : 0;
+    t_.end = clamp_row(bins[t_.e], rows);
+    t_.end = t_.end < t_.start ? t_.start : t_.end;
+    return true;
+  };
+  auto next_tile = [&](int64_t& i, Entry& t_) -> bool {   // the first entry from i on that is a tile
+    for (; i < last; i += 32)
+      if (decode(i, t_)) return true;
+    return false;
+  };
+  if constexpr (!GATHER) {
+    Entry cur;
+    for (int64_t i = first; next_tile(i, cur); i += 32) {
+      g.tick_ordinal = (int)((i - first) / 32);
+      MBX_TICK(g.tick_ordinal, 0);
+      g.a_r0 = cur.tm * T::BM;
+      g.b_r0 = cur.tn * T::BN;
+      uint16_t* const c_e = c + (int64_t)cur.e * k * n;
+      if (kMixed && k - g.a_r0 <= TS::BM) {
+        tn_tile<DT, TS, SEGMENTED>(g, a, b, c_e, cur.start, cur.end, k, n, seg_rows, lds);
+      } else {
+        tn_tile<DT, T, SEGMENTED>(g, a, b, c_e, cur.start, cur.end, k, n, seg_rows, lds);
+      }
+      tile_done();
+      MBX_TICK(g.tick_ordinal, 5);
     }
-    tile_done();
-    MBX_TICK(g.tick_ordinal, 5);
+  } else {
+    // The row entries of a tile's first two K tiles are fetched while the tile before it is computed (its loads cannot
+    // start without them): T::LB entries per K tile and lane, see row_entry_lane_offset().
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t entry_lane = row_entry_lane_offset(wave);
+    g.rsrc_b = make_rsrc(b, clip_bytes((int64_t)src_rows * n * 2));   // the whole source matrix, below 2 GiB
+    uint32_t ahead[2][T::LB];
+    // the expert's part of the table: exactly its assignments, so that an entry past them reads as zero = "no row"
+    auto table_of = [&](const Entry& t_) -> u32x4 {
+      int xs = t_.e > 0 ? src_bins[t_.e - 1] : 0, xe = src_bins[t_.e];
+      xs = xs < 0 ? 0 : (xs > n_slots ? n_slots : xs);
+      xe = xe < xs ? xs : (xe > n_slots ? n_slots : xe);
+      const uint64_t base = (uint64_t)(uintptr_t)(row_table + xs + (int64_t)kRowTableTile * t_.e);
+      u32x4 d;
+      d[0] = (uint32_t)base;
+      d[1] = (uint32_t)(base >> 32) & 0xffffu;
+      d[2] = (uint32_t)((xe - xs + kRowTableTile - 1) / kRowTableTile * kRowTableTile) * 4u;   // whole K tiles
+      d[3] = 0x00020000u;
+      return d;
+    };
+    auto fetch_ahead = [&](const u32x4& table) {
+      fetch_row_entries(ahead[0], table, entry_lane, 0u);
+      fetch_row_entries(ahead[1], table, entry_lane, (uint32_t)kRowTableTile * 4u);
+    };
+    Entry cur, nxt;
+    int64_t i = first;
+    bool have = next_tile(i, cur);
+    u32x4 table_next = {0u, 0u, 0u, 0x00020000u};
+    if (have) {
+      table_next = table_of(cur);
+      fetch_ahead(table_next);
+    }
+    bool arrived = false;   // whether a wait since fetch_ahead() has covered its loads
+    while (have) {
+      g.row_table = table_next;
+      // The entries asked for a tile ago have arrived with that tile's main loop, which ends without a load in flight;
+      // those of the workgroup's first tile, or behind a tile without rows (no main loop), are waited for here.
+      if (!arrived) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int q = 0; q < T::LB; ++q) {
+        asm volatile("" : "+v"(ahead[0][q]), "+v"(ahead[1][q]));
+        g.gather_row[q] = ahead[0][q];
+        g.gather_row2[q] = ahead[1][q];
+      }
+      int64_t i_next = i + 32;
+      const bool have_next = next_tile(i_next, nxt);
+      if (have_next) {
+        table_next = table_of(nxt);
+        fetch_ahead(table_next);
+      }
+      g.tick_ordinal = (int)((i - first) / 32);
+      MBX_TICK(g.tick_ordinal, 0);
+      g.a_r0 = cur.tm * T::BM;
+      g.b_r0 = cur.tn * T::BN;
+      tn_tile<DT, T, false, true>(g, a, b, c + (int64_t)cur.e * k * n, cur.start, cur.end, k, n, seg_rows, lds);
+      arrived = g.nk > 0;
+      tile_done();
+      MBX_TICK(g.tick_ordinal, 5);
+      cur = nxt;
+      i = i_next;
+      have = have_next;
+    }
   }
+}
+
+// The row table of the GATHER instantiation of gmm_tn_kernel, one thread per entry (see row_entry_slot() for the
+// layout): the entry of row r of K tile kt of expert e is the byte offset in the source matrix of the row of the expert's
+// (64 kt + r)-th sorted assignment (slot / top_k, as (slot * magic) >> (32 + shift), see gather_divisor()) with bit 31
+// flipped; zero -- which reads as bit 31 set: "no row" -- past the expert's assignments and for an assignment outside
+// [0, src_rows * top_k).
+__global__ void gather_row_table_kernel(const int32_t* __restrict__ slots, const int32_t* __restrict__ src_bins, int num_groups,
+                                        int n_slots, int src_rows, uint32_t pitch_bytes, uint32_t top_k_magic, int top_k_shift,
+                                        uint32_t* __restrict__ table) {
+  const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= row_table_entries(n_slots, num_groups)) return;
+  auto bound = [&](int e) -> int { const int v = src_bins[e]; return v < 0 ? 0 : (v > n_slots ? n_slots : v); };
+  // the expert whose part holds entry s: the last one that starts at or before it
+  int lo = 0, hi = num_groups - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) / 2;
+    if ((int64_t)bound(mid - 1) + (int64_t)kRowTableTile * mid <= s) lo = mid; else hi = mid - 1;
+  }
+  const int e = lo;
+  const int xs = e > 0 ? bound(e - 1) : 0;
+  int xe = bound(e);
+  xe = xe < xs ? xs : xe;
+  const int64_t local = s - ((int64_t)xs + (int64_t)kRowTableTile * e);
+  const int64_t l = local / kRowTableTile * kRowTableTile + row_of_entry_slot((int)(local % kRowTableTile));
+  uint32_t v = 0u;
+  if (l < xe - xs) {
+    const int slot = slots[xs + l];
+    const uint32_t row = top_k_magic ? __umulhi((uint32_t)slot, top_k_magic) >> top_k_shift : (uint32_t)slot;
+    if (slot >= 0 && row < (uint32_t)src_rows) v = (row * pitch_bytes) ^ 0x80000000u;
+  }
+  table[s] = v;
 }
 
 }  // namespace dma

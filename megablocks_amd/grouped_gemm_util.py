@@ -297,9 +297,10 @@ def gmm_glu(a, b1, b2, batch_sizes, act, fuse=None):
 
 
 # Whether the dMoE layer hands the experts the ungathered tokens (`gmm_gather`) instead of calling ops.gather /
-# ops.padded_gather first: 'auto' = where no gradient is recorded (the forward then never writes the gathered copy;
-# with gradients the weight gradients need that copy anyway, so fusing only moves the gather into the backward),
-# '1' = always (the copy then exists only during the backward), '0' = never.
+# ops.padded_gather first: 'auto' = where no gradient is recorded and, with gradients, for top_k >= 2 (the weight
+# gradients then read the tokens through a row table, `gmm_tn_gather`; no gathered copy is written or kept), '1' =
+# always, '0' = never.  Where a weight gradient's shape is outside what the indexed kernel takes, the copy is made in the
+# backward and exists only there.
 FUSED_GATHER = os.environ.get('MBX_FUSED_GATHER', 'auto')
 
 
@@ -317,6 +318,17 @@ class GatheredRows:
         if self.padded_bins is None:
             return kernels.gather(self.x, self.indices, self.bin_ids, None, self.bins, self.top_k)
         return kernels.padded_gather(self.x, self.indices, self.bin_ids, None, self.bins, self.padded_bins, self.top_k)
+
+    def weight_gradient(self, d, batch_sizes):
+        """gmm(d, self.materialize(), batch_sizes, trans_a=True): the weight gradient of a product whose operand these
+        rows were (mlp.py:485-491, glu.py:154-159), read from the ungathered tokens where the library has a kernel for
+        the shapes (`gmm_tn_gather`), else from the copy, which is then made once and kept for the next call."""
+        out = gmm_tn_gather(d, self, batch_sizes)
+        if out is None:
+            if getattr(self, '_copy', None) is None:
+                self._copy = self.materialize()
+            out = gmm(d, self._copy, batch_sizes, trans_a=True)
+        return out
 
     def scatter_grad(self, grad):
         """The gradient of x from the gradient of the gathered matrix (gather.py:28-35, padded_gather.py:36-52)."""
@@ -368,6 +380,50 @@ def gmm_gather(src: GatheredRows, b1, batch_sizes, b2=None, act=None):
         return None
     _lib.check(rc, 'gmm_gather')
     return (c,) if act is None else (c, h) if b2 is None else (c, c2, h)
+
+
+def gmm_tn_gather(a, src: GatheredRows, batch_sizes, c=None):
+    """out[e] = a[r_e].T @ X[r_e] with X the rows `src` describes, read from the ungathered tokens (one launch,
+    `mbx_gmm_tn_gather`; bit-identical to `gmm(a, src.materialize(), batch_sizes, trans_a=True)`).  The table of row
+    offsets the kernel reads is built by the first call for a `src` and kept on it (the weight gradients of w1 and v1
+    share it).  Returns None where the library has no kernel for the operands: the caller gathers first."""
+    x = src.x
+    if not (x.is_cuda and x.ndim == 2 and x.dtype in (torch.bfloat16, torch.float16) and a.ndim == 2 and a.dtype == x.dtype
+            and a.is_cuda and a.shape[0] == src.rows and src.indices.dtype == torch.int32 and src.bins.dtype == torch.int32):
+        return None
+    if src.padded_bins is not None and src.padded_bins.dtype != torch.int32:
+        return None
+    if src.indices.ndim != 1 or src.indices.shape[0] != x.shape[0] * src.top_k:
+        raise ValueError('gmm_tn_gather: one assignment per token and top_k choice')
+    _lib.require_cuda(src.indices, src.bins, src.padded_bins, c)
+    a, x = a.contiguous(), x.contiguous()
+    rows, k, n = a.shape[0], a.shape[1], x.shape[1]
+    bins = _device_bins(batch_sizes, a.device, rows)
+    groups = bins.shape[0]
+    if src.bins.numel() != groups:
+        return None
+    x_bins = None if src.padded_bins is None else src.bins.contiguous()
+    if c is None:
+        c = torch.empty((groups, k, n), dtype=a.dtype, device=a.device)
+    elif tuple(c.shape) != (groups, k, n) or c.dtype != a.dtype or not c.is_contiguous():
+        raise ValueError('gmm_tn_gather: c has the wrong shape, dtype or layout')
+    table = getattr(src, '_row_table', None)
+    ready = table is not None and table[1] == n
+    if not ready:
+        table = (torch.empty(max(lib.mbx_gmm_tn_gather_table_bytes(x.shape[0], src.top_k, groups) // 4, 4), dtype=torch.int32,
+                             device=x.device), n)
+    with _lib.device_of(a), _lib.record('gmm_tn', rows=rows, k=k, n=n, elem=a.element_size(), groups=groups) as rec:
+        rc = lib.mbx_gmm_tn_gather(_lib.ptr(a), _lib.ptr(x), x.shape[0], _lib.ptr(src.indices.contiguous()), src.top_k,
+                                   _lib.ptr(x_bins), _lib.ptr(c), _lib.dtype_of(a), _lib.ptr(bins), groups, rows, k, n,
+                                   _lib.ptr(table[0]), table[0].numel() * 4, 1 if ready else 0, _lib.stream())
+        if rc == _lib.EUNSUPPORTED:
+            rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        return None
+    _lib.check(rc, 'gmm_tn_gather')
+    if not torch.cuda.is_current_stream_capturing():
+        src._row_table = table
+    return c
 
 
 def gmm_dglu(a, b, x1, x2, batch_sizes, act, fuse=None):

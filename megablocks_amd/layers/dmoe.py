@@ -88,18 +88,22 @@ class ParallelDroplessMLP(moe.ParallelMLP):
         bins = promote_scalar(ops.inclusive_cumsum(tokens_per_expert, 0))
         return indices, bin_ids, bins, padded_bins, tokens_per_expert
 
-    def _fuse_gather(self, x):
-        """Whether the experts get the ungathered tokens (gg.FUSED_GATHER): the built-in experts on the GPU only."""
+    def _fuse_gather(self, x, top_k):
+        """Whether the experts get the ungathered tokens (gg.FUSED_GATHER): the built-in experts on the GPU only.  'auto':
+        always without gradients; with them for top_k >= 2, where the step is as fast or faster (the weight gradient
+        reads the tokens through a row table, a few percent slower than from a copy, and the gather kernel is gone) and
+        the copy of top_k times the input's size is not kept for the backward pass; for top_k = 1 the gather is cheap
+        next to what the indexed weight gradient loses."""
         if gg.FUSED_GATHER == '0' or not x.is_cuda or not hasattr(self.mlp, 'forward_tokens'):
             return False
-        if gg.FUSED_GATHER == 'auto':
+        if gg.FUSED_GATHER == 'auto' and top_k < 2:
             return not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.mlp.parameters())))
         return True
 
     def _sparse_experts(self, x, indices, bin_ids, bins, padded_bins, top_k):
         """dmoe.py:219-226: padded gather, topology, experts.  Where the experts take the ungathered tokens the gather
         is part of their first product."""
-        if self._fuse_gather(x):
+        if self._fuse_gather(x, top_k):
             padded_rows = int(padded_bins[-1].item()) if padded_bins.numel() else 0   # as ops.padded_gather reads it
             with torch.no_grad():
                 topo = self.topology(x.new_empty((padded_rows, 0)), padded_bins)
@@ -147,7 +151,7 @@ class ParallelDroplessMLP(moe.ParallelMLP):
         """dmoe.py:260-280."""
         x = x.view(-1, x.shape[-1])
         out = None
-        if self._fuse_gather(x):
+        if self._fuse_gather(x, top_k):
             src = gg.GatheredRows(x, indices, bin_ids, bins, None, top_k, indices.shape[0])
             out = self.mlp.forward_tokens(src, tokens_per_expert)
         if out is None:

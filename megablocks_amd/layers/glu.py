@@ -132,17 +132,19 @@ class GroupedGLUExperts(torch.autograd.Function):
 
 def _glu_experts_backward(needs, x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, ddsd_out, act):
     """(dx, dw1, dv1, dw2) of GroupedGLUExperts from what its forward saved; needs = which of (x, w1, v1, w2) want a
-    gradient."""
+    gradient.  x: the experts' input rows, or a `gg.GatheredRows` that describes them (the weight gradients then read
+    the rows from the ungathered tokens)."""
     ddsd_out = ddsd_out.contiguous()
     dx = dw1 = dv1 = dw2 = None
     if needs[3]:
         dw2 = gg.backend.gmm(activation_fn_out, ddsd_out, batch_sizes, trans_a=True)
     if needs[0] or needs[1] or needs[2]:
         dsdd_out, dv1_out = gg.gmm_dglu(ddsd_out, w2, sdd_out, v1_out, batch_sizes, act)
+        wgrad = x.weight_gradient if isinstance(x, gg.GatheredRows) else (lambda d, sizes: gg.backend.gmm(d, x, sizes, trans_a=True))
         if needs[1]:
-            dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
+            dw1 = wgrad(dsdd_out, batch_sizes)
         if needs[2]:
-            dv1 = gg.backend.gmm(dv1_out, x, batch_sizes, trans_a=True)
+            dv1 = wgrad(dv1_out, batch_sizes)
         if needs[0]:
             dx = gg.gmm_dual(dsdd_out, w1, dv1_out, v1, batch_sizes)
     return dx, dw1, dv1, dw2
@@ -175,8 +177,7 @@ class GatheredGLUExperts(torch.autograd.Function):
         (x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, indices, bin_ids, bins,
          padded_bins) = ctx.saved_tensors
         src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, ctx.top_k, ctx.rows)
-        rows_of_x = src.materialize() if ctx.needs_input_grad[1] or ctx.needs_input_grad[2] else None
-        dx, dw1, dv1, dw2 = _glu_experts_backward(ctx.needs_input_grad, rows_of_x, w1, v1, w2, batch_sizes, sdd_out,
+        dx, dw1, dv1, dw2 = _glu_experts_backward(ctx.needs_input_grad, src, w1, v1, w2, batch_sizes, sdd_out,
                                                   v1_out, activation_fn_out, ddsd_out, ctx.act)
         if dx is not None:
             dx = src.scatter_grad(dx)

@@ -166,7 +166,9 @@ class GroupedGeluMLP(torch.autograd.Function):
 
 
 def _gelu_mlp_backward(needs, x, w1, w2, batch_sizes, sdd_out, activation_fn_out, ddsd_out):
-    """(dx, dw1, dw2) of GroupedGeluMLP from what its forward saved; needs = which of (x, w1, w2) want a gradient."""
+    """(dx, dw1, dw2) of GroupedGeluMLP from what its forward saved; needs = which of (x, w1, w2) want a gradient.
+    x: the experts' input rows, or a `gg.GatheredRows` that describes them (the weight gradient then reads the rows from
+    the ungathered tokens)."""
     ddsd_out = ddsd_out.contiguous()
     dx = dw1 = dw2 = None
     if needs[2]:
@@ -174,7 +176,8 @@ def _gelu_mlp_backward(needs, x, w1, w2, batch_sizes, sdd_out, activation_fn_out
     if needs[0] or needs[1]:
         dsdd_out = gg.gmm_dact(ddsd_out, w2, sdd_out, batch_sizes)
         if needs[1]:
-            dw1 = gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
+            dw1 = x.weight_gradient(dsdd_out, batch_sizes) if isinstance(x, gg.GatheredRows) else \
+                gg.backend.gmm(dsdd_out, x, batch_sizes, trans_a=True)
         if needs[0]:
             dx = gg.backend.gmm(dsdd_out, w1, batch_sizes)
     return dx, dw1, dw2
@@ -183,9 +186,9 @@ def _gelu_mlp_backward(needs, x, w1, w2, batch_sizes, sdd_out, activation_fn_out
 class GatheredGeluMLP(torch.autograd.Function):
     """GroupedGeluMLP on the rows ops.gather / ops.padded_gather would copy out of the tokens `x` (dmoe.py:219 / :273
     followed by mlp.py:499-523), without that copy in the forward: the first product reads its rows from `x` through
-    the sorted assignments (`gg.gmm_gather`).  The weight gradient of w1 needs the gathered rows as an operand, so the
-    backward makes the copy then, and returns the gradient of the tokens (the sum over each token's rows, which is
-    the backward of the gather).  Same values as the two separate nodes."""
+    the sorted assignments (`gg.gmm_gather`), and so does the weight gradient of w1 in the backward
+    (`gg.gmm_tn_gather`), which returns the gradient of the tokens (the sum over each token's rows, which is the
+    backward of the gather).  Same values as the two separate nodes."""
 
     @staticmethod
     @torch.amp.custom_fwd(device_type='cuda')
@@ -207,8 +210,7 @@ class GatheredGeluMLP(torch.autograd.Function):
     def backward(ctx: Any, ddsd_out: torch.Tensor):
         w1, w2, batch_sizes, x, sdd_out, activation_fn_out, indices, bin_ids, bins, padded_bins = ctx.saved_tensors
         src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, ctx.top_k, ctx.rows)
-        rows_of_x = src.materialize() if ctx.needs_input_grad[1] else None
-        dx, dw1, dw2 = _gelu_mlp_backward(ctx.needs_input_grad, rows_of_x, w1, w2, batch_sizes, sdd_out,
+        dx, dw1, dw2 = _gelu_mlp_backward(ctx.needs_input_grad, src, w1, w2, batch_sizes, sdd_out,
                                           activation_fn_out, ddsd_out)
         if dx is not None:
             dx = src.scatter_grad(dx)

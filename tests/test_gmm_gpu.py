@@ -750,6 +750,69 @@ def test_gmm_on_rows_gathered_on_the_fly(gg, tokens, experts, top_k, k, n, block
     assert bool((guard == 7.0).all())
 
 
+GATHERED_TN = [  # tokens, experts, top_k, hidden of the tokens (n), columns of the other operand (k), blocking
+    (4096, 8, 2, 1024, 512, 0), (3000, 5, 1, 320, 264, 0), (700, 3, 4, 128, 1408, 0), (2048, 16, 4, 256, 384, 128),
+    (1000, 72, 2, 128, 264, 128), (5000, 64, 1, 1024, 1024, 0), (9, 4, 2, 64, 136, 128), (4000, 64, 6, 192, 1408, 0),
+    (1111, 9, 7, 64, 256, 128), (500, 40, 33, 64, 192, 0), (2500, 4, 2, 2048, 320, 0),
+]
+
+
+@pytest.mark.parametrize('tokens,experts,top_k,n,k,blocking', GATHERED_TN)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_gmm_weight_gradient_on_rows_gathered_on_the_fly(gg, tokens, experts, top_k, n, k, blocking, dtype):
+    """gmm_tn_gather: the weight gradient d^T @ x_gathered of the experts' first product (mlp.py:485-491, glu.py:154-159)
+    reading the rows of x through the sorted assignments must equal, bit for bit, ops.gather / ops.padded_gather
+    (dmoe.py:219 / :273) followed by gmm(trans_a=True), and the CPU oracle's gather and product to 1e-2."""
+    torch.manual_seed(tokens + k)
+    indices, bin_ids, bins, padded_bins, tpe = _routing(tokens, experts, top_k, seed=tokens + n, blocking=blocking)
+    x = torch.randn(tokens, n, device='cuda').to(dtype)
+    rows = tokens * top_k if padded_bins is None else int(padded_bins[-1])
+    sizes = tpe if padded_bins is None else torch.diff(padded_bins, prepend=padded_bins.new_zeros(1))
+    d = torch.randn(rows, k, device='cuda').to(dtype)
+    src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, top_k, rows)
+    guard = torch.full((experts + 2, k, n), 7.0, device='cuda', dtype=dtype)
+    got = gg.gmm_tn_gather(d, src, sizes)
+    assert got is not None and got.shape == (experts, k, n)
+    copy = src.materialize()
+    assert torch.equal(got, gg.backend.gmm(d, copy, sizes, trans_a=True))
+    again = gg.gmm_tn_gather(d, src, sizes)                       # with the row table the first call left on src
+    assert torch.equal(again, got) and getattr(src, '_row_table', None) is not None
+    assert torch.equal(src.weight_gradient(d, sizes), got)
+    cpu = lambda t: None if t is None else t.cpu()
+    if padded_bins is None:
+        o_x = oracle.gather(cpu(x), cpu(indices), cpu(bin_ids), None, cpu(bins), top_k)
+    else:
+        o_x = oracle.padded_gather(cpu(x), cpu(indices), cpu(bin_ids), None, cpu(bins), cpu(padded_bins), top_k)
+    want = oracle.gmm(cpu(d), o_x, cpu(sizes), trans_a=True)
+    assert rel_err(got.cpu(), want) < TOL
+    for e, cnt in enumerate(tpe.tolist()):
+        if cnt == 0:
+            assert int(torch.count_nonzero(got[e])) == 0          # an expert without tokens: exactly zero
+    assert bool((guard == 7.0).all())
+
+
+def test_gmm_weight_gradient_on_gathered_rows_edge_cases(gg):
+    """Assignments outside [0, tokens * top_k) read as rows of zeros; shapes the kernel does not take come back as None
+    and `weight_gradient` then gathers once and multiplies."""
+    tokens, experts, top_k, n, k = 600, 4, 2, 128, 256
+    indices, bin_ids, bins, _, tpe = _routing(tokens, experts, top_k, seed=5)
+    x = torch.randn(tokens, n, device='cuda').bfloat16()
+    d = torch.randn(tokens * top_k, k, device='cuda').bfloat16()
+    bad = indices.clone()
+    bad[::7] = -1
+    bad[3::11] = tokens * top_k + 5
+    got = gg.gmm_tn_gather(d, gg.GatheredRows(x, bad, bin_ids, bins, None, top_k, tokens * top_k), tpe)
+    rows_of_x = x[(indices.long() // top_k)].clone()
+    rows_of_x[::7] = 0
+    rows_of_x[3::11] = 0
+    assert torch.equal(got, gg.backend.gmm(d, rows_of_x, tpe, trans_a=True))
+    src = gg.GatheredRows(x, indices, bin_ids, bins, None, top_k, tokens * top_k)
+    narrow = d[:, :128].contiguous()                               # at most 128 columns: the half-height tile, no gathered form
+    assert gg.gmm_tn_gather(narrow, src, tpe) is None
+    assert torch.equal(src.weight_gradient(narrow, tpe), gg.backend.gmm(narrow, src.materialize(), tpe, trans_a=True))
+    assert gg.gmm_tn_gather(d.float(), gg.GatheredRows(x.float(), indices, bin_ids, bins, None, top_k, tokens * top_k), tpe) is None
+
+
 def test_gmm_on_gathered_rows_with_assignments_out_of_range(gg):
     """An assignment outside [0, tokens * top_k) reads as a row of zeros (nothing outside x is fetched), and what the
     library has no kernel for comes back as None (the caller gathers first)."""

@@ -941,8 +941,8 @@ def test_memory_optimized_requires_all_grads():
 @pytest.mark.parametrize('mlp_type,mlp_impl', [('glu', 'grouped'), ('mlp', 'grouped'), ('glu', 'sparse'), ('mlp', 'sparse')])
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, mlp_impl, dtype):
-    """The layer with the token gather of dmoe.py:219 / :273 done by the experts' first product (gg.FUSED_GATHER): without
-    gradients that is the default; with gradients it is opt-in and the backward gathers for the weight gradients.
+    """The layer with the token gather of dmoe.py:219 / :273 done by the operand loads of the experts' first product and,
+    in the backward, of its weight gradients (gg.FUSED_GATHER).
     Output and every gradient must be the unfused layer's bit for bit (the same kernels on the same values), and the
     gather kernel must be gone from the forward."""
     from megablocks_amd import _lib
@@ -983,11 +983,16 @@ def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, m
     got, _, launched = step('auto', False)
     assert torch.equal(got, want) and 'gather' not in launched
     assert rel_err(got, oracle_out) < 1e-2                                    # the fused forward against the CPU oracle
-    want, want_grads, launched = step('auto', True)                           # gradients recorded: not fused by default
+    want, want_grads, launched = step('0', True)
     assert launched.count('gather') == 1 and launched.index('gather') < launched.index(first)
-    got, got_grads, launched = step('1', True)
+    got, got_grads, launched = step('auto', True)          # top_k = 2: fused with gradients recorded too
     assert torch.equal(got, want)
-    assert launched.count('gather') == 1 and launched.index('gather') > launched.index(first)   # now in the backward
+    assert 'gather' not in launched                        # nor in the backward: the weight gradients read the tokens
+    probe = torch.zeros(1, device='cuda', requires_grad=True)
+    assert layer.experts._fuse_gather(probe, 2) and not layer.experts._fuse_gather(probe, 1)   # 'auto' with gradients
+    assert layer.experts._fuse_gather(probe.detach(), 1) == (not any(p.requires_grad for p in layer.experts.mlp.parameters()))
+    got1, got1_grads, launched = step('1', True)
+    assert torch.equal(got1, want) and 'gather' not in launched and all(torch.equal(a, b) for a, b in zip(got1_grads, want_grads))
     assert len(got_grads) == len(want_grads) >= 4
     for g, wg in zip(got_grads, want_grads):
         assert torch.equal(g, wg)
