@@ -946,7 +946,7 @@ int mbx_gmm_tn_gather(const void* a, const void* x, int64_t x_rows, const int32_
   if (x_rows < 0 || top_k <= 0 || k < 0 || n < 0 || num_groups < 0 || rows < 0) return MBX_EINVAL;
   if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
   if (num_groups == 0 || (int64_t)k * n == 0) return 0;
-  if (!c || !bins || !indices || (rows > 0 && !a) || (x_rows > 0 && !x)) return MBX_EINVAL;
+  if (!c || !bins || (x_rows > 0 && (!x || !indices)) || (rows > 0 && !a)) return MBX_EINVAL;
   if (rows > 0x7fffffff) return MBX_ERANGE;
   const int64_t n_slots = x_rows * top_k;
   // the kernel with the full tile, 16-byte pieces of rows, one segment of the reduction, row offsets of 31 bits

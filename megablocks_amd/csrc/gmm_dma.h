@@ -458,7 +458,8 @@ __device__ __forceinline__ void block_multiply16(const Args& g, typename T::Acc 
   } while (0)
 
   const int nk = g.nk;
-  constexpr int WAIT_PROLOGUE = (SB - 1) * (LA + LB) + (GATHER_B ? LB : 0);   // tile 0 has landed
+  constexpr int kEntryLoads = 2;   // fetch_row_entries()
+  constexpr int WAIT_PROLOGUE = (SB - 1) * (LA + LB) + (GATHER_B ? kEntryLoads : 0);   // tile 0 has landed (the loads behind it: tile 1's, the entries of tile SB)
   constexpr int WAIT_LOOP = (SB - 2) * (LA + LB) + LA;       // tile kt + 1 has landed: everything up to B tile kt + 1
   static_assert(SB * (LA + LB) < 64, "vmcnt is a 6-bit counter");
   MBX_TICK(g.tick_ordinal, 6);

@@ -811,6 +811,10 @@ def test_gmm_weight_gradient_on_gathered_rows_edge_cases(gg):
     assert gg.gmm_tn_gather(narrow, src, tpe) is None
     assert torch.equal(src.weight_gradient(narrow, tpe), gg.backend.gmm(narrow, src.materialize(), tpe, trans_a=True))
     assert gg.gmm_tn_gather(d.float(), gg.GatheredRows(x.float(), indices, bin_ids, bins, None, top_k, tokens * top_k), tpe) is None
+    # no tokens at all: every expert's gradient is zero
+    none = gg.GatheredRows(x[:0], indices[:0], bin_ids[:0], torch.zeros_like(bins), None, top_k, 0)
+    got = gg.gmm_tn_gather(d[:0], none, torch.zeros_like(tpe))
+    assert got.shape == (experts, k, n) and not got.any()
 
 
 def test_gmm_on_gathered_rows_with_assignments_out_of_range(gg):
