@@ -297,7 +297,7 @@ def gmm_glu(a, b1, b2, batch_sizes, act, fuse=None):
 
 
 # Whether the dMoE layer hands the experts the ungathered tokens (`gmm_gather`) instead of calling ops.gather /
-# ops.padded_gather first: 'auto' = where no gradient is recorded and, with gradients, for top_k >= 2 (the weight
+# ops.padded_gather first: 'auto' = where no gradient is recorded and, with gradients, from top_k = 4 on (the weight
 # gradients then read the tokens through a row table, `gmm_tn_gather`; no gathered copy is written or kept), '1' =
 # always, '0' = never.  Where a weight gradient's shape is outside what the indexed kernel takes, the copy is made in the
 # backward and exists only there.
