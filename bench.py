@@ -175,7 +175,8 @@ def summarize(w, agg, slots_scale):
                 (m['rows'] * slots_scale * (m['k'] + m['n']) + m['groups'] * m['k'] * m['n']) * m['elem']
             # [rows, n] tensors the epilogues read or write besides the product: its activation; the saved product; the
             # gated activation (half as wide as the two products side by side); x1, x2 and a second gradient
-            for suffix, more in (('_act', 1.0), ('_dact', 1.0), ('_glu', 0.5), ('_dglu', 3.0)):
+            # ... ; the combined output next to the product (one row per product row: one expert per token)
+            for suffix, more in (('_act', 1.0), ('_dact', 1.0), ('_glu', 0.5), ('_dglu', 3.0), ('_scatter', 1.0)):
                 if name.endswith(suffix):
                     nbytes += more * m['rows'] * slots_scale * m['n'] * m['elem']
             gemm[name] = dict(avg_ms=round(avg_ms, 4), launches=launches, flops_per_launch=flops,

@@ -282,6 +282,23 @@ int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int to
                    const void* b1, const void* b2, void* c, void* c2, void* h, int dtype, const int32_t* bins,
                    int num_groups, int64_t rows, int k, int n, int act, mbx_stream_t stream);
 
+/* The experts' second product and the weighted combine in one launch, for top_k = 1: megablocks/layers/mlp.py:523 /
+ * glu.py:205 (`gmm(x, w2, batch_sizes)`) followed by megablocks/layers/dmoe.py:280 (`ops.scatter(x, indices, bin_ids,
+ * expert_weights, bins, top_k)`, megablocks/backend/kernels.py:173-207).  With one expert per token an output row is one
+ * product row times the token's weight -- no sum over top_k, no two tiles that write the same row -- so the store phase
+ * of the product writes it:
+ *   y = a[r_e] @ b[e]        (MBX_NN; a: [rows, k], b: [E, k, n])
+ *   c[r] = y[r]                                  (c: [rows, n], or NULL: not wanted -- the backward pass reads it)
+ *   out[indices[r]] = round(weights[indices[r]] * round(y[r]))        (out: [tokens, n]; weights NULL: 1)
+ * for every row r of the product (rows == tokens * 1: the unpadded grouped layout).  indices: the sorted assignments
+ * (int32 [rows]); weights: [tokens] of type w_dtype (an mbx_dtype).  The roundings are those of mbx_gmm followed by
+ * mbx_scatter: the results are bit-identical.  A row whose assignment is outside [0, tokens) is not combined.  out rows
+ * that no assignment names are left as they are.  MBX_EUNSUPPORTED: fp32, k not a multiple of 64, unaligned, an
+ * expert's weights of 2 GiB or more -- multiply, then scatter. */
+int mbx_gmm_scatter(const void* a, const void* b, void* c, void* out, int dtype, const int32_t* bins, int num_groups,
+                    int64_t rows, int k, int n, const int32_t* indices, const void* weights, int w_dtype, int64_t tokens,
+                    mbx_stream_t stream);
+
 /* The weight gradient of the experts' first product(s) on token rows that were never gathered: the backward's
  * `gmm(dsdd_out, x, batch_sizes, trans_a=True)` of megablocks/layers/mlp.py:485-491 / glu.py:154-159, where x is what
  * megablocks/layers/dmoe.py:219 / :273 gathered (`ops.padded_gather` / `ops.gather`), with that gather done by the

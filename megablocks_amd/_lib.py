@@ -50,6 +50,7 @@ _SIGNATURES = {
     'mbx_gmm_act': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_dact': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     'mbx_gmm_glu': (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
+    'mbx_gmm_scatter': (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _vp, _vp, _i, _i64, _vp]),
     'mbx_gmm_tn_gather_table_bytes': (_sz, [_i64, _i, _i]),
     'mbx_gmm_tn_gather': (_i, [_vp, _vp, _i64, _vp, _i, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _vp, _sz, _i, _vp]),
     'mbx_gmm_dglu': (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i64, _i, _i, _i, _vp]),

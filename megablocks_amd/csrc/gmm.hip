@@ -565,6 +565,15 @@ static inline int persistent_grid(int64_t tiles_upper_bound) {
 // epi / extra (NT, one operand pair only): dma::kEpiAct with the second output, dma::kEpiDact with the second input.
 // Rows of `a` gathered on the fly (NT; no epilogue, kEpiAct or kEpiGlu*): see GatherRows.
 // Device memory a launch may use for the parts of tiles it cuts along the reduction (gmm_rows_kernel's split-K tail):
+// The weighted combine in the epilogue (kEpiCombine): the sorted assignments (top_k = 1: tokens) of the product's rows,
+// the weights by token (or null) and their type, the row count of the combined output.
+struct CombineRows {
+  const int32_t* indices = nullptr;
+  const void* weights = nullptr;
+  int w_dtype = 0;
+  int tokens = 0;
+};
+
 // kWorkspaceCounters int32 counters, zero before the launch and zero again after it, then room for fp32 tiles.
 constexpr size_t kWorkspaceCounters = 1024, kWorkspacePartBytes = (size_t)256 * 256 * 4, kWorkspaceParts = 320;
 struct Workspace {
@@ -584,7 +593,8 @@ struct GatherRows {
 template <int DT, typename T, typename TS>
 int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_groups, int64_t rows, int k, int n,
             int layout, hipStream_t s, const void* a2 = nullptr, const void* b2 = nullptr, int epi = dma::kEpiNone,
-            void* extra = nullptr, void* out2 = nullptr, GatherRows gather = GatherRows(), Workspace ws = Workspace()) {
+            void* extra = nullptr, void* out2 = nullptr, GatherRows gather = GatherRows(), Workspace ws = Workspace(),
+            CombineRows combine = CombineRows()) {
   const uint16_t* ap = (const uint16_t*)a;
   const uint16_t* bp = (const uint16_t*)b;
   const uint16_t* ap2 = (const uint16_t*)a2;
@@ -680,9 +690,19 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (rc) return rc;                                                                                \
     kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2,  \
                                        gather.slots, gather.src_bins, gather.top_k, gather.src_rows, gather_magic, gather_shift, half_limit,  \
-                                       ws_counters, ws_parts, ws_capacity);                           \
+                                       ws_counters, ws_parts, ws_capacity, combine.weights, combine.w_dtype, combine.tokens);  \
   } while (0)
 #define MBX_LAUNCH_ROWS(B_MC, DUAL, EPI) MBX_LAUNCH_ROWS_G(B_MC, DUAL, EPI, false)
+  // the combine epilogue takes the sorted assignments where the gathered launches take theirs
+#define MBX_LAUNCH_ROWS_C(B_MC, DUAL, EPI)                                                            \
+  do {                                                                                                \
+    auto kern = dma::gmm_rows_kernel<DT, B_MC, T, TS, DUAL, EPI, false>;                              \
+    int rc = allow_lds(kern, lds);                                                                    \
+    if (rc) return rc;                                                                                \
+    kern<<<grid, T::THREADS, lds, s>>>(ap, bp, cp, bins, num_groups, rows, k, n, tiles_n, ap2, bp2, (uint16_t*)extra, (uint16_t*)out2,  \
+                                       combine.indices, nullptr, 1, 0, 0u, 0, half_limit, nullptr, nullptr, 0,          \
+                                       combine.weights, combine.w_dtype, combine.tokens);             \
+  } while (0)
   if (gather.slots) {
     if (layout != MBX_NT || a2 || !gather.src_bins || gather.top_k <= 0) return MBX_EINVAL;
     switch (epi) {
@@ -706,6 +726,12 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (epi == dma::kEpiDgluSilu) MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluSilu); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDgluGelu);
     return launch_status();
   }
+  if (epi == dma::kEpiCombine) {
+    // extra is the combined output [tokens, n]; c (the product itself) may be absent
+    if (layout != MBX_NN || a2 || !extra || !combine.indices) return MBX_EINVAL;
+    MBX_LAUNCH_ROWS_C(true, false, dma::kEpiCombine);
+    return launch_status();
+  }
   if (epi != dma::kEpiNone) {
     if (layout != MBX_NT || dual || !extra) return MBX_EINVAL;
     if (epi == dma::kEpiAct) MBX_LAUNCH_ROWS(false, false, dma::kEpiAct); else MBX_LAUNCH_ROWS(false, false, dma::kEpiDact);
@@ -717,6 +743,7 @@ int gmm_dma(const void* a, const void* b, void* c, const int32_t* bins, int num_
     if (dual) MBX_LAUNCH_ROWS(true, true, dma::kEpiNone); else MBX_LAUNCH_ROWS(true, false, dma::kEpiNone);
   }
 #undef MBX_LAUNCH_ROWS
+#undef MBX_LAUNCH_ROWS_C
 #undef MBX_LAUNCH_ROWS_G
   return launch_status();
 }
@@ -933,6 +960,36 @@ int mbx_gmm_gather(const void* x, int64_t x_rows, const int32_t* indices, int to
   gather.src_rows = (int)x_rows;
   const int epi = b2 ? (act == MBX_ACT_SILU ? dma::kEpiGluSilu : dma::kEpiGluGelu) : h ? dma::kEpiAct : dma::kEpiNone;
   return gmm_nt_epilogue(x, b1, c, h, dtype, bins, num_groups, rows, k, n, act, epi, stream, nullptr, c2, b2, gather);
+}
+
+int mbx_gmm_scatter(const void* a, const void* b, void* c, void* out, int dtype, const int32_t* bins, int num_groups,
+                    int64_t rows, int k, int n, const int32_t* indices, const void* weights, int w_dtype, int64_t tokens,
+                    mbx_stream_t stream) {
+  if (num_groups < 0 || rows < 0 || k < 0 || n < 0 || tokens < 0) return MBX_EINVAL;
+  if (dtype != MBX_BF16 && dtype != MBX_F16 && dtype != MBX_F32) return MBX_EINVAL;
+  if (weights && w_dtype != MBX_BF16 && w_dtype != MBX_F16 && w_dtype != MBX_F32) return MBX_EINVAL;
+  if (num_groups == 0 || rows == 0 || n == 0) return 0;
+  if (!out || !bins || !indices || (k > 0 && (!a || !b))) return MBX_EINVAL;
+  if (rows > 0x7fffffff || tokens > 0x7fffffff) return MBX_ERANGE;
+  // the direct-to-LDS NN kernel (16-bit types, whole K tiles, 16-byte pieces of rows); the combined output is addressed
+  // with 64 bits
+  const bool ok = dtype != MBX_F32 && aligned16(a) && aligned16(b) && (!c || aligned16(c)) && aligned16(out) && k > 0 &&
+                  k % TileDma::BK == 0 && n % 8 == 0 && dma_sizes_ok(k, n);
+  if (!ok) return MBX_EUNSUPPORTED;
+  CombineRows combine;
+  combine.indices = indices;
+  combine.weights = weights;
+  combine.w_dtype = w_dtype;
+  combine.tokens = (int)tokens;
+  hipStream_t s = as_stream(stream);
+  const GatherRows none;
+  const Workspace no_ws;
+  if (half_height_only(rows, num_groups, n)) {
+    if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NN, s, nullptr, nullptr, dma::kEpiCombine, out, nullptr, none, no_ws, combine);
+    return gmm_dma<MBX_F16, TileDmaSmallM, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NN, s, nullptr, nullptr, dma::kEpiCombine, out, nullptr, none, no_ws, combine);
+  }
+  if (dtype == MBX_BF16) return gmm_dma<MBX_BF16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NN, s, nullptr, nullptr, dma::kEpiCombine, out, nullptr, none, no_ws, combine);
+  return gmm_dma<MBX_F16, TileDma, TileDmaSmallM>(a, b, c, bins, num_groups, rows, k, n, MBX_NN, s, nullptr, nullptr, dma::kEpiCombine, out, nullptr, none, no_ws, combine);
 }
 
 size_t mbx_gmm_tn_gather_table_bytes(int64_t x_rows, int top_k, int num_groups) {

@@ -640,7 +640,11 @@ __device__ __forceinline__ void gelu_tanh_bwd8(float (&g)[8], const float (&x)[8
 //                 and not g itself.
 //   kEpiGluSilu, kEpiGluGelu   the tile is [x1 | x2], the same BN / 2 output columns of two products side by side (see
 //                 block_multiply16's GLU): stores x1, x2 and round(round(act(x1)) * x2), three outputs.
-enum { kEpiNone = 0, kEpiAct = 1, kEpiDact = 2, kEpiDgluSilu = 3, kEpiDgluGelu = 4, kEpiGluSilu = 5, kEpiGluGelu = 6 };
+//   kEpiCombine   also (or only, when c is null) stores every row of the (rounded) tile, multiplied by a weight and
+//                 rounded again, to the row of a second output that the row's assignment names: the weighted combine
+//                 of megablocks/backend/kernels.py:173-207 for top_k = 1, where a token's output row is one product
+//                 row and needs no sum (see Combine).
+enum { kEpiNone = 0, kEpiAct = 1, kEpiDact = 2, kEpiDgluSilu = 3, kEpiDgluGelu = 4, kEpiGluSilu = 5, kEpiGluGelu = 6, kEpiCombine = 7 };
 constexpr bool epi_is_dglu(int epi) { return epi == kEpiDgluSilu || epi == kEpiDgluGelu; }
 constexpr bool epi_is_glu(int epi) { return epi == kEpiGluSilu || epi == kEpiGluGelu; }
 
@@ -771,6 +775,27 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 // checks pitch and alignment).
 // STAGED: the caller has already put the rounded tile into the staging area (stage_product_tile() for every product
 // tile, after a barrier of its own); acc is not read.
+// kEpiCombine: where the rows of a tile go.  `token` is per thread: the assignment (= token, top_k = 1) of tile row
+// threadIdx.x as the caller loaded it before the main loop (not looked at until the store phase, so that nothing waits
+// for the load), `row_exists` whether the expert has that row.  A row whose assignment is outside [0, tokens) is not
+// combined.  weights (or null: 1) are indexed by token, in the type w_dtype names.
+struct Combine {
+  uint16_t* out = nullptr;        // [tokens, ldc]
+  const void* weights = nullptr;
+  int w_dtype = 0, tokens = 0;
+  int token = -1;
+  bool row_exists = false;
+};
+__device__ __forceinline__ int combine_token(const Combine& cb) {
+  return cb.row_exists && (uint32_t)cb.token < (uint32_t)cb.tokens ? cb.token : -1;
+}
+__device__ __forceinline__ float combine_weight(const Combine& cb, int token) {
+  if (cb.weights == nullptr || token < 0) return 1.f;
+  if (cb.w_dtype == 2) return ((const float*)cb.weights)[token];
+  const uint16_t raw = ((const uint16_t*)cb.weights)[token];
+  return cb.w_dtype == 0 ? Elem<0>::to_f32(__builtin_bit_cast(typename Elem<0>::type, raw)) : Elem<1>::to_f32(__builtin_bit_cast(typename Elem<1>::type, raw));
+}
+
 template <int DT, typename T>
 __device__ __forceinline__ void stage_product_tile(char* lds_generic, int i, int j, const f32x4& v) {
   const lds_ptr lds = (lds_ptr)lds_generic;
@@ -788,11 +813,21 @@ template <int DT, typename T, int EPI = kEpiNone, bool STAGED = false>
 __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][T::TN], uint16_t* __restrict__ c, int64_t ldc,
                                             int m_base, int m_lim, int n_base, int n_lim, char* lds_generic,
                                             uint16_t* __restrict__ extra = nullptr, const uint16_t* __restrict__ pre2 = nullptr,
-                                            uint16_t* __restrict__ out2 = nullptr) {
+                                            uint16_t* __restrict__ out2 = nullptr, const Combine& combine = Combine()) {
   const lds_ptr lds = (lds_ptr)lds_generic;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = lane_id();
   const int wm = (wave / T::WN) * T::WTM, wn = (wave % T::WN) * T::WTN;
+  // kEpiCombine: (token, weight) of tile row threadIdx.x, handed to the lanes that store the row through the LDS
+  // behind the staging area; the weight's load (it depends on the token) is under way while the tile is staged
+  static_assert(EPI != kEpiCombine || T::EPILOGUE_BYTES + T::BM * 8 <= T::LDS_BYTES, "room for the rows' tokens and weights");
+  constexpr uint32_t kPairs = (uint32_t)T::EPILOGUE_BYTES;
+  int cb_token = -1;
+  float cb_weight = 1.f;
+  if constexpr (EPI == kEpiCombine) {
+    cb_token = combine_token(combine);
+    cb_weight = combine_weight(combine, cb_token);
+  }
   // accumulator (i, j), register r of lane l holds c[m][n] with
   //   m = m_base + wm + 16 i + (l % 16),  n = n_base + wn + 16 j + 4 (l / 16) + r
   // i.e. a run of four consecutive columns per lane and product tile.
@@ -816,6 +851,12 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
           w[1] = pack2<DT>(v[2], v[3]);
           *(__attribute__((address_space(3))) u32x2*)(lds + ml * ROW + nl * 2) = w;
         }
+      }
+    }
+    if constexpr (EPI == kEpiCombine) {
+      if (threadIdx.x < T::BM) {   // the tokens, then the weights
+        *(__attribute__((address_space(3))) int*)(lds + kPairs + threadIdx.x * 4u) = cb_token;
+        *(__attribute__((address_space(3))) float*)(lds + kPairs + (uint32_t)T::BM * 4u + threadIdx.x * 4u) = cb_weight;
       }
     }
     __syncthreads();
@@ -958,7 +999,41 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
           dglu_chunk<DT, EPI == kEpiDgluGelu>(gv, pre[u], preb[u], v[u], y[u]);
         }
       }
-      if (full_n) {
+      if constexpr (EPI == kEpiCombine) {
+        // the product's row (where the caller wants it: the backward pass does) and the token's row of the output
+        int row_token[BATCH];
+        float row_weight[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          const uint32_t at = kPairs + (uint32_t)((wave * ROWS_PER_INSTR + rl + (b + u) * ROW_STEP) * 4);
+          row_token[u] = *(const __attribute__((address_space(3))) int*)(lds + at);
+          row_weight[u] = *(const __attribute__((address_space(3))) float*)(lds + at + (uint32_t)T::BM * 4u);
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          if (m + u * ROW_STEP >= m_lim || n >= n_lim) continue;
+          const int token = row_token[u];
+          const float w = row_weight[u];
+          float f[8];
+          unpack8<DT>(v[u], f);
+#pragma unroll
+          for (int t = 0; t < 8; ++t) f[t] *= w;
+          const u32x4 scaled = pack8<DT>(f);
+          uint16_t* const dst = (uint16_t*)(cb + (off + (uint32_t)u * off_step));
+          uint16_t* const dst2 = token >= 0 ? combine.out + ((int64_t)token * ldc + n) : nullptr;
+          if (full_n || n + 8 <= n_lim) {
+            if (c != nullptr) __builtin_nontemporal_store(v[u], (u32x4*)dst);
+            if (dst2 != nullptr) __builtin_nontemporal_store(scaled, (u32x4*)dst2);
+          } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+              if (n + t < n_lim) {
+                if (c != nullptr) dst[t] = (uint16_t)(v[u][t >> 1] >> ((t & 1) * 16));
+                if (dst2 != nullptr) dst2[t] = (uint16_t)(scaled[t >> 1] >> ((t & 1) * 16));
+              }
+          }
+        }
+      } else if (full_n) {
 #pragma unroll
         for (int u = 0; u < BATCH; ++u)
           if (m + u * ROW_STEP < m_lim) {
@@ -996,11 +1071,12 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
 template <int DT, bool A_MC, bool B_MC, typename T, bool DUAL = false, int EPI = kEpiNone, bool GATHER = false>
 __device__ __forceinline__ void block_gemm(const Args& g, uint16_t* __restrict__ c, int64_t ldc, int m_base, int m_lim,
                                            int n_base, int n_lim, char* lds, uint16_t* __restrict__ extra = nullptr,
-                                           const uint16_t* __restrict__ pre2 = nullptr, uint16_t* __restrict__ out2 = nullptr) {
+                                           const uint16_t* __restrict__ pre2 = nullptr, uint16_t* __restrict__ out2 = nullptr,
+                                           const Combine& combine = Combine()) {
   typename T::Acc acc[T::TM][T::TN];
   block_multiply<DT, A_MC, B_MC, T, DUAL, epi_is_glu(EPI), GATHER>(g, acc, true, lds);
   MBX_TICK(g.tick_ordinal, 2);
-  block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra, pre2, out2);
+  block_store<DT, T, EPI>(acc, c, ldc, m_base, m_lim, n_base, n_lim, lds, extra, pre2, out2, combine);
   MBX_TICK(g.tick_ordinal, 4);
 }
 
@@ -1182,9 +1258,11 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
                 const uint16_t* __restrict__ a2, const uint16_t* __restrict__ b2, uint16_t* __restrict__ extra,
                 uint16_t* __restrict__ out2, const int32_t* __restrict__ slots, const int32_t* __restrict__ src_bins,
                 int top_k, int src_rows, uint32_t top_k_magic, int top_k_shift, int half_limit,
-                int32_t* __restrict__ ws_counters, float* ws_parts, int ws_capacity) {
+                int32_t* __restrict__ ws_counters, float* ws_parts, int ws_capacity,
+                const void* __restrict__ combine_weights, int combine_w_dtype, int combine_tokens) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   static_assert(T::THREADS == TS::THREADS && T::BN == TS::BN && T::BK == TS::BK, "tail tile");
+  static_assert(EPI != kEpiCombine || (!GATHER && !DUAL), "the combine: one operand pair, rows as they are");
   static_assert(!(DUAL && (epi_is_dglu(EPI) || epi_is_glu(EPI))), "a2 / b2 are the second operand pair, the epilogue's x2 or the second matrix");
   constexpr int kTileCols = epi_is_glu(EPI) ? T::BN / 2 : T::BN;   // output columns of a tile
   constexpr bool kSplit = T::BM != TS::BM;
@@ -1407,16 +1485,27 @@ gmm_rows_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, 
       // the second matrix of a [w1 | v1] tile: rows BN / 2 .. BN - 1 of the tile are its rows b_r0 .. b_r0 + BN / 2 - 1
       if (epi_is_glu(EPI)) g.rsrc_b2 = make_rsrc(b2 + ((int64_t)e * n - T::BN / 2) * k, (uint32_t)(((int64_t)n + T::BN / 2) * k * 2));
       g.b_r0 = tn * kTileCols;
-      uint16_t* const c_tile = c + (int64_t)row0 * n;
-      uint16_t* const e_tile = EPI != kEpiNone ? extra + (int64_t)row0 * n : nullptr;
+      uint16_t* const c_tile = EPI == kEpiCombine && c == nullptr ? nullptr : c + (int64_t)row0 * n;
+      uint16_t* const e_tile = EPI != kEpiNone && EPI != kEpiCombine ? extra + (int64_t)row0 * n : nullptr;
       const uint16_t* const p_tile = epi_is_dglu(EPI) ? a2 + (int64_t)row0 * n : nullptr;   // x2 of the gated activation
       uint16_t* const o_tile = epi_is_dglu(EPI) || epi_is_glu(EPI) ? out2 + (int64_t)row0 * n : nullptr;
       // the last row tile of an expert, when at most half full, is computed as a half-height tile as well
       use_ts = kSplit && (use_ts || end - row0 <= half_limit);
+      Combine combine;
+      if constexpr (EPI == kEpiCombine) {
+        // the assignment of tile row threadIdx.x (top_k = 1: the token itself), on its way during the main loop
+        combine.out = extra;
+        combine.weights = combine_weights;
+        combine.w_dtype = combine_w_dtype;
+        combine.tokens = combine_tokens;
+        const int row = row0 + (int)threadIdx.x;
+        combine.row_exists = row < end;
+        combine.token = slots[combine.row_exists ? row : end - 1];
+      }
       if (use_ts) {
-        block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
+        block_gemm<DT, false, B_MC, TS, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile, combine);
       } else {
-        block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile);
+        block_gemm<DT, false, B_MC, T, DUAL, EPI>(g, c_tile, n, 0, end - row0, g.b_r0, n, lds, e_tile, p_tile, o_tile, combine);
       }
       tile_done();
       MBX_TICK(r, 5);

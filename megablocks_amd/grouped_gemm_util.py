@@ -426,6 +426,71 @@ def gmm_tn_gather(a, src: GatheredRows, batch_sizes, c=None):
     return c
 
 
+# Whether, with one expert per token, the dMoE layer has the experts' second product write the weighted combine of
+# ops.scatter (dmoe.py:280) from its store phase (`gmm_scatter`): 'auto' / '1' = where the experts support it, '0' =
+# never.  top_k > 1 always combines in a pass of its own (a token's row is then a sum over products of several tiles).
+FUSED_COMBINE = os.environ.get('MBX_FUSED_COMBINE', 'auto')
+
+
+class CombinedRows:
+    """Where ops.scatter (dmoe.py:280, kernels.py:173-207) puts the rows of the experts' output when every token has one
+    expert (top_k = 1), as a description: row r goes to row indices[r] of the output, times weights[indices[r]]."""
+
+    def __init__(self, indices, bin_ids, bins, weights):
+        self.indices, self.bin_ids, self.bins, self.weights = indices, bin_ids, bins, weights
+        self.tokens = indices.shape[0]
+
+    def scatter(self, y):
+        """The combine as a pass of its own (what the fused launch replaces)."""
+        from megablocks_amd.backend import kernels
+        return kernels.scatter(y, self.indices, self.bin_ids, self.weights, self.bins, 1)
+
+    def backward(self, y, grad, need_rows=True, need_weights=True):
+        """(gradient of the rows y, gradient of the weights or None) of `scatter`, as ops/scatter.py:34-62."""
+        from megablocks_amd.backend import kernels
+        grad = grad.contiguous()
+        if need_rows and need_weights and self.weights is not None:
+            return kernels.scatter_backward(y, grad, self.indices, self.bin_ids, self.weights, self.bins, None, 1)
+        rows = kernels.gather(grad, self.indices, self.bin_ids, self.weights, self.bins, 1) if need_rows else None
+        wgrad = kernels.scatter_wgrad(y, grad, self.indices, self.bin_ids, self.bins, 1) \
+            if need_weights and self.weights is not None else None
+        return rows, wgrad
+
+
+def gmm_scatter(a, b, batch_sizes, combine: CombinedRows, keep_product=True):
+    """(y, out): y[r_e] = a[r_e] @ b[e], the experts' second product (mlp.py:523, glu.py:205), and out =
+    ops.scatter(y, indices, bin_ids, weights, bins, top_k = 1) (dmoe.py:280), the combine written by the product's
+    store phase (`mbx_gmm_scatter`; bit-identical to the two steps).  y is None when `keep_product` is False and the
+    launch did not have to write it (nothing will differentiate).  Shapes the kernel does not take: two steps."""
+    _lib.require_cuda(a, b, combine.indices, combine.weights)
+    if a.ndim != 2 or b.ndim != 3 or a.dtype != b.dtype or b.shape[1] != a.shape[1]:
+        raise ValueError('gmm_scatter: a must be [rows, k] and b [num_groups, k, n] of the same dtype')
+    a, b = a.contiguous(), b.contiguous()
+    rows, k, n = a.shape[0], a.shape[1], b.shape[2]
+    bins = _device_bins(batch_sizes, a.device, rows)
+    groups = bins.shape[0]
+    indices, weights = combine.indices, combine.weights
+    if b.shape[0] != groups or indices.shape[0] != rows:
+        raise ValueError('gmm_scatter: b, batch_sizes and the assignments do not match a')
+    rc = _lib.EUNSUPPORTED
+    if indices.dtype == torch.int32 and a.dtype in (torch.bfloat16, torch.float16) and rows > 0 and \
+            (weights is None or (weights.dtype in _lib.DTYPE and weights.numel() == combine.tokens)):
+        y = torch.empty((rows, n), dtype=a.dtype, device=a.device) if keep_product else None
+        out = torch.empty((combine.tokens, n), dtype=a.dtype, device=a.device)
+        w = None if weights is None else weights.contiguous()
+        with _lib.device_of(a), _lib.record('gmm_nn_scatter', rows=rows, k=k, n=n, elem=a.element_size(), groups=groups) as rec:
+            rc = lib.mbx_gmm_scatter(_lib.ptr(a), _lib.ptr(b), _lib.ptr(y), _lib.ptr(out), _lib.dtype_of(a), _lib.ptr(bins),
+                                     groups, rows, k, n, _lib.ptr(indices.contiguous()), _lib.ptr(w),
+                                     0 if w is None else _lib.dtype_of(w), combine.tokens, _lib.stream())
+            if rc == _lib.EUNSUPPORTED:
+                rec.cancel()
+    if rc == _lib.EUNSUPPORTED:
+        y = gmm(a, b, batch_sizes)
+        return y, combine.scatter(y)
+    _lib.check(rc, 'gmm_scatter')
+    return y, out
+
+
 def gmm_dglu(a, b, x1, x2, batch_sizes, act, fuse=None):
     """The gradients (d x1, d x2) of `activation(x1) * x2` where the incoming gradient is g = a[r_e] @ b[e].T: the
     `gmm(ddsd_out, w2, trans_b=True)` of the GLU experts' backward and the backward of their gated activation

@@ -103,6 +103,18 @@ class ParallelDroplessMLP(moe.ParallelMLP):
             return not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.mlp.parameters())))
         return True
 
+    def _mlp_takes_combine(self):
+        """Whether the experts' forward / forward_tokens accept the layer's combine (the built-in grouped experts do; an
+        expert class from the registry that overrides forward without it gets ops.scatter as before)."""
+        known = getattr(self, '_takes_combine', None)
+        if known is None:
+            import inspect
+            mlp = self.mlp
+            known = bool(getattr(mlp, 'takes_combine', False)) and all(
+                'combine' in inspect.signature(getattr(mlp, name)).parameters for name in ('forward', 'forward_tokens'))
+            self._takes_combine = known
+        return known
+
     def _sparse_experts(self, x, indices, bin_ids, bins, padded_bins, top_k):
         """dmoe.py:219-226: padded gather, topology, experts.  Where the experts take the ungathered tokens the gather
         is part of their first product."""
@@ -153,13 +165,22 @@ class ParallelDroplessMLP(moe.ParallelMLP):
                                     expert_capactiy, top_k):
         """dmoe.py:260-280."""
         x = x.view(-1, x.shape[-1])
+        # One expert per token: the combine is one output row per product row, and the built-in experts write it from
+        # the store phase of their second product (gg.FUSED_COMBINE).
+        combine = None
+        if top_k == 1 and gg.FUSED_COMBINE != '0' and x.is_cuda and self._mlp_takes_combine() and \
+                indices.dtype == torch.int32:
+            combine = gg.CombinedRows(indices, bin_ids, bins, expert_weights)
+        extra = () if combine is None else (combine,)
         out = None
         if self._fuse_gather(x, top_k):
             src = gg.GatheredRows(x, indices, bin_ids, bins, None, top_k, indices.shape[0])
-            out = self.mlp.forward_tokens(src, tokens_per_expert)
+            out = self.mlp.forward_tokens(src, tokens_per_expert, *extra)
         if out is None:
             x = ops.gather(x, indices, bin_ids, bins, top_k)
-            out = self.mlp(x, tokens_per_expert)
+            out = self.mlp(x, tokens_per_expert, *extra)
+        if combine is not None:
+            return out
         return ops.scatter(out, indices, bin_ids, expert_weights, bins, top_k)
 
     def forward_once(self, x, expert_weights, top_experts):

@@ -10,7 +10,7 @@ from megablocks_amd import grouped_gemm_util as gg
 from megablocks_amd._lib import lib
 from megablocks_amd.layers import common, mpu
 from megablocks_amd.layers.arguments import DEFAULT_ACTIVATION_FN, Arguments
-from megablocks_amd.layers.mlp import SparseMLP, Topology, create_dmoe_expert_weights
+from megablocks_amd.layers.mlp import SparseMLP, Topology, create_dmoe_expert_weights, second_product, second_product_grad
 
 _ACT_SILU, _ACT_GELU_TANH = 0, 1
 
@@ -115,19 +115,23 @@ class GroupedGLUExperts(torch.autograd.Function):
 
     @staticmethod
     @torch.amp.custom_fwd(device_type='cuda')
-    def forward(ctx, x, w1, v1, w2, batch_sizes, act):
+    def forward(ctx, x, w1, v1, w2, batch_sizes, act, c_indices=None, c_bin_ids=None, c_bins=None, c_weights=None):
+        # c_*: the layer's combine (`gg.CombinedRows`), when the node is to return the combined output
         x = x.contiguous()
         sdd_out, v1_out, activation_fn_out = gg.gmm_glu(x, w1, v1, batch_sizes, act)
         ctx.act = act
-        ctx.save_for_backward(x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out)
-        return gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+        combine = None if c_indices is None else gg.CombinedRows(c_indices, c_bin_ids, c_bins, c_weights)
+        out, kept = second_product(activation_fn_out, w2, batch_sizes, combine, ctx.needs_input_grad[9])
+        ctx.save_for_backward(x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, *kept)
+        return out
 
     @staticmethod
     @torch.amp.custom_bwd(device_type='cuda')
-    def backward(ctx, ddsd_out):
-        x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out = ctx.saved_tensors
+    def backward(ctx, grad):
+        x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, *kept = ctx.saved_tensors
+        ddsd_out, dweights = second_product_grad(kept, grad, ctx.needs_input_grad[9])
         return (*_glu_experts_backward(ctx.needs_input_grad, x, w1, v1, w2, batch_sizes, sdd_out, v1_out,
-                                       activation_fn_out, ddsd_out, ctx.act), None, None)
+                                       activation_fn_out, ddsd_out, ctx.act), None, None, None, None, None, dweights)
 
 
 def _glu_experts_backward(needs, x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, ddsd_out, act):
@@ -159,7 +163,9 @@ class GatheredGLUExperts(torch.autograd.Function):
 
     @staticmethod
     @torch.amp.custom_fwd(device_type='cuda')
-    def forward(ctx, x, w1, v1, w2, batch_sizes, act, indices, bin_ids, bins, padded_bins, top_k, rows):
+    def forward(ctx, x, w1, v1, w2, batch_sizes, act, indices, bin_ids, bins, padded_bins, top_k, rows, combined=False,
+                c_weights=None):
+        # combined: the node returns the layer's combine of its output (top_k = 1; the same assignments, c_weights)
         x = x.contiguous()
         src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, top_k, rows)
         out = gg.gmm_gather(src, w1, batch_sizes, b2=v1, act=act)
@@ -167,21 +173,24 @@ class GatheredGLUExperts(torch.autograd.Function):
             out = gg.gmm_glu(src.materialize(), w1, v1, batch_sizes, act)
         sdd_out, v1_out, activation_fn_out = out
         ctx.act, ctx.top_k, ctx.rows = act, top_k, rows
+        combine = gg.CombinedRows(indices, bin_ids, bins, c_weights) if combined else None
+        out, kept = second_product(activation_fn_out, w2, batch_sizes, combine, ctx.needs_input_grad[13])
         ctx.save_for_backward(x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, indices, bin_ids, bins,
-                              padded_bins)
-        return gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+                              padded_bins, *kept)
+        return out
 
     @staticmethod
     @torch.amp.custom_bwd(device_type='cuda')
-    def backward(ctx, ddsd_out):
+    def backward(ctx, grad):
         (x, w1, v1, w2, batch_sizes, sdd_out, v1_out, activation_fn_out, indices, bin_ids, bins,
-         padded_bins) = ctx.saved_tensors
+         padded_bins, *kept) = ctx.saved_tensors
+        ddsd_out, dweights = second_product_grad(kept, grad, ctx.needs_input_grad[13])
         src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, ctx.top_k, ctx.rows)
         dx, dw1, dv1, dw2 = _glu_experts_backward(ctx.needs_input_grad, src, w1, v1, w2, batch_sizes, sdd_out,
                                                   v1_out, activation_fn_out, ddsd_out, ctx.act)
         if dx is not None:
             dx = src.scatter_grad(dx)
-        return dx, dw1, dv1, dw2, None, None, None, None, None, None, None, None
+        return dx, dw1, dv1, dw2, None, None, None, None, None, None, None, None, None, dweights
 
 
 def _one_node(x, w1, v1, w2, act):
@@ -269,27 +278,29 @@ class SparseGLU(SparseMLP):
                                                      args.hidden_size, args.init_method))
         mpu.set_expert_model_parallel_attributes(self.v1, self._should_set_parallelism_attribute)
 
-    def _compute(self, x, batch_sizes, allow_memory_optimized=True):
+    def _compute(self, x, batch_sizes, allow_memory_optimized=True, combine=None):
         w1, v1, w2 = self._expert_views(self.w1, self.v1, self.w2)
         if self.args.memory_optimized_mlp:
             if not allow_memory_optimized:
                 raise NotImplementedError(
                     'Memory optimized implementation not yet supported with GLU with sparse kernels.')
-            return memory_optimized_grouped_glu(x, w1, v1, w2, batch_sizes, self.args.activation_fn)
+            return self._combined(memory_optimized_grouped_glu(x, w1, v1, w2, batch_sizes, self.args.activation_fn), combine)
         act = _activation_code(self.args.activation_fn)
         operands = gg.autocast_operands(x, w1, v1, w2)
         if _one_node(*operands, act):
-            return GroupedGLUExperts.apply(*operands, batch_sizes, act)
+            c = (None, None, None, None) if combine is None else (combine.indices, combine.bin_ids, combine.bins, combine.weights)
+            return GroupedGLUExperts.apply(*operands, batch_sizes, act, *c)
         x1, x2 = GLUProjection.apply(*operands[:3], batch_sizes)
         x1 = gated_activation(self.args.activation_fn, x1, x2)
-        return gg.ops.gmm(x1, w2, batch_sizes)
+        return self._combined(gg.ops.gmm(x1, w2, batch_sizes), combine)
 
     def forward(self, x, topo: Topology):
         return self._compute(x, topo.padded_tokens_per_expert, allow_memory_optimized=False)   # glu.py:47-50
 
-    def forward_tokens(self, src, batch_sizes):
+    def forward_tokens(self, src, batch_sizes, combine=None):
         """forward on the rows of the tokens that `src` (a `gg.GatheredRows`) describes, which are then never copied
-        out in the forward; None where that is not built (the caller gathers and calls forward)."""
+        out in the forward; None where that is not built (the caller gathers and calls forward).  combine: as for
+        forward (its assignments are src's)."""
         if self.args.memory_optimized_mlp and (torch.is_grad_enabled() or not isinstance(self, GroupedGLU)):
             # the memory-optimised schedule is a matter of what the backward keeps (without one, the same forward);
             # with the block-sparse experts it raises (glu.py:47-50), which is left to forward()
@@ -300,11 +311,12 @@ class SparseGLU(SparseMLP):
         if not _one_node(x, w1, v1, w2, act):
             return None
         return GatheredGLUExperts.apply(x, w1, v1, w2, batch_sizes, act, src.indices, src.bin_ids, src.bins,
-                                        src.padded_bins, src.top_k, src.rows)
+                                        src.padded_bins, src.top_k, src.rows, combine is not None,
+                                        None if combine is None else combine.weights)
 
 
 class GroupedGLU(SparseGLU):
     """glu.py:173-205."""
 
-    def forward(self, x, tokens_per_expert):
-        return self._compute(x, tokens_per_expert)
+    def forward(self, x, tokens_per_expert, combine=None):
+        return self._compute(x, tokens_per_expert, combine=combine)

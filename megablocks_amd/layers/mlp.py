@@ -139,6 +139,26 @@ class Topology:
         return self.column_indices.numel()
 
 
+def second_product(h, w2, batch_sizes, combine, weights_need_grad):
+    """The experts' second product h[r_e] @ w2[e] (mlp.py:523, glu.py:205) -- or, with `combine` (a `gg.CombinedRows`:
+    one expert per token), the layer's weighted combine of it (dmoe.py:280), written by the product's store phase
+    (`gg.gmm_scatter`).  Returns what the node returns and what its backward needs on top of that: nothing, or (the
+    product itself -- kept only if the combine's weights want a gradient --, indices, bin_ids, bins, weights)."""
+    if combine is None:
+        return gg.backend.gmm(h, w2, batch_sizes), ()
+    y, out = gg.gmm_scatter(h, w2, batch_sizes, combine, keep_product=weights_need_grad)
+    return out, (y, combine.indices, combine.bin_ids, combine.bins, combine.weights)
+
+
+def second_product_grad(kept, grad, weights_need_grad):
+    """(gradient of the second product's rows, gradient of the combine's weights or None) from the gradient of what
+    `second_product` returned; `kept`: the tensors it asked to keep."""
+    if not kept:
+        return grad, None
+    y, indices, bin_ids, bins, weights = kept
+    return gg.CombinedRows(indices, bin_ids, bins, weights).backward(y, grad, True, weights_need_grad)
+
+
 class GroupedGeluMLP(torch.autograd.Function):
     """GroupedMLP.forward with the default activation (mlp.py:499-523: gmm, tanh-GELU, gmm) and the backward autograd
     derives for it, with the two element-wise passes moved into the epilogues of the products next to them: the
@@ -148,21 +168,24 @@ class GroupedGeluMLP(torch.autograd.Function):
 
     @staticmethod
     @torch.amp.custom_fwd(device_type='cuda')
-    def forward(ctx, x, w1, w2, batch_sizes):
+    def forward(ctx, x, w1, w2, batch_sizes, c_indices=None, c_bin_ids=None, c_bins=None, c_weights=None):
+        # c_*: the layer's combine (`gg.CombinedRows`), when the node is to return the combined output
         if ctx._fwd_used_autocast:
             x, w1, w2 = x.to(ctx._dtype), w1.to(ctx._dtype), w2.to(ctx._dtype)
         x, w1, w2 = x.contiguous(), w1.contiguous(), w2.contiguous()
         sdd_out, activation_fn_out = gg.gmm_act(x, w1, batch_sizes)
-        dsd_out = gg.backend.gmm(activation_fn_out, w2, batch_sizes)
-        ctx.save_for_backward(w1, w2, batch_sizes, x, sdd_out, activation_fn_out)
-        return dsd_out
+        combine = None if c_indices is None else gg.CombinedRows(c_indices, c_bin_ids, c_bins, c_weights)
+        out, kept = second_product(activation_fn_out, w2, batch_sizes, combine, ctx.needs_input_grad[7])
+        ctx.save_for_backward(w1, w2, batch_sizes, x, sdd_out, activation_fn_out, *kept)
+        return out
 
     @staticmethod
     @torch.amp.custom_bwd(device_type='cuda')
-    def backward(ctx: Any, ddsd_out: torch.Tensor):
-        w1, w2, batch_sizes, x, sdd_out, activation_fn_out = ctx.saved_tensors
+    def backward(ctx: Any, grad: torch.Tensor):
+        w1, w2, batch_sizes, x, sdd_out, activation_fn_out, *kept = ctx.saved_tensors
+        ddsd_out, dweights = second_product_grad(kept, grad, ctx.needs_input_grad[7])
         return (*_gelu_mlp_backward(ctx.needs_input_grad, x, w1, w2, batch_sizes, sdd_out, activation_fn_out, ddsd_out),
-                None)
+                None, None, None, None, dweights)
 
 
 def _gelu_mlp_backward(needs, x, w1, w2, batch_sizes, sdd_out, activation_fn_out, ddsd_out):
@@ -192,7 +215,9 @@ class GatheredGeluMLP(torch.autograd.Function):
 
     @staticmethod
     @torch.amp.custom_fwd(device_type='cuda')
-    def forward(ctx, x, w1, w2, batch_sizes, indices, bin_ids, bins, padded_bins, top_k, rows):
+    def forward(ctx, x, w1, w2, batch_sizes, indices, bin_ids, bins, padded_bins, top_k, rows, combined=False,
+                c_weights=None):
+        # combined: the node returns the layer's combine of its output (top_k = 1; the same assignments, c_weights)
         if ctx._fwd_used_autocast:
             x, w1, w2 = x.to(ctx._dtype), w1.to(ctx._dtype), w2.to(ctx._dtype)
         x, w1, w2 = x.contiguous(), w1.contiguous(), w2.contiguous()
@@ -202,22 +227,29 @@ class GatheredGeluMLP(torch.autograd.Function):
             out = gg.gmm_act(src.materialize(), w1, batch_sizes)
         sdd_out, activation_fn_out = out
         ctx.top_k, ctx.rows = top_k, rows
-        ctx.save_for_backward(w1, w2, batch_sizes, x, sdd_out, activation_fn_out, indices, bin_ids, bins, padded_bins)
-        return gg.backend.gmm(activation_fn_out, w2, batch_sizes)
+        combine = gg.CombinedRows(indices, bin_ids, bins, c_weights) if combined else None
+        out, kept = second_product(activation_fn_out, w2, batch_sizes, combine, ctx.needs_input_grad[11])
+        ctx.save_for_backward(w1, w2, batch_sizes, x, sdd_out, activation_fn_out, indices, bin_ids, bins, padded_bins,
+                              *kept)
+        return out
 
     @staticmethod
     @torch.amp.custom_bwd(device_type='cuda')
-    def backward(ctx: Any, ddsd_out: torch.Tensor):
-        w1, w2, batch_sizes, x, sdd_out, activation_fn_out, indices, bin_ids, bins, padded_bins = ctx.saved_tensors
+    def backward(ctx: Any, grad: torch.Tensor):
+        w1, w2, batch_sizes, x, sdd_out, activation_fn_out, indices, bin_ids, bins, padded_bins, *kept = ctx.saved_tensors
+        ddsd_out, dweights = second_product_grad(kept, grad, ctx.needs_input_grad[11])
         src = gg.GatheredRows(x, indices, bin_ids, bins, padded_bins, ctx.top_k, ctx.rows)
         dx, dw1, dw2 = _gelu_mlp_backward(ctx.needs_input_grad, src, w1, w2, batch_sizes, sdd_out,
                                           activation_fn_out, ddsd_out)
         if dx is not None:
             dx = src.scatter_grad(dx)
-        return dx, dw1, dw2, None, None, None, None, None, None, None
+        return dx, dw1, dw2, None, None, None, None, None, None, None, None, dweights
 
 
-grouped_gelu_mlp = GroupedGeluMLP.apply
+def grouped_gelu_mlp(x, w1, w2, batch_sizes, combine=None):
+    """GroupedGeluMLP; with `combine` (a `gg.CombinedRows`) the node returns the layer's combine of its output."""
+    c = (None, None, None, None) if combine is None else (combine.indices, combine.bin_ids, combine.bins, combine.weights)
+    return GroupedGeluMLP.apply(x, w1, w2, batch_sizes, *c)
 
 
 class MemoryOptimizedGroupedMLP(torch.autograd.Function):
@@ -314,34 +346,47 @@ class SparseMLP(torch.nn.Module):
         ne = mpu.experts_per_rank(self.args)
         return [resolve_dtensor(self.scale_grad(w)).view(ne, -1, self.args.hidden_size) for w in weights]
 
-    def _compute(self, x, batch_sizes):
+    takes_combine = True   # forward / forward_tokens accept the layer's combine (`gg.CombinedRows`) and then return the combined output
+
+    @staticmethod
+    def _combined(y, combine):
+        """The combine as ops.scatter (dmoe.py:280), for the paths whose second product does not write it."""
+        if combine is None:
+            return y
+        from megablocks_amd import ops
+        return ops.scatter(y, combine.indices, combine.bin_ids, combine.weights, combine.bins, 1)
+
+    def _compute(self, x, batch_sizes, combine=None):
         w1, w2 = self._expert_views(self.w1, self.w2)
         if self.args.memory_optimized_mlp:
-            return memory_optimized_grouped_mlp(x, w1, w2, batch_sizes, self.args.activation_fn)
+            return self._combined(memory_optimized_grouped_mlp(x, w1, w2, batch_sizes, self.args.activation_fn), combine)
         if self.args.activation_fn is DEFAULT_ACTIVATION_FN and x.is_cuda:
-            return grouped_gelu_mlp(x, w1, w2, batch_sizes)
+            return grouped_gelu_mlp(x, w1, w2, batch_sizes, combine)
         x = gg.ops.gmm(x, w1, batch_sizes, trans_b=True)
         x = self.args.activation_fn(x)
-        return gg.ops.gmm(x, w2, batch_sizes)
+        return self._combined(gg.ops.gmm(x, w2, batch_sizes), combine)
 
     def forward(self, x, topo: Topology):
         return self._compute(x, topo.padded_tokens_per_expert)
 
-    def forward_tokens(self, src, batch_sizes):
+    def forward_tokens(self, src, batch_sizes, combine=None):
         """forward on the rows of the tokens that `src` (a `gg.GatheredRows`) describes, which are then never copied
-        out in the forward; None where that is not built (the caller gathers and calls forward)."""
+        out in the forward; None where that is not built (the caller gathers and calls forward).  combine: as for
+        forward (its assignments are src's)."""
         if self.args.activation_fn is not DEFAULT_ACTIVATION_FN or not src.x.is_cuda:
             return None
         if self.args.memory_optimized_mlp and torch.is_grad_enabled():
             return None   # the memory-optimised schedule is a matter of what the backward keeps: without one, the same forward
         w1, w2 = self._expert_views(self.w1, self.w2)
         return GatheredGeluMLP.apply(src.x, w1, w2, batch_sizes, src.indices, src.bin_ids, src.bins, src.padded_bins,
-                                     src.top_k, src.rows)
+                                     src.top_k, src.rows, combine is not None, None if combine is None else combine.weights)
 
 
 class GroupedMLP(SparseMLP):
     """mlp.py:499-523.  `tokens_per_expert` stays on the device: the grouped GEMM reads the row
     bins there, so the reference's `.cpu()` copy (mlp.py:502) is not needed."""
 
-    def forward(self, x, tokens_per_expert):
-        return self._compute(x, tokens_per_expert)
+    def forward(self, x, tokens_per_expert, combine=None):
+        """combine (a `gg.CombinedRows`, one expert per token): return the layer's weighted combine of the experts' output
+        (dmoe.py:280) instead of the output itself."""
+        return self._compute(x, tokens_per_expert, combine)

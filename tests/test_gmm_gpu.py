@@ -750,6 +750,58 @@ def test_gmm_on_rows_gathered_on_the_fly(gg, tokens, experts, top_k, k, n, block
     assert bool((guard == 7.0).all())
 
 
+COMBINED = [  # tokens (= rows: one expert per token), experts, k, n
+    (4096, 8, 1024, 512), (3000, 5, 320, 264), (37, 1, 64, 8), (5000, 64, 1024, 1024), (16384, 64, 512, 1024),
+    (700, 3, 128, 1408), (2600, 4, 2048, 256), (300, 40, 64, 136),
+]
+
+
+@pytest.mark.parametrize('tokens,experts,k,n', COMBINED)
+@pytest.mark.parametrize('dtype,w_dtype', [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+                                           (torch.bfloat16, torch.float32), (torch.bfloat16, None)])
+def test_gmm_with_the_combine_in_the_epilogue(gg, tokens, experts, k, n, dtype, w_dtype):
+    """gmm_scatter: with one expert per token the experts' second product (mlp.py:523, glu.py:205) writes the layer's
+    weighted combine (dmoe.py:280, kernels.py:173-207) from its store phase.  Product and combined output must equal,
+    bit for bit, gmm followed by the scatter kernel (the same roundings in the same places), and meet the CPU oracle's
+    product and scatter directly; rows of the output that no assignment names are left alone."""
+    from megablocks_amd.backend import kernels
+    torch.manual_seed(tokens + n)
+    indices, bin_ids, bins, _, tpe = _routing(tokens, experts, 1, seed=tokens + k)
+    h = torch.randn(tokens, k, device='cuda').to(dtype)
+    w2 = (torch.randn(experts, k, n, device='cuda') * (1.5 / k ** 0.5)).to(dtype)
+    weights = None if w_dtype is None else (torch.rand(tokens, device='cuda') + 0.25).to(w_dtype)
+    combine = gg.CombinedRows(indices, bin_ids, bins, weights)
+    want_y = gg.backend.gmm(h, w2, tpe)
+    want_out = kernels.scatter(want_y, indices, bin_ids, weights, bins, 1)
+    y, out = gg.gmm_scatter(h, w2, tpe, combine)
+    assert torch.equal(y, want_y) and torch.equal(out, want_out)
+    y2, out2 = gg.gmm_scatter(h, w2, tpe, combine, keep_product=False)
+    assert torch.equal(out2, want_out) and (y2 is None or torch.equal(y2, want_y))
+    cpu = lambda t: None if t is None else t.cpu()
+    o_y = oracle.gmm(cpu(h), cpu(w2), cpu(tpe))
+    o_out = oracle.scatter(o_y, cpu(indices), cpu(bin_ids), cpu(weights), cpu(bins), 1)
+    assert rel_err(y.cpu(), o_y) < TOL and rel_err(out.cpu(), o_out) < TOL
+    # assignments outside the tokens, and a token nobody names: those rows are not combined, that row is not written
+    bad = indices.clone()
+    bad[::5] = -3
+    bad[2::7] = tokens + 11
+    lib, _lib = gg.lib, gg._lib
+    canvas = torch.full((tokens, n), 3.0, device='cuda', dtype=dtype)
+    dbins = tpe.cumsum(0).int()
+    rc = lib.mbx_gmm_scatter(_lib.ptr(h), _lib.ptr(w2), None, _lib.ptr(canvas), _lib.dtype_of(h), _lib.ptr(dbins), experts,
+                             tokens, k, n, _lib.ptr(bad), _lib.ptr(weights), 0 if weights is None else _lib.dtype_of(weights),
+                             tokens, _lib.stream())
+    if k % 64 == 0 and n % 8 == 0:
+        assert rc == 0
+        keep = (bad >= 0) & (bad < tokens)
+        want = torch.full_like(canvas, 3.0)
+        want[bad[keep].long()] = want_out[indices[keep].long()] if weights is None else \
+            (want_y[keep].float() * weights[bad[keep].long()].float().unsqueeze(1)).to(dtype)
+        assert torch.equal(canvas, want)
+    else:
+        assert rc == _lib.EUNSUPPORTED
+
+
 GATHERED_TN = [  # tokens, experts, top_k, hidden of the tokens (n), columns of the other operand (k), blocking
     (4096, 8, 2, 1024, 512, 0), (3000, 5, 1, 320, 264, 0), (700, 3, 4, 128, 1408, 0), (2048, 16, 4, 256, 384, 128),
     (1000, 72, 2, 128, 264, 128), (5000, 64, 1, 1024, 1024, 0), (9, 4, 2, 64, 136, 128), (4000, 64, 6, 192, 1408, 0),

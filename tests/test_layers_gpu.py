@@ -1001,6 +1001,65 @@ def test_dmoe_with_the_gather_in_the_first_product(syn, monkeypatch, mlp_type, m
         assert rel_err(g, oracle_grads[name]) < 1e-2, name
 
 
+@pytest.mark.parametrize('mlp_type', ['mlp', 'glu'])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('fused_gather', ['0', '1'])
+def test_dmoe_with_the_combine_in_the_second_product(syn, monkeypatch, mlp_type, dtype, fused_gather):
+    """One expert per token: the weighted combine of dmoe.py:280 written by the store phase of the experts' second
+    product (gg.FUSED_COMBINE).  Output and every gradient -- the router weights' included, which the backward takes
+    from the product the launch also keeps -- must be the unfused layer's bit for bit, the combine kernel must be gone
+    from the forward, and the step must meet the oracle."""
+    from megablocks_amd import _lib
+    from megablocks_amd import grouped_gemm_util as gg
+    w = syn.Workload('t', 1500, 256, 768, 8, 1, mlp_type, 'grouped', dtype, 'logits')
+    inp = syn.make_inputs(w, seed=11)
+    for k in ('x', 'grad', 'w1', 'v1', 'w2', 'expert_weights'):
+        if inp[k] is not None:
+            inp[k] = inp[k].to(dtype).float()
+    oracle_out, _, oracle_grads, _ = _oracle_step(w, inp, True)
+    layer = syn.build_layer(w, inp)
+    routing = lambda ew: (inp['scores'].to(dtype).cuda(), ew, inp['top_experts'].cuda())
+    grad = inp['grad'].to(dtype).cuda()
+    monkeypatch.setattr(gg, 'FUSED_GATHER', fused_gather)
+
+    def step(mode, with_grad):
+        monkeypatch.setattr(gg, 'FUSED_COMBINE', mode)
+        layer.zero_grad(set_to_none=True)
+        x = inp['x'].to(dtype).cuda().requires_grad_(with_grad)
+        ew = inp['expert_weights'].to(dtype).cuda().requires_grad_(with_grad)
+        _lib.profile_hook = []
+        try:
+            if with_grad:
+                out = syn.layer_step(layer, w, x, grad, routing(ew))
+            else:
+                with torch.no_grad():
+                    out = layer.experts(x, *routing(ew))
+            torch.cuda.synchronize()
+            launched = [name for name, *_ in _lib.profile_hook]
+        finally:
+            _lib.profile_hook = None
+        mlp = layer.experts.mlp
+        grads = [x.grad, ew.grad] + [getattr(mlp, n).grad for n in ('w1', 'v1', 'w2') if hasattr(mlp, n)] if with_grad else []
+        return out.detach().clone(), [g.clone() for g in grads], launched
+
+    want, _, launched = step('0', False)
+    assert 'scatter_weighted' in launched and 'gmm_nn_scatter' not in launched
+    got, _, launched = step('auto', False)
+    assert torch.equal(got, want) and 'scatter_weighted' not in launched and 'gmm_nn_scatter' in launched
+    assert rel_err(got, oracle_out) < 1e-2
+    want, want_grads, launched = step('0', True)
+    assert 'scatter_weighted' in launched
+    got, got_grads, launched = step('auto', True)
+    assert torch.equal(got, want) and 'scatter_weighted' not in launched and launched.count('gmm_nn_scatter') == 1
+    assert len(got_grads) == len(want_grads) >= 4
+    for g, wg in zip(got_grads, want_grads):
+        assert torch.equal(g, wg)
+    assert rel_err(got, oracle_out) < 1e-2
+    names = ['x', 'expert_weights', 'w1'] + (['v1'] if mlp_type == 'glu' else []) + ['w2']
+    for name, g in zip(names, got_grads):
+        assert rel_err(g, oracle_grads[name]) < 1e-2, name
+
+
 @pytest.mark.parametrize('mlp_type,tokens,hs,ffn,ne,top_k', [('mlp', 2048, 1024, 1024, 64, 1), ('glu', 1024, 512, 1408, 8, 2)])
 def test_dmoe_forward_replays_from_a_captured_graph(monkeypatch, mlp_type, tokens, hs, ffn, ne, top_k):
     """The forward pass without gradients, where the first product of the experts reads the ungathered tokens: captured
