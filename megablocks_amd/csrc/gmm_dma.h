@@ -756,6 +756,25 @@ __device__ __forceinline__ u32x4 gelu_bwd_chunk(const u32x4& gv, const u32x4& xv
   return pack8<DT>(g);
 }
 
+// round(x * w) on the eight values of a chunk, formed the way the permutation kernels' scaled row copy forms it (a
+// conversion, a product and a conversion back per element): in fp16 the compiler makes one mixed-precision instruction
+// of the three, which rounds once, and the results of the two paths must agree to the bit.
+template <int DT>
+__device__ __forceinline__ u32x4 scale_chunk(const u32x4& v, float w) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint16_t lo = (uint16_t)(v[i] & 0xffffu), hi = (uint16_t)(v[i] >> 16);
+    if (DT == MBX_BF16) {
+      r[i] = (uint32_t)f32_to_bf16(bf16_to_f32(lo) * w) | ((uint32_t)f32_to_bf16(bf16_to_f32(hi) * w) << 16);
+    } else {
+      const _Float16 a = (_Float16)((float)__builtin_bit_cast(_Float16, lo) * w), b = (_Float16)((float)__builtin_bit_cast(_Float16, hi) * w);
+      r[i] = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+    }
+  }
+  return r;
+}
+
 // Buffer sizes stay below 2 GiB: bit 31 of a byte offset marks a load that must fetch nothing.
 __device__ __forceinline__ uint32_t clip_bytes(int64_t bytes) {
   return (uint32_t)(bytes < 0x7fffffff ? bytes : 0x7fffffff);
@@ -1014,11 +1033,7 @@ __device__ __forceinline__ void block_store(const typename T::Acc (&acc)[T::TM][
           if (m + u * ROW_STEP >= m_lim || n >= n_lim) continue;
           const int token = row_token[u];
           const float w = row_weight[u];
-          float f[8];
-          unpack8<DT>(v[u], f);
-#pragma unroll
-          for (int t = 0; t < 8; ++t) f[t] *= w;
-          const u32x4 scaled = pack8<DT>(f);
+          const u32x4 scaled = scale_chunk<DT>(v[u], w);
           uint16_t* const dst = (uint16_t*)(cb + (off + (uint32_t)u * off_step));
           uint16_t* const dst2 = token >= 0 ? combine.out + ((int64_t)token * ldc + n) : nullptr;
           if (full_n || n + 8 <= n_lim) {
